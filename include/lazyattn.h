@@ -1,0 +1,145 @@
+/* lazyattn.h -- C ABI of the MI355X (gfx950) deferred-RoPE prefix-prefill library.
+ *
+ * Plain pointers and sizes only; every pointer that is dereferenced on the GPU is a
+ * device pointer.  No entry point allocates, frees, synchronises or throws: each
+ * returns 0 or a negative LAZYATTN_E_* code and enqueues its work on the given HIP
+ * stream.  Paths in the comments are relative to the reference checkout.
+ */
+#ifndef LAZYATTN_H
+#define LAZYATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types */
+enum {
+    LAZYATTN_F32 = 0,
+    LAZYATTN_BF16 = 1,
+    LAZYATTN_F16 = 2,
+    LAZYATTN_FP8_E4M3 = 3, /* OCP e4m3fn, cache only */
+    LAZYATTN_FP8_E5M2 = 4  /* cache only */
+};
+
+/* how the rotation position of a cached key is derived */
+enum {
+    LAZYATTN_POS_NATURAL = 0,      /* p = n                      old_ops/prefix_prefill.py:183-184 */
+    LAZYATTN_POS_OFFSET = 1,       /* p = q_offset-1+o | n       old_ops/prefix_prefill.py:186-191 */
+    LAZYATTN_POS_BLOCK_UNIFORM = 2 /* p = q_offset-1 | 0 (page)  ops/prefix_prefill.py:180-186     */
+};
+
+/* kernel selection */
+enum {
+    LAZYATTN_KERNEL_AUTO = 0,
+    LAZYATTN_KERNEL_GENERIC = 1, /* fp32 arithmetic, any geometry */
+    LAZYATTN_KERNEL_MFMA = 2     /* bf16 MFMA, head_dim 128 / 64, 16-token pages */
+};
+
+/* which launches of a call to enqueue (profiling aid; default = both) */
+enum { LAZYATTN_PHASE_MAIN = 1, LAZYATTN_PHASE_COMBINE = 2, LAZYATTN_PHASE_ALL = 3 };
+
+enum {
+    LAZYATTN_OK = 0,
+    LAZYATTN_E_NULL = -1,        /* a required pointer is null */
+    LAZYATTN_E_SHAPE = -2,       /* inconsistent sizes (heads, head_dim, x, block_size ...) */
+    LAZYATTN_E_DTYPE = -3,       /* unsupported type combination */
+    LAZYATTN_E_UNSUPPORTED = -4, /* valid request the selected kernel cannot run */
+    LAZYATTN_E_WORKSPACE = -5,   /* workspace missing or too small */
+    LAZYATTN_E_LAUNCH = -6       /* hipLaunchKernel failed */
+};
+
+/* Arguments of one prefix-prefill call.  Replaces the Triton launch in
+ *   lazy_attn/lazy/attention/old_ops/prefix_prefill.py:491-554  (un-rotated cache)
+ *   lazy_attn/lazy/attention/ops/prefix_prefill.py:681-743      (block-uniform rotation)
+ * with the same operands.  Strides are in ELEMENTS.  q_offset / q_mask carry their
+ * own strides (the reference indexes them with the block table's strides,
+ * ops/prefix_prefill.py:180-182,267-268 -- pass the same values to get that).  */
+typedef struct lazyattn_prefill_params {
+    const void *q;       /* [T, Hq, D]   already rotated by the caller */
+    const void *k;       /* [T, Hkv, D]  new-token keys */
+    const void *v;       /* [T, Hkv, D] */
+    void *o;             /* [T, Hq, D]   written in place, rows t >= q_len untouched */
+    const void *k_cache; /* [NB, Hkv, D/x, BS, x] */
+    const void *v_cache; /* [NB, Hkv, D, BS] */
+    const int32_t *block_table; /* [B, NBmax] */
+    const int32_t *q_offset;    /* [B, NBmax] or NULL (= zeros) */
+    const int32_t *q_mask;      /* [B, NBmax] or NULL (= zeros) */
+    const uint8_t *is_lazy;     /* [B] bytes or NULL (= all set); only read for
+                                   LAZYATTN_POS_BLOCK_UNIFORM (ops/prefix_prefill.py:98) */
+    const void *b_start_loc;    /* [B+1] int32 or int64, see index_bits */
+    const void *b_seq_len;      /* [B] */
+    const void *cos_sin_cache;  /* [max_pos, rotary_dim]: row p = cos(p*inv) | sin(p*inv) */
+    const float *k_scale;       /* 1 element, read only for fp8 caches */
+    const float *v_scale;
+    void *workspace;            /* split-KV partials; lazyattn_prefill_workspace_bytes() */
+    int64_t workspace_bytes;
+
+    int64_t q_stride[3], k_stride[3], v_stride[3], o_stride[3];
+    int64_t kc_stride[5], vc_stride[4];
+    int64_t bt_stride[2], qo_stride[2], qm_stride[2];
+    int64_t table_stride;       /* row stride of cos_sin_cache */
+
+    int32_t batch, num_q_heads, num_kv_heads, head_dim;
+    int32_t block_size, x;      /* x = k_cache.shape[4] */
+    int32_t max_q_len;          /* max_input_len: sizes the grid (ops/prefix_prefill.py:681-682) */
+    int32_t rotary_dim;         /* must equal head_dim (the reference assumes it too) */
+    int32_t sliding_window;     /* <= 0 disables */
+    int32_t dtype;              /* q/k/v/o element type */
+    int32_t cache_dtype;        /* dtype, or FP8_* */
+    int32_t table_dtype;        /* dtype or F32 */
+    int32_t index_bits;         /* 32 or 64: b_start_loc / b_seq_len */
+    int32_t pos_mode;           /* LAZYATTN_POS_* */
+    int32_t rotate_new_k;       /* 1: rotate new-token K at ctx_len+m (old_ops:342-362) */
+    int32_t skip_decode;        /* 1: requests with q_len == 1 are not written (old_ops:109-110) */
+    int32_t fp32_rotary;        /* FORCE_FP32_ROTARY (old_ops:248-254); the MFMA kernel always
+                                   rotates in fp32 and rounds once */
+    int32_t kernel;             /* LAZYATTN_KERNEL_* */
+    int32_t num_splits;         /* context splits per work item; 0 = choose */
+    int32_t phases;             /* LAZYATTN_PHASE_*; 0 = all */
+    float sm_scale;
+    int32_t reserved;
+} lazyattn_prefill_params;
+
+/* Bytes of workspace lazyattn_prefix_prefill() may need for these sizes (0 when the
+ * chosen kernel writes `o` directly).  Pure host arithmetic.  No reference
+ * counterpart: Triton's launch has no split-KV. */
+size_t lazyattn_prefill_workspace_bytes(const lazyattn_prefill_params *p);
+
+/* Deferred-RoPE prefix-prefill attention.  Replaces `_fwd_kernel[grid](...)`
+ * (old_ops/prefix_prefill.py:493, ops/prefix_prefill.py:683). `stream` is a hipStream_t. */
+int lazyattn_prefix_prefill(const lazyattn_prefill_params *p, void *stream);
+
+/* q_len == 1 rows: every key (the new token included) comes from the paged cache.
+ * pos_mode NATURAL: each key is rotated at its natural position; replaces
+ *   `kernel_paged_attention_2d[(num_seqs, num_kv_heads)](...)`
+ *   (old_ops/chunked_prefill_paged_decode.py:396-442).
+ * pos_mode BLOCK_UNIFORM: each page of a lazy request is rotated forward by q_offset-1
+ *   (the reference de-rotates Q by the same angle instead, which gives the same scores);
+ *   other requests are not rotated; replaces `kernel_paged_attention_2d_llama`
+ *   (ops/models/llama_v1.py:91-288, launched at ops/chunked_prefill_paged_decode.py:171-221).
+ * Uses the same struct: k, v, rotate_new_k are ignored; requests with q_len != 1 are
+ * skipped (old_ops/chunked_prefill_paged_decode.py:72-79). */
+int lazyattn_paged_decode_rotary(const lazyattn_prefill_params *p, void *stream);
+
+/* cos/sin table builder on the device: out[p, i] = cos(p*inv[i]), out[p, R/2+i] = sin(..),
+ * inv = base^(-2i/R), optionally Llama-3 smoothed.  Restates
+ * lazy_attn/lazy/model_executor/rope/cos_sin.py:24-66 and the third-party table layout
+ * the kernels read (old_ops/prefix_prefill.py:192-193,231-232).  rope_type 0 = plain,
+ * 1 = Llama-3.  Angles are formed in float64 so rows at positions beyond 2^16 keep
+ * full float32 accuracy. */
+int lazyattn_build_cos_sin_cache(void *out, int32_t out_dtype, int64_t row_stride,
+                                 int32_t max_position, int32_t rotary_dim, double base,
+                                 int32_t rope_type, double scaling_factor,
+                                 double low_freq_factor, double high_freq_factor,
+                                 int32_t orig_max_position, void *stream);
+
+const char *lazyattn_error_string(int code);
+int lazyattn_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LAZYATTN_H */

@@ -1,0 +1,113 @@
+// C ABI: argument checks and kernel selection.  Nothing here allocates or synchronises.
+#include "common.hpp"
+
+namespace lazyattn {
+int launch_prefill_generic(const lazyattn_prefill_params &p, int decode, hipStream_t stream);
+int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream);
+bool mfma_supports(const lazyattn_prefill_params &p);
+size_t mfma_workspace_bytes(const lazyattn_prefill_params &p);
+int launch_cos_sin_table(void *out, int out_dtype, int64_t row_stride, int max_position,
+                         int rotary_dim, double base, int rope_type, double factor, double low,
+                         double high, int orig_max, hipStream_t stream);
+}  // namespace lazyattn
+
+using namespace lazyattn;
+
+static int elem_bytes(int dt) {
+    switch (dt) {
+        case LAZYATTN_F32: return 4;
+        case LAZYATTN_BF16:
+        case LAZYATTN_F16: return 2;
+        case LAZYATTN_FP8_E4M3:
+        case LAZYATTN_FP8_E5M2: return 1;
+        default: return 0;
+    }
+}
+
+static int check_common(const lazyattn_prefill_params *p, bool decode) {
+    if (!p) return LAZYATTN_E_NULL;
+    if (!p->q || !p->o || !p->k_cache || !p->v_cache || !p->block_table || !p->b_start_loc ||
+        !p->b_seq_len || !p->cos_sin_cache)
+        return LAZYATTN_E_NULL;
+    if (!decode && (!p->k || !p->v)) return LAZYATTN_E_NULL;
+    if (p->batch < 0 || p->num_q_heads <= 0 || p->num_kv_heads <= 0 || p->head_dim <= 0 ||
+        p->block_size <= 0 || p->x <= 0)
+        return LAZYATTN_E_SHAPE;
+    if (p->num_q_heads % p->num_kv_heads) return LAZYATTN_E_SHAPE;
+    if (p->head_dim % 2 || p->head_dim % p->x || p->head_dim > 256) return LAZYATTN_E_SHAPE;
+    if (p->rotary_dim != p->head_dim) return LAZYATTN_E_UNSUPPORTED;
+    if (p->index_bits != 32 && p->index_bits != 64) return LAZYATTN_E_DTYPE;
+    if (p->dtype != LAZYATTN_F32 && p->dtype != LAZYATTN_BF16 && p->dtype != LAZYATTN_F16)
+        return LAZYATTN_E_DTYPE;
+    const bool fp8 = p->cache_dtype == LAZYATTN_FP8_E4M3 || p->cache_dtype == LAZYATTN_FP8_E5M2;
+    if (!fp8 && p->cache_dtype != p->dtype) return LAZYATTN_E_DTYPE;
+    if (fp8 && (!p->k_scale || !p->v_scale)) return LAZYATTN_E_NULL;
+    if (p->table_dtype != p->dtype && p->table_dtype != LAZYATTN_F32) return LAZYATTN_E_DTYPE;
+    if (p->pos_mode < LAZYATTN_POS_NATURAL || p->pos_mode > LAZYATTN_POS_BLOCK_UNIFORM)
+        return LAZYATTN_E_UNSUPPORTED;
+    if (p->pos_mode != LAZYATTN_POS_NATURAL && !p->q_offset) return LAZYATTN_E_NULL;
+    (void)elem_bytes;
+    return LAZYATTN_OK;
+}
+
+extern "C" size_t lazyattn_prefill_workspace_bytes(const lazyattn_prefill_params *p) {
+    if (!p || check_common(p, false) != LAZYATTN_OK) return 0;
+    if (p->kernel == LAZYATTN_KERNEL_GENERIC) return 0;
+    if (!mfma_supports(*p)) return 0;
+    return mfma_workspace_bytes(*p);
+}
+
+extern "C" int lazyattn_prefix_prefill(const lazyattn_prefill_params *p, void *stream) {
+    int rc = check_common(p, false);
+    if (rc != LAZYATTN_OK) return rc;
+    if (p->batch == 0 || p->max_q_len <= 0) return LAZYATTN_OK;
+    hipStream_t s = (hipStream_t)stream;
+    int kernel = p->kernel;
+    if (kernel == LAZYATTN_KERNEL_AUTO)
+        kernel = mfma_supports(*p) ? LAZYATTN_KERNEL_MFMA : LAZYATTN_KERNEL_GENERIC;
+    if (kernel == LAZYATTN_KERNEL_MFMA) {
+        if (!mfma_supports(*p)) return LAZYATTN_E_UNSUPPORTED;
+        return launch_prefill_mfma(*p, s);
+    }
+    if (kernel == LAZYATTN_KERNEL_GENERIC) return launch_prefill_generic(*p, 0, s);
+    return LAZYATTN_E_UNSUPPORTED;
+}
+
+extern "C" int lazyattn_paged_decode_rotary(const lazyattn_prefill_params *p, void *stream) {
+    int rc = check_common(p, true);
+    if (rc != LAZYATTN_OK) return rc;
+    if (p->pos_mode == LAZYATTN_POS_OFFSET) return LAZYATTN_E_UNSUPPORTED;
+    if (p->batch == 0) return LAZYATTN_OK;
+    return launch_prefill_generic(*p, 1, (hipStream_t)stream);
+}
+
+extern "C" int lazyattn_build_cos_sin_cache(void *out, int32_t out_dtype, int64_t row_stride,
+                                            int32_t max_position, int32_t rotary_dim, double base,
+                                            int32_t rope_type, double scaling_factor,
+                                            double low_freq_factor, double high_freq_factor,
+                                            int32_t orig_max_position, void *stream) {
+    if (!out) return LAZYATTN_E_NULL;
+    if (max_position < 0 || rotary_dim <= 0 || rotary_dim % 2 || row_stride < rotary_dim)
+        return LAZYATTN_E_SHAPE;
+    if (rope_type != 0 && rope_type != 1) return LAZYATTN_E_UNSUPPORTED;
+    if (rope_type == 1 && (high_freq_factor == low_freq_factor || scaling_factor == 0.0))
+        return LAZYATTN_E_SHAPE;
+    return launch_cos_sin_table(out, out_dtype, row_stride, max_position, rotary_dim, base, rope_type,
+                                scaling_factor, low_freq_factor, high_freq_factor, orig_max_position,
+                                (hipStream_t)stream);
+}
+
+extern "C" const char *lazyattn_error_string(int code) {
+    switch (code) {
+        case LAZYATTN_OK: return "ok";
+        case LAZYATTN_E_NULL: return "a required pointer is null";
+        case LAZYATTN_E_SHAPE: return "inconsistent sizes";
+        case LAZYATTN_E_DTYPE: return "unsupported element type combination";
+        case LAZYATTN_E_UNSUPPORTED: return "request not supported by the selected kernel";
+        case LAZYATTN_E_WORKSPACE: return "workspace missing or too small";
+        case LAZYATTN_E_LAUNCH: return "kernel launch failed";
+        default: return "unknown error";
+    }
+}
+
+extern "C" int lazyattn_abi_version(void) { return 1; }

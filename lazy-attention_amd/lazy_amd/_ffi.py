@@ -1,0 +1,149 @@
+"""ctypes binding of liblazyattn.so (the C ABI declared in include/lazyattn.h).
+
+The library is loaded from ``lazy_amd/_lib``; if it is missing the import of any
+operator raises -- there is no fallback path.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import Optional
+
+import torch
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_lib", "liblazyattn.so")
+_lib = None
+
+F32, BF16, F16, FP8_E4M3, FP8_E5M2 = 0, 1, 2, 3, 4
+POS_NATURAL, POS_OFFSET, POS_BLOCK_UNIFORM = 0, 1, 2
+KERNEL_AUTO, KERNEL_GENERIC, KERNEL_MFMA = 0, 1, 2
+PHASE_MAIN, PHASE_COMBINE, PHASE_ALL = 1, 2, 3
+
+ERRORS = {-1: "NULL", -2: "SHAPE", -3: "DTYPE", -4: "UNSUPPORTED", -5: "WORKSPACE", -6: "LAUNCH"}
+EXPORTS = ("lazyattn_prefill_workspace_bytes", "lazyattn_prefix_prefill",
+           "lazyattn_paged_decode_rotary", "lazyattn_build_cos_sin_cache",
+           "lazyattn_error_string", "lazyattn_abi_version")
+
+_DTYPE = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
+
+
+class PrefillParams(C.Structure):
+    _fields_ = (
+        [(n, C.c_void_p) for n in ("q", "k", "v", "o", "k_cache", "v_cache", "block_table",
+                                   "q_offset", "q_mask", "is_lazy", "b_start_loc", "b_seq_len",
+                                   "cos_sin_cache", "k_scale", "v_scale", "workspace")]
+        + [("workspace_bytes", C.c_int64),
+           ("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3),
+           ("v_stride", C.c_int64 * 3), ("o_stride", C.c_int64 * 3),
+           ("kc_stride", C.c_int64 * 5), ("vc_stride", C.c_int64 * 4),
+           ("bt_stride", C.c_int64 * 2), ("qo_stride", C.c_int64 * 2), ("qm_stride", C.c_int64 * 2),
+           ("table_stride", C.c_int64)]
+        + [(n, C.c_int32) for n in ("batch", "num_q_heads", "num_kv_heads", "head_dim", "block_size",
+                                    "x", "max_q_len", "rotary_dim", "sliding_window", "dtype",
+                                    "cache_dtype", "table_dtype", "index_bits", "pos_mode",
+                                    "rotate_new_k", "skip_decode", "fp32_rotary", "kernel",
+                                    "num_splits", "phases")]
+        + [("sm_scale", C.c_float), ("reserved", C.c_int32)])
+
+
+def lib() -> C.CDLL:
+    """Load the HIP library.  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            raise RuntimeError(
+                f"{_LIB_PATH} is missing: build it with `python lazy-attention_amd/build.py` "
+                "(there is no non-HIP path)")
+        L = C.CDLL(_LIB_PATH)
+        L.lazyattn_prefill_workspace_bytes.restype = C.c_size_t
+        L.lazyattn_prefill_workspace_bytes.argtypes = [C.POINTER(PrefillParams)]
+        for name in ("lazyattn_prefix_prefill", "lazyattn_paged_decode_rotary"):
+            fn = getattr(L, name)
+            fn.restype = C.c_int
+            fn.argtypes = [C.POINTER(PrefillParams), C.c_void_p]
+        L.lazyattn_build_cos_sin_cache.restype = C.c_int
+        L.lazyattn_build_cos_sin_cache.argtypes = [
+            C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.c_int32, C.c_double, C.c_int32,
+            C.c_double, C.c_double, C.c_double, C.c_int32, C.c_void_p]
+        L.lazyattn_error_string.restype = C.c_char_p
+        L.lazyattn_error_string.argtypes = [C.c_int]
+        L.lazyattn_abi_version.restype = C.c_int
+        _lib = L
+    return _lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = lib().lazyattn_error_string(rc).decode()
+        if rc == -4:
+            raise NotImplementedError(f"{what}: {msg}")
+        raise RuntimeError(f"{what}: {msg} (code {rc})")
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    try:
+        return _DTYPE[dt]
+    except KeyError:
+        raise TypeError(f"unsupported tensor dtype {dt}") from None
+
+
+_workspaces: dict = {}
+
+
+def workspace(device: torch.device, nbytes: int) -> Optional[torch.Tensor]:
+    """Per-device scratch for split-KV partials, grown on demand and kept."""
+    if nbytes <= 0:
+        return None
+    key = (device.type, device.index)
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def fill_params(*, q, k, v, o, k_cache, v_cache, block_table, b_start_loc, b_seq_len,
+                cos_sin_cache, k_scale, v_scale, q_offset, q_mask, is_lazy, cache_code: int,
+                max_q_len: int, rotary_dim: int, sliding_window: int, sm_scale: float,
+                pos_mode: int, rotate_new_k: bool, skip_decode: bool, fp32_rotary: bool = False,
+                kernel: int = KERNEL_AUTO, num_splits: int = 0, phases: int = PHASE_ALL) -> PrefillParams:
+    p = PrefillParams()
+    p.q, p.k, p.v, p.o = _ptr(q), _ptr(k), _ptr(v), _ptr(o)
+    p.k_cache, p.v_cache = _ptr(k_cache), _ptr(v_cache)
+    p.block_table, p.q_offset, p.q_mask, p.is_lazy = _ptr(block_table), _ptr(q_offset), _ptr(q_mask), _ptr(is_lazy)
+    p.b_start_loc, p.b_seq_len = _ptr(b_start_loc), _ptr(b_seq_len)
+    p.cos_sin_cache, p.k_scale, p.v_scale = _ptr(cos_sin_cache), _ptr(k_scale), _ptr(v_scale)
+    p.q_stride[:] = q.stride()
+    p.k_stride[:] = k.stride() if k is not None else (0, 0, 0)
+    p.v_stride[:] = v.stride() if v is not None else (0, 0, 0)
+    p.o_stride[:] = o.stride()
+    p.kc_stride[:] = k_cache.stride()
+    p.vc_stride[:] = v_cache.stride()
+    p.bt_stride[:] = block_table.stride()
+    p.qo_stride[:] = q_offset.stride() if q_offset is not None else (0, 0)
+    p.qm_stride[:] = q_mask.stride() if q_mask is not None else (0, 0)
+    p.table_stride = cos_sin_cache.stride(0)
+    p.batch = b_seq_len.shape[0]
+    p.num_q_heads, p.head_dim = q.shape[1], q.shape[2]
+    p.num_kv_heads = k_cache.shape[1]
+    p.block_size, p.x = v_cache.shape[3], k_cache.shape[4]
+    p.max_q_len = int(max_q_len)
+    p.rotary_dim = int(rotary_dim)
+    p.sliding_window = int(sliding_window)
+    p.dtype = dtype_code(q.dtype)
+    p.cache_dtype = cache_code
+    p.table_dtype = dtype_code(cos_sin_cache.dtype)
+    p.index_bits = 64 if b_start_loc.dtype == torch.int64 else 32
+    p.pos_mode = pos_mode
+    p.rotate_new_k = int(rotate_new_k)
+    p.skip_decode = int(skip_decode)
+    p.fp32_rotary = int(fp32_rotary)
+    p.kernel = kernel
+    p.num_splits = num_splits
+    p.phases = phases
+    p.sm_scale = float(sm_scale)
+    return p

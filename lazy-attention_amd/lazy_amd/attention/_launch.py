@@ -1,0 +1,106 @@
+"""Host side shared by the two operator variants: the reference's argument checks
+(``lazy_attn/lazy/attention/ops/prefix_prefill.py:627-676``,
+``old_ops/prefix_prefill.py:437-486``) and the hand-off to the C ABI."""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .. import _ffi
+
+
+def _cache_code(kv_cache_dtype: str, k_cache: torch.Tensor, v_cache: torch.Tensor, q_dtype) -> int:
+    # ops/prefix_prefill.py:637-654
+    if "fp8" in kv_cache_dtype:
+        assert k_cache.dtype == torch.uint8
+        assert v_cache.dtype == torch.uint8
+        if kv_cache_dtype in ("fp8", "fp8_e4m3"):
+            return _ffi.FP8_E4M3
+        if kv_cache_dtype == "fp8_e5m2":
+            return _ffi.FP8_E5M2
+        raise ValueError("Unsupported FP8 dtype:", kv_cache_dtype)
+    if k_cache.dtype == torch.uint8 or v_cache.dtype == torch.uint8:
+        raise ValueError("kv_cache_dtype='auto' unsupported for FP8 KV Cache prefill kernel")
+    if k_cache.dtype != q_dtype or v_cache.dtype != q_dtype:
+        raise TypeError(f"cache dtype {k_cache.dtype} does not match query dtype {q_dtype}")
+    return _ffi.dtype_code(q_dtype)
+
+
+def _i32(t: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    if t is None or t.dtype == torch.int32:
+        return t
+    return t.to(torch.int32)
+
+
+def _require_gpu(*tensors) -> torch.device:
+    dev = tensors[0].device
+    if dev.type != "cuda":
+        raise RuntimeError("lazy_amd operators run on the GPU only (got a tensor on "
+                           f"'{dev}'); there is no CPU path")
+    for t in tensors:
+        if t is not None and t.device != dev:
+            raise RuntimeError(f"tensors on different devices: {dev} vs {t.device}")
+    return dev
+
+
+def launch_prefill(*, q, k, v, o, kv_cache_dtype, k_cache, v_cache, b_loc, b_start_loc, b_seq_len,
+                   max_input_len, k_scale, v_scale, alibi_slopes, sliding_window, sm_scale,
+                   skip_decode, cos_sin_cache, rotary_dim, is_neox_style, is_lazy, q_offset, q_mask,
+                   pos_mode: int, rotate_new_k: bool, fp32_rotary: bool = False,
+                   kernel: int = _ffi.KERNEL_AUTO, num_splits: int = 0,
+                   phases: int = _ffi.PHASE_ALL, decode: bool = False) -> None:
+    lib = _ffi.lib()
+    cache_code = _cache_code(kv_cache_dtype, k_cache, v_cache, q.dtype)
+    if not decode:
+        Lq, Lk, Lv = q.shape[-1], k.shape[-1], v.shape[-1]
+        assert Lq == Lk and Lk == Lv                                   # ops/prefix_prefill.py:657-658
+    else:
+        Lq = q.shape[-1]
+    if sm_scale is None:
+        sm_scale = 1.0 / (Lq ** 0.5)
+    batch = b_seq_len.shape[0]
+    assert batch + 1 == len(b_start_loc)                               # ops/prefix_prefill.py:667
+    if sliding_window is None or sliding_window <= 0:
+        sliding_window = 0
+    if alibi_slopes is not None:
+        raise NotImplementedError("Alibi slopes are not implemented for prefix prefill")
+    if not is_neox_style:
+        raise NotImplementedError("only NeoX-style rotary embedding is supported")
+    dev = _require_gpu(q, k, v, o, k_cache, v_cache, b_loc, b_start_loc, b_seq_len,
+                       cos_sin_cache, q_offset, q_mask, is_lazy)
+    if rotary_dim is None:
+        rotary_dim = cos_sin_cache.shape[-1] if cos_sin_cache is not None else Lq
+    if cos_sin_cache is None:
+        raise ValueError("cos_sin_cache is required")
+    if b_start_loc.dtype != b_seq_len.dtype:
+        b_seq_len = b_seq_len.to(b_start_loc.dtype)
+    if b_start_loc.dtype not in (torch.int32, torch.int64):
+        raise TypeError("b_start_loc / b_seq_len must be int32 or int64")
+    if is_lazy is not None and is_lazy.dtype != torch.bool and is_lazy.dtype != torch.uint8:
+        is_lazy = is_lazy != 0
+    if cache_code in (_ffi.FP8_E4M3, _ffi.FP8_E5M2):
+        k_scale = k_scale.to(device=dev, dtype=torch.float32) if (
+            k_scale.device != dev or k_scale.dtype != torch.float32) else k_scale
+        v_scale = v_scale.to(device=dev, dtype=torch.float32) if (
+            v_scale.device != dev or v_scale.dtype != torch.float32) else v_scale
+    else:
+        k_scale = v_scale = None
+    p = _ffi.fill_params(
+        q=q, k=k, v=v, o=o, k_cache=k_cache, v_cache=v_cache, block_table=_i32(b_loc),
+        b_start_loc=b_start_loc, b_seq_len=b_seq_len, cos_sin_cache=cos_sin_cache,
+        k_scale=k_scale, v_scale=v_scale, q_offset=_i32(q_offset), q_mask=_i32(q_mask),
+        is_lazy=is_lazy, cache_code=cache_code, max_q_len=max_input_len, rotary_dim=rotary_dim,
+        sliding_window=sliding_window, sm_scale=sm_scale, pos_mode=pos_mode,
+        rotate_new_k=rotate_new_k, skip_decode=skip_decode, fp32_rotary=fp32_rotary,
+        kernel=kernel, num_splits=num_splits, phases=phases)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    if decode:
+        _ffi.check(lib.lazyattn_paged_decode_rotary(p, stream), "lazyattn_paged_decode_rotary")
+        return
+    nbytes = lib.lazyattn_prefill_workspace_bytes(p)
+    ws = _ffi.workspace(dev, nbytes)
+    if ws is not None:
+        p.workspace = ws.data_ptr()
+        p.workspace_bytes = ws.numel()
+    _ffi.check(lib.lazyattn_prefix_prefill(p, stream), "lazyattn_prefix_prefill")

@@ -1,0 +1,43 @@
+"""Entry point the attention backend calls, un-rotated-cache variant.
+
+Drop-in for ``lazy_attn/lazy/attention/old_ops/chunked_prefill_paged_decode.py:283-454``:
+requests with more than one new token go through ``context_attention_fwd`` with
+``skip_decode=True`` (``:324-351``); requests with exactly one are handled by the
+fused-rotary q_len==1 kernel (``:396-442``).  The reference raises
+``NotImplementedError`` when vLLM's ROCm custom paged-attention op would be selected
+(``:380-386``); that op does not exist here, so nothing is refused.
+"""
+from __future__ import annotations
+
+from .. import _launch
+from ... import _ffi
+from .prefix_prefill import context_attention_fwd
+
+
+def chunked_prefill_paged_decode(query, key, value, output, kv_cache_dtype, key_cache, value_cache,
+                                 block_table, query_start_loc, seq_lens, max_seq_len, max_query_len,
+                                 k_scale, v_scale, alibi_slopes=None, sliding_window=None,
+                                 sm_scale=None, rotary_dim=None, cos_sin_cache=None,
+                                 is_neox_style=True, q_offset=None, q_mask=None,
+                                 is_mepic: bool = True, force_fp32_rotary: bool = False):
+    if sm_scale is None:
+        sm_scale = 1.0 / (query.shape[1] ** 0.5)        # sic: old_ops/chunked...:311-312
+    if sliding_window is None or sliding_window <= 0:
+        sliding_window = 0
+    if max_query_len > 1:
+        context_attention_fwd(
+            q=query, k=key, v=value, o=output, kv_cache_dtype=kv_cache_dtype, k_cache=key_cache,
+            v_cache=value_cache, b_loc=block_table, b_start_loc=query_start_loc, b_seq_len=seq_lens,
+            max_seq_len=max_seq_len, max_input_len=max_query_len, k_scale=k_scale, v_scale=v_scale,
+            alibi_slopes=alibi_slopes, sliding_window=sliding_window, sm_scale=sm_scale,
+            skip_decode=True, rotary_dim=rotary_dim, cos_sin_cache=cos_sin_cache,
+            is_neox_style=is_neox_style, q_mask=q_mask, q_offset=q_offset, is_mepic=is_mepic,
+            force_fp32_rotary=force_fp32_rotary)
+    _launch.launch_prefill(
+        q=query, k=key, v=value, o=output, kv_cache_dtype=kv_cache_dtype, k_cache=key_cache,
+        v_cache=value_cache, b_loc=block_table, b_start_loc=query_start_loc, b_seq_len=seq_lens,
+        max_input_len=1, k_scale=k_scale, v_scale=v_scale, alibi_slopes=alibi_slopes,
+        sliding_window=sliding_window, sm_scale=sm_scale, skip_decode=False,
+        cos_sin_cache=cos_sin_cache, rotary_dim=rotary_dim, is_neox_style=is_neox_style,
+        is_lazy=None, q_offset=None, q_mask=q_mask, pos_mode=_ffi.POS_NATURAL, rotate_new_k=True,
+        fp32_rotary=force_fp32_rotary, decode=True)

@@ -1,0 +1,43 @@
+"""Prefix-prefill attention with a block-uniform rotation of cached keys.
+
+Drop-in for ``lazy_attn/lazy/attention/ops/prefix_prefill.py:599-744``
+(``context_attention_fwd``).  Requests with ``is_lazy[b]`` set: every page of cached K
+(stored rotated at its document-local position) is rotated forward by ``q_offset-1``
+(``:180-190``), pad slots are masked through ``q_mask`` (``:267-271``), new-token K is
+used as given (``:341-354``).  Other requests take the un-rotated branch (``:398-592``).
+``is_lazy=None`` means no request is lazy (plain paged prefix-prefill).
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import _launch
+from ... import _ffi
+
+
+@torch.inference_mode()
+def context_attention_fwd(q, k, v, o, kv_cache_dtype: str, k_cache, v_cache, b_loc, b_start_loc,
+                          b_seq_len, max_seq_len, max_input_len, k_scale: torch.Tensor,
+                          v_scale: torch.Tensor, alibi_slopes=None, sliding_window=None,
+                          sm_scale=None, skip_decode=False, cos_sin_cache=None, rotary_dim=None,
+                          is_neox_style=True, is_lazy=None, q_offset=None, q_mask=None, *,
+                          _kernel: int = _ffi.KERNEL_AUTO, _num_splits: int = 0,
+                          _phases: int = _ffi.PHASE_ALL):
+    if is_lazy is None:
+        is_lazy = torch.zeros(b_seq_len.shape[0], dtype=torch.bool, device=q.device)
+        if cos_sin_cache is None:
+            cos_sin_cache = q.new_zeros((1, q.shape[-1]))
+            rotary_dim = q.shape[-1]
+        if q_offset is None:
+            q_offset = torch.zeros_like(b_loc, dtype=torch.int32)
+    elif q_offset is None:
+        raise ValueError("q_offset is required when is_lazy is given")
+    _launch.launch_prefill(
+        q=q, k=k, v=v, o=o, kv_cache_dtype=kv_cache_dtype, k_cache=k_cache, v_cache=v_cache,
+        b_loc=b_loc, b_start_loc=b_start_loc, b_seq_len=b_seq_len, max_input_len=max_input_len,
+        k_scale=k_scale, v_scale=v_scale, alibi_slopes=alibi_slopes, sliding_window=sliding_window,
+        sm_scale=sm_scale, skip_decode=skip_decode, cos_sin_cache=cos_sin_cache,
+        rotary_dim=rotary_dim, is_neox_style=is_neox_style, is_lazy=is_lazy, q_offset=q_offset,
+        q_mask=q_mask, pos_mode=_ffi.POS_BLOCK_UNIFORM, rotate_new_k=False, kernel=_kernel,
+        num_splits=_num_splits, phases=_phases)
+    return

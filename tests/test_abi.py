@@ -1,0 +1,115 @@
+"""The C-ABI library loads and exports every symbol include/lazyattn.h declares, and the
+host-side checks of the operators raise what the reference raises.  No GPU needed."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from lazy_amd import _ffi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "lazyattn.h")).read()
+    return sorted(set(re.findall(r"\b(lazyattn_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _ffi.lib()
+    names = _declared()
+    assert set(names) == set(_ffi.EXPORTS)
+    for n in names:
+        assert getattr(lib, n) is not None
+    assert lib.lazyattn_abi_version() == 1
+    assert lib.lazyattn_error_string(-4).decode().startswith("request not supported")
+
+
+def test_struct_layout_matches_header(tmp_path):
+    """Compile the header with gcc and compare sizeof/offsetof with the ctypes mirror."""
+    import subprocess
+    fields = [n for n, _ in _ffi.PrefillParams._fields_]
+    src = tmp_path / "layout.c"
+    src.write_text(
+        '#include <stdio.h>\n#include <stddef.h>\n#include "lazyattn.h"\nint main(void){\n'
+        + 'printf("%zu\\n", sizeof(lazyattn_prefill_params));\n'
+        + "".join(f'printf("%zu\\n", offsetof(lazyattn_prefill_params, {f}));\n' for f in fields)
+        + "return 0;}\n")
+    exe = tmp_path / "layout"
+    subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)])
+    out = [int(x) for x in subprocess.check_output([str(exe)]).split()]
+    assert out[0] == ctypes.sizeof(_ffi.PrefillParams)
+    assert out[1:] == [getattr(_ffi.PrefillParams, f).offset for f in fields]
+
+
+def test_null_and_shape_errors_without_gpu():
+    lib = _ffi.lib()
+    p = _ffi.PrefillParams()
+    assert lib.lazyattn_prefix_prefill(ctypes.byref(p), None) == -1
+    assert lib.lazyattn_prefix_prefill(None, None) == -1
+    assert lib.lazyattn_build_cos_sin_cache(None, 0, 8, 4, 8, 1e4, 0, 1.0, 1.0, 1.0, 8192, None) == -1
+    assert lib.lazyattn_build_cos_sin_cache(1, 0, 8, 4, 7, 1e4, 0, 1.0, 1.0, 1.0, 8192, None) == -2
+
+
+def _args(dtype=torch.float32, cache_dtype=None):
+    q = torch.zeros(4, 4, 64, dtype=dtype); k = torch.zeros(4, 2, 64, dtype=dtype); v = k.clone()
+    cd = cache_dtype or dtype
+    kc = torch.zeros(8, 2, 16, 16, 4, dtype=cd); vc = torch.zeros(8, 2, 64, 16, dtype=cd)
+    bt = torch.zeros(1, 4, dtype=torch.int32)
+    return [q, k, v, torch.zeros_like(q), "auto", kc, vc, bt, torch.tensor([0, 4]), torch.tensor([20]),
+            20, 4, torch.tensor(1.0), torch.tensor(1.0)]
+
+
+def test_reference_error_behaviour():
+    from lazy_amd.attention.old_ops.prefix_prefill import context_attention_fwd as f_old
+    from lazy_amd.attention.ops.prefix_prefill import context_attention_fwd as f_new
+    tab = torch.zeros(64, 64)
+    a = _args()
+    with pytest.raises(NotImplementedError):                   # ops/prefix_prefill.py:673-674
+        f_old(*a, alibi_slopes=torch.zeros(4), cos_sin_cache=tab, rotary_dim=64)
+    a = _args(); a[4] = "fp8"
+    with pytest.raises(AssertionError):                        # ops/prefix_prefill.py:637-639
+        f_old(*a, cos_sin_cache=tab, rotary_dim=64)
+    a = _args(cache_dtype=torch.uint8); a[4] = "fp8_e3m4"
+    with pytest.raises(ValueError, match="Unsupported FP8"):   # ops/prefix_prefill.py:646
+        f_new(*a, cos_sin_cache=tab, rotary_dim=64, is_lazy=torch.ones(1, dtype=torch.bool),
+              q_offset=torch.zeros(1, 4, dtype=torch.int32))
+    a = _args(cache_dtype=torch.uint8)
+    with pytest.raises(ValueError, match="auto"):              # ops/prefix_prefill.py:651-654
+        f_old(*a, cos_sin_cache=tab, rotary_dim=64)
+    a = _args(); a[8] = torch.tensor([0, 4, 8])
+    with pytest.raises(AssertionError):                        # ops/prefix_prefill.py:667
+        f_old(*a, cos_sin_cache=tab, rotary_dim=64)
+    a = _args(); a[2] = torch.zeros(4, 2, 32)
+    with pytest.raises(AssertionError):                        # ops/prefix_prefill.py:657-658
+        f_old(*a, cos_sin_cache=tab, rotary_dim=64)
+    with pytest.raises(RuntimeError, match="GPU only"):        # no CPU path
+        f_old(*_args(), cos_sin_cache=tab, rotary_dim=64)
+
+
+def test_metadata_producer_known_answer():
+    from lazy_amd.core.sched.metadata import (metadata_for_lazy_attention, metadata_for_mepic,
+                                              max_rotation_offset)
+    # lazy_attn/tests/core/test_scheduler.py:49-61
+    assert metadata_for_lazy_attention([6, 15, 8, 2], [8, 16, 8, 8], 8) == (
+        [10, 16, 16, 31, 39, 1], [2, 0, 1, 0, 6, 0])
+    assert metadata_for_mepic([6, 15, 8, 2], [8, 16, 8, 8], 8) == ([0] * 6, [2, 0, 1, 0, 6, 0])
+    # lazy_attn/tests/core/test_rotation_offset_bound.py:47-75
+    assert max_rotation_offset([1024] * 64, [1024] * 64) == 1024 * 63 + 1
+    assert max_rotation_offset([1] * 8, [16] * 8) == 8 * 15 + 7 + 1
+    for lens in ([6], [16, 16], [6, 15, 8, 2], [1] * 5, [4096, 17], [100] * 32):
+        padded = [((n + 15) // 16) * 16 for n in lens]
+        assert max_rotation_offset(lens, padded) == max(metadata_for_lazy_attention(lens, padded, 16)[0])
+
+
+def test_unpack_block_table_layout():
+    from lazy_amd.attention.ops.chunked_prefill_paged_decode import unpack_block_table
+    packed = torch.tensor([[(6 << 32) | (0xFFFF << 16) | 3, (123456 << 32) | (1 << 16)]], dtype=torch.int64)
+    blk, off, msk = unpack_block_table(packed)
+    assert blk.tolist() == [[6, 123456]] and off.tolist() == [[0xFFFF, 1]] and msk.tolist() == [[3, 0]]
+    # lazy_attn/tests/worker/test_q_offset_range.py:71-79: one past the limit carries into the block
+    over = (6 << 32) | ((0xFFFF + 1) << 16)
+    blk, off, _ = unpack_block_table(torch.tensor([[over]], dtype=torch.int64))
+    assert blk.item() == 7 and off.item() == 0
