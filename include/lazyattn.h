@@ -100,6 +100,8 @@ typedef struct lazyattn_prefill_params {
     int32_t num_splits;         /* context splits per work item; 0 = choose */
     int32_t phases;             /* LAZYATTN_PHASE_*; 0 = all */
     float sm_scale;
+    int32_t num_tokens;         /* rows of `o` (>= b_start_loc[B]); sizes the split-KV workspace */
+    int32_t max_seq_len;        /* upper bound of b_seq_len, 0 = unknown; only steers the split count */
     int32_t reserved;
 } lazyattn_prefill_params;
 

@@ -121,6 +121,7 @@ prefill_generic_kernel(const lazyattn_prefill_params p, const int decode) {
             kvalid[tid] = ok;
             kidx[tid] = (int)n;
         }
+        __syncthreads();   // masked slots are never loaded: they may hold anything, NaN included
         // ---- K tile: gather, rotate, store ----
         for (int i = tid; i < G_NT * half; i += G_THREADS) {
             const int kk = i / half, d1 = i % half, d2 = d1 + half;
@@ -134,7 +135,7 @@ prefill_generic_kernel(const lazyattn_prefill_params p, const int decode) {
                     k2 = to_f32(Kn[base + d2 * p.k_stride[2]]);
                     if (rot_new) pos = ctx_len + n;                    // old_ops:342-343
                 }
-            } else if (n < ctx_len) {
+            } else if (kvalid[kk]) {
                 const int64_t j = n / BS;
                 const int o = (int)(n % BS);
                 const int64_t pb = p.block_table[b * p.bt_stride[0] + j * p.bt_stride[1]];
@@ -177,7 +178,7 @@ prefill_generic_kernel(const lazyattn_prefill_params p, const int decode) {
             } else {
                 kk = i % G_NT; d = i / G_NT;     // slots fastest: matches [.., D, BS]
                 const int64_t n = n0 + kk;
-                if (n < ctx_len) {
+                if (kvalid[kk]) {
                     const int64_t pb = p.block_table[b * p.bt_stride[0] + (n / BS) * p.bt_stride[1]];
                     x = to_f32(VC[pb * p.vc_stride[0] + (int64_t)g * p.vc_stride[1] + d * p.vc_stride[2] +
                                   (n % BS) * p.vc_stride[3]]);

@@ -43,7 +43,8 @@ class PrefillParams(C.Structure):
                                     "cache_dtype", "table_dtype", "index_bits", "pos_mode",
                                     "rotate_new_k", "skip_decode", "fp32_rotary", "kernel",
                                     "num_splits", "phases")]
-        + [("sm_scale", C.c_float), ("reserved", C.c_int32)])
+        + [("sm_scale", C.c_float), ("num_tokens", C.c_int32), ("max_seq_len", C.c_int32),
+           ("reserved", C.c_int32)])
 
 
 def lib() -> C.CDLL:
@@ -110,7 +111,8 @@ def fill_params(*, q, k, v, o, k_cache, v_cache, block_table, b_start_loc, b_seq
                 cos_sin_cache, k_scale, v_scale, q_offset, q_mask, is_lazy, cache_code: int,
                 max_q_len: int, rotary_dim: int, sliding_window: int, sm_scale: float,
                 pos_mode: int, rotate_new_k: bool, skip_decode: bool, fp32_rotary: bool = False,
-                kernel: int = KERNEL_AUTO, num_splits: int = 0, phases: int = PHASE_ALL) -> PrefillParams:
+                kernel: int = KERNEL_AUTO, num_splits: int = 0, phases: int = PHASE_ALL,
+                max_seq_len: int = 0) -> PrefillParams:
     p = PrefillParams()
     p.q, p.k, p.v, p.o = _ptr(q), _ptr(k), _ptr(v), _ptr(o)
     p.k_cache, p.v_cache = _ptr(k_cache), _ptr(v_cache)
@@ -146,4 +148,6 @@ def fill_params(*, q, k, v, o, k_cache, v_cache, block_table, b_start_loc, b_seq
     p.num_splits = num_splits
     p.phases = phases
     p.sm_scale = float(sm_scale)
+    p.num_tokens = o.shape[0]
+    p.max_seq_len = int(max_seq_len or 0)
     return p

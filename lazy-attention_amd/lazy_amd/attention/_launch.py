@@ -45,7 +45,7 @@ def _require_gpu(*tensors) -> torch.device:
 
 
 def launch_prefill(*, q, k, v, o, kv_cache_dtype, k_cache, v_cache, b_loc, b_start_loc, b_seq_len,
-                   max_input_len, k_scale, v_scale, alibi_slopes, sliding_window, sm_scale,
+                   max_input_len, max_seq_len=0, k_scale, v_scale, alibi_slopes, sliding_window, sm_scale,
                    skip_decode, cos_sin_cache, rotary_dim, is_neox_style, is_lazy, q_offset, q_mask,
                    pos_mode: int, rotate_new_k: bool, fp32_rotary: bool = False,
                    kernel: int = _ffi.KERNEL_AUTO, num_splits: int = 0,
@@ -93,7 +93,7 @@ def launch_prefill(*, q, k, v, o, kv_cache_dtype, k_cache, v_cache, b_loc, b_sta
         is_lazy=is_lazy, cache_code=cache_code, max_q_len=max_input_len, rotary_dim=rotary_dim,
         sliding_window=sliding_window, sm_scale=sm_scale, pos_mode=pos_mode,
         rotate_new_k=rotate_new_k, skip_decode=skip_decode, fp32_rotary=fp32_rotary,
-        kernel=kernel, num_splits=num_splits, phases=phases)
+        kernel=kernel, num_splits=num_splits, phases=phases, max_seq_len=max_seq_len)
     stream = torch.cuda.current_stream(dev).cuda_stream
     if decode:
         _ffi.check(lib.lazyattn_paged_decode_rotary(p, stream), "lazyattn_paged_decode_rotary")

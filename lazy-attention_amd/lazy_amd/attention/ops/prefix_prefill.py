@@ -34,7 +34,7 @@ def context_attention_fwd(q, k, v, o, kv_cache_dtype: str, k_cache, v_cache, b_l
         raise ValueError("q_offset is required when is_lazy is given")
     _launch.launch_prefill(
         q=q, k=k, v=v, o=o, kv_cache_dtype=kv_cache_dtype, k_cache=k_cache, v_cache=v_cache,
-        b_loc=b_loc, b_start_loc=b_start_loc, b_seq_len=b_seq_len, max_input_len=max_input_len,
+        b_loc=b_loc, b_start_loc=b_start_loc, b_seq_len=b_seq_len, max_input_len=max_input_len, max_seq_len=max_seq_len,
         k_scale=k_scale, v_scale=v_scale, alibi_slopes=alibi_slopes, sliding_window=sliding_window,
         sm_scale=sm_scale, skip_decode=skip_decode, cos_sin_cache=cos_sin_cache,
         rotary_dim=rotary_dim, is_neox_style=is_neox_style, is_lazy=is_lazy, q_offset=q_offset,

@@ -24,7 +24,8 @@ def test_config1_fp32_plumbing():
     ref = run_oracle(w)
     got = run_op(w.to(DEV), kernel=_ffi.KERNEL_GENERIC).cpu()
     assert got.shape == (64, 32, 64)
-    assert (got - ref).abs().max().item() < 1e-5
+    err = (got - ref).abs().max().item()
+    assert err < 1e-5, err
 
 
 @pytest.mark.parametrize("variant", ["natural", "offset", "block_uniform"])
@@ -34,7 +35,8 @@ def test_generic_variants(variant, dtype):
     w = _small(variant, dtype)
     ref = run_oracle(w).float()
     got = run_op(w.to(DEV), kernel=_ffi.KERNEL_GENERIC).cpu().float()
-    assert (got - ref).abs().max().item() < TOL[dtype]
+    err = (got - ref).abs().max().item()
+    assert err < TOL[dtype], err
 
 
 @pytest.mark.parametrize("d,bs", [(32, 8), (128, 16), (96, 32), (256, 16)])
@@ -43,7 +45,8 @@ def test_generic_geometries(d, bs):
     w = _small("offset", torch.float32, d=d, bs=bs)
     ref = run_oracle(w)
     got = run_op(w.to(DEV), kernel=_ffi.KERNEL_GENERIC).cpu()
-    assert (got - ref).abs().max().item() < 1e-5
+    err = (got - ref).abs().max().item()
+    assert err < 1e-5, err
 
 
 def test_generic_sliding_window_skip_decode_and_int64_index():
@@ -53,7 +56,8 @@ def test_generic_sliding_window_skip_decode_and_int64_index():
     got = run_op(w.to(DEV), kernel=_ffi.KERNEL_GENERIC, sliding_window=37, skip_decode=True,
                  out=torch.full_like(w.q, 3.0).to(DEV), index_dtype=torch.int64).cpu()
     assert torch.all(got[70] == 3.0)                       # q_len == 1 request untouched
-    assert (got - ref).abs().max().item() < 1e-5
+    err = (got - ref).abs().max().item()
+    assert err < 1e-5, err
 
 
 def test_generic_vanilla_requests():
@@ -62,7 +66,8 @@ def test_generic_vanilla_requests():
     lazy = torch.tensor([True, False, False, True])
     ref = run_oracle(w, is_lazy=lazy)
     got = run_op(w.to(DEV), kernel=_ffi.KERNEL_GENERIC, is_lazy=lazy.to(DEV)).cpu()
-    assert (got - ref).abs().max().item() < 1e-5
+    err = (got - ref).abs().max().item()
+    assert err < 1e-5, err
 
 
 @pytest.mark.parametrize("kv", ["fp8", "fp8_e5m2"])
@@ -76,7 +81,8 @@ def test_generic_fp8_cache(kv):
         w.k_scale = torch.tensor(2.0 ** -12); w.v_scale = torch.tensor(2.0 ** -12)
     ref = run_oracle(w).float()
     got = run_op(w.to(DEV), kernel=_ffi.KERNEL_GENERIC).cpu().float()
-    assert (got - ref).abs().max().item() < 5e-2
+    err = (got - ref).abs().max().item()
+    assert err < 5e-2, err
 
 
 def test_pad_slots_may_hold_nan():
@@ -92,7 +98,8 @@ def test_pad_slots_may_hold_nan():
                 w.k_cache[pb, :, :, bs - m:, :] = float("nan")
                 w.v_cache[pb, :, :, bs - m:] = float("nan")
     got = run_op(w.to(DEV), kernel=_ffi.KERNEL_GENERIC).cpu()
-    assert (got - ref).abs().max().item() < 1e-5
+    err = (got - ref).abs().max().item()
+    assert err < 1e-5, err
 
 
 def test_no_context_request():
@@ -102,7 +109,8 @@ def test_no_context_request():
                          variant="natural", seed=2)
     ref = run_oracle(w)
     got = run_op(w.to(DEV), kernel=_ffi.KERNEL_GENERIC).cpu()
-    assert (got - ref).abs().max().item() < 1e-5
+    err = (got - ref).abs().max().item()
+    assert err < 1e-5, err
 
 
 def test_cos_sin_builder_matches_closed_form():
@@ -117,7 +125,8 @@ def test_cos_sin_builder_matches_closed_form():
         got = build_cos_sin_cache(66000, 128, meta, base=500000.0, dtype=torch.float32).cpu()
         ref = orc.build_cos_sin_table(66000, 128, 500000.0, llama3=l3, dtype=torch.float64,
                                       math_dtype=torch.float64)
-        assert (got.double() - ref).abs().max().item() < 1e-7
+        err = (got.double() - ref).abs().max().item()
+    assert err < 1e-7, err
     got = build_cos_sin_cache(4096, 64, None, base=10000.0, dtype=torch.bfloat16).cpu()
     ref = orc.build_cos_sin_table(4096, 64, 10000.0, dtype=torch.float64, math_dtype=torch.float64)
     assert torch.equal(got, ref.to(torch.bfloat16))
