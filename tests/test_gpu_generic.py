@@ -129,4 +129,8 @@ def test_cos_sin_builder_matches_closed_form():
     assert err < 1e-7, err
     got = build_cos_sin_cache(4096, 64, None, base=10000.0, dtype=torch.bfloat16).cpu()
     ref = orc.build_cos_sin_table(4096, 64, 10000.0, dtype=torch.float64, math_dtype=torch.float64)
-    assert torch.equal(got, ref.to(torch.bfloat16))
+    want = ref.float().to(torch.bfloat16)
+    # bf16 rounding of the same fp32 value; a last-place difference of the device's double
+    # cos/sin can flip a tie, so allow one bf16 ulp on a vanishing fraction of entries
+    assert (got.float() - want.float()).abs().max().item() <= 2.0 ** -8
+    assert (got != want).float().mean().item() < 1e-3
