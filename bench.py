@@ -1,0 +1,143 @@
+#!/usr/bin/env python3
+"""Benchmark of the deferred-RoPE prefix-prefill operator on one MI355X.
+
+A step is one call of the operator (rotate cached K per page, QK^T, online softmax, PV,
+split-KV merge) on a synthetic batch that is already resident in HBM.  The default
+workload is the north-star configuration: Llama-3-8B geometry, bf16, 10 x 512-token
+shuffled documents, 128 query tokens.  Prints one JSON line.
+
+    python bench.py [--steps K] [--warmup W] [--config 2|3|4|5] [--num-splits S] [--no-cpu]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "lazy-attention_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0
+
+
+def make_plan(g, num_splits, phases):
+    import torch
+    from lazy_amd import _ffi
+    from lazy_amd.attention.old_ops.prefix_prefill import context_attention_fwd
+    o = torch.zeros_like(g.q)
+    plan = context_attention_fwd(
+        g.q, g.k, g.v, o, g.kv_cache_dtype, g.k_cache, g.v_cache, g.block_table, g.b_start_loc,
+        g.b_seq_len, g.max_seq_len, g.max_query_len, g.k_scale, g.v_scale,
+        cos_sin_cache=g.cos_sin_cache, rotary_dim=g.q.shape[-1], q_mask=g.q_mask, q_offset=g.q_offset,
+        is_mepic=True, _num_splits=num_splits, _phases=phases, _return_plan=True)
+    return plan, o
+
+
+def time_calls(plan, n):
+    """ms per call over n back-to-back launches, HIP events on the launch stream."""
+    import torch
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(n):
+        plan.run()
+    end.record()
+    end.synchronize()
+    return start.elapsed_time(end) / n
+
+
+def cpu_baseline(w, reps):
+    """The float32 PyTorch-eager statement of the same op on the host cores."""
+    import torch
+    from oracle import deferred_rope as orc
+
+    def once():
+        t = time.perf_counter()
+        orc.prefix_prefill(w.q, w.k, w.v, w.k_cache, w.v_cache, w.block_table, w.b_start_loc,
+                           w.b_seq_len, w.cos_sin_cache, w.q_offset, w.q_mask, pos_mode=w.pos_mode,
+                           rotate_new_k=w.rotate_new_k, kv_cache_dtype=w.kv_cache_dtype,
+                           k_scale=w.k_scale, v_scale=w.v_scale)
+        return time.perf_counter() - t
+    once()
+    return statistics.median(once() for _ in range(reps))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5])
+    ap.add_argument("--num-splits", type=int, default=0)
+    ap.add_argument("--no-cpu", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: the operator has no multi-GPU path "
+              "(kv-heads / requests shard without any exchange); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from lazy_amd import _ffi, workloads as wl
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    _ffi.lib()
+    torch.cuda.set_device(0)
+    w = wl.config(a.config)
+    g = w.to("cuda:0")
+    plan, o = make_plan(g, a.num_splits, _ffi.PHASE_ALL)
+    main_only, _ = make_plan(g, a.num_splits, _ffi.PHASE_MAIN)
+
+    for _ in range(a.warmup):
+        plan.run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ms = time_calls(plan, a.steps)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / a.steps
+    # the dominant kernel alone (no merge launch), same stream, same events
+    for _ in range(a.warmup):
+        main_only.run()
+    torch.cuda.synchronize()
+    reps = [time_calls(main_only, max(a.steps // 4, 10)) for _ in range(7)]
+    main_ms = statistics.median(reps)
+    plan.run()
+    torch.cuda.synchronize()
+
+    tflops = w.flops / (ms * 1e-3) / 1e12
+    main_tflops = w.flops / (main_ms * 1e-3) / 1e12
+    out = {
+        "metric": "deferred-RoPE prefix-prefill TFLOP/s (8B geometry, 5K context); ms/call and MFMA fraction alongside",
+        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms, 5), "ms_per_call": round(ms, 5), "wall_ms_per_step": round(wall_ms, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": w.name, "hq": 32, "hkv": 8, "head_dim": 128, "page": 16,
+                   "requests": int(w.b_seq_len.numel()), "ctx_keys": int(w.b_seq_len[0] - w.max_query_len),
+                   "query_tokens": int(w.max_query_len), "kv_cache": w.kv_cache_dtype,
+                   "gflop_per_call": round(w.flops / 1e9, 3), "mb_per_call": round(w.bytes / 1e6, 2)},
+        "roofline": {"bound": "mfma", "achieved": round(main_tflops, 2), "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(main_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "kernel": "prefill_mfma_kernel", "kernel_ms": round(main_ms, 5),
+                     "hbm_gbs_algorithmic": round(w.bytes / (main_ms * 1e-3) / 1e9, 1)},
+    }
+    if not a.no_cpu:
+        torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))
+        reps_cpu = 5 if a.config in (2, 3) else 3
+        wc = w if a.config in (2, 3) else wl.config(a.config, shrink=8)
+        sec = cpu_baseline(wc, reps_cpu)
+        out["cpu_baseline"] = {"value": round(wc.flops / sec / 1e12, 4), "unit": "TFLOP/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"{wc.name}: {reps_cpu} full calls, median {sec * 1e3:.1f} ms/call"
+                                         + ("" if wc is w else " (1/8 of the documents)")}
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

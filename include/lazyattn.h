@@ -72,6 +72,9 @@ typedef struct lazyattn_prefill_params {
     const void *b_start_loc;    /* [B+1] int32 or int64, see index_bits */
     const void *b_seq_len;      /* [B] */
     const void *cos_sin_cache;  /* [max_pos, rotary_dim]: row p = cos(p*inv) | sin(p*inv) */
+    const void *cos_sin_packed; /* optional: the same table re-laid out by lazyattn_pack_cos_sin_cache()
+                                   as [2][rotary_dim/16][packed_rows][8], so that the 16 slots of a page
+                                   read 16 consecutive 16-byte chunks; NULL = read the row-major table */
     const float *k_scale;       /* 1 element, read only for fp8 caches */
     const float *v_scale;
     void *workspace;            /* split-KV partials; lazyattn_prefill_workspace_bytes() */
@@ -102,7 +105,7 @@ typedef struct lazyattn_prefill_params {
     float sm_scale;
     int32_t num_tokens;         /* rows of `o` (>= b_start_loc[B]); sizes the split-KV workspace */
     int32_t max_seq_len;        /* upper bound of b_seq_len, 0 = unknown; only steers the split count */
-    int32_t reserved;
+    int32_t packed_rows;        /* rows of cos_sin_packed (0 when it is NULL) */
 } lazyattn_prefill_params;
 
 /* Bytes of workspace lazyattn_prefix_prefill() may need for these sizes (0 when the
@@ -137,6 +140,13 @@ int lazyattn_build_cos_sin_cache(void *out, int32_t out_dtype, int64_t row_strid
                                  int32_t rope_type, double scaling_factor,
                                  double low_freq_factor, double high_freq_factor,
                                  int32_t orig_max_position, void *stream);
+
+/* Re-layout of a cos/sin table for the MFMA kernel's per-token gather:
+ * packed[h][c][p][e] = table[p, h*R/2 + c*8 + e]  (h = 0 cos, 1 sin; c < R/16; e < 8).
+ * `packed` holds rows * rotary_dim elements of the table's type.  Done once per table
+ * (the table is a model constant); no reference counterpart. */
+int lazyattn_pack_cos_sin_cache(const void *table, void *packed, int32_t dtype, int64_t row_stride,
+                                int32_t rows, int32_t rotary_dim, void *stream);
 
 const char *lazyattn_error_string(int code);
 int lazyattn_abi_version(void);

@@ -9,6 +9,8 @@ size_t mfma_workspace_bytes(const lazyattn_prefill_params &p);
 int launch_cos_sin_table(void *out, int out_dtype, int64_t row_stride, int max_position,
                          int rotary_dim, double base, int rope_type, double factor, double low,
                          double high, int orig_max, hipStream_t stream);
+int launch_pack_cos_sin(const void *table, void *packed, int dtype, int64_t row_stride, int rows,
+                        int rotary_dim, hipStream_t stream);
 }  // namespace lazyattn
 
 using namespace lazyattn;
@@ -95,6 +97,13 @@ extern "C" int lazyattn_build_cos_sin_cache(void *out, int32_t out_dtype, int64_
     return launch_cos_sin_table(out, out_dtype, row_stride, max_position, rotary_dim, base, rope_type,
                                 scaling_factor, low_freq_factor, high_freq_factor, orig_max_position,
                                 (hipStream_t)stream);
+}
+
+extern "C" int lazyattn_pack_cos_sin_cache(const void *table, void *packed, int32_t dtype, int64_t row_stride,
+                                           int32_t rows, int32_t rotary_dim, void *stream) {
+    if (!table || !packed) return LAZYATTN_E_NULL;
+    if (rows < 0 || rotary_dim <= 0 || rotary_dim % 16 || row_stride < rotary_dim) return LAZYATTN_E_SHAPE;
+    return launch_pack_cos_sin(table, packed, dtype, row_stride, rows, rotary_dim, (hipStream_t)stream);
 }
 
 extern "C" const char *lazyattn_error_string(int code) {

@@ -9,18 +9,20 @@
 // reference's grid (batch, q_head, m_tile) does (ops/prefix_prefill.py:681-682).
 //
 // Per 64-key tile:
-//   gather   4 pages of K ([D/x][16][x], 4 KB each for bf16) with 16-byte loads, the
-//            matching cos/sin rows, and 4 pages of V ([D][16]);
+//   gather   4 pages of K ([D/x][16][x], one contiguous 4 KB run per page and kv-head for
+//            bf16) with 16-byte loads off a wave-uniform base, the matching cos/sin rows,
+//            and 4 pages of V ([D][16]);
 //   rotate   k1*c - k2*s, k1*s + k2*c in fp32 registers, one rounding to bf16
 //            (old_ops/prefix_prefill.py:248-257 with FORCE_FP32_ROTARY), write to LDS in
 //            the cache's own [page][D/8][slot][8] order, which is exactly the A-operand
 //            order of v_mfma_f32_32x32x16_bf16;
-//   S^T      = K . Q^T (keys x rows), 32x32x16 MFMA, Q fragments stay in registers;
+//   S^T      = K . Q^T (keys x rows) in two 32-key halves, Q fragments stay in registers;
 //   softmax  per lane one query row; row max via one v_permlane32_swap; exp2 with
 //            sm_scale*log2(e) folded into one fma (old_ops:287-291);
 //   O^T     += V^T . P^T: the S^T accumulator registers ARE the B operand (the k index of
 //            the MFMA is permuted so that no shuffle is needed), V^T comes from LDS.
-// The new tokens' K/V (old_ops:326-396) are appended as further tiles with a causal mask.
+// Tiles come in three kinds: full context tiles (no masking code at all), edge context
+// tiles (pad slots / end of context) and new-token tiles (old_ops:326-396, causal mask).
 // With more than one split every workgroup writes (O/l, log2-sum-exp) partials and a
 // second kernel merges them.
 #include "common.hpp"
@@ -30,7 +32,6 @@ namespace lazyattn {
 namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
-typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 typedef __attribute__((ext_vector_type(2))) float f32x2_t;
@@ -41,304 +42,111 @@ constexpr int BS = 16;          // page size (tokens)
 constexpr int NT = 64;          // keys per tile
 constexpr int PAGES = NT / BS;  // pages per tile
 constexpr int UNIT = 32;        // query rows per wave
-// LDS tile layouts (bytes)
-constexpr int K_PAGE = 4096;            // [d8 = 16][slot = 16][8 bf16]
-constexpr int K_TILE = PAGES * K_PAGE;  // 16 KB
-constexpr int V_SG = 1024 + 64;         // [sg = slot/4][d = 128][4 slots], padded
-constexpr int V_PAGE = 4 * V_SG;
-constexpr int V_TILE = PAGES * V_PAGE;  // 17 KB
-constexpr int LDS_BYTES = 2 * (K_TILE + V_TILE);
+// LDS tiles (bytes).  K: [page][d8 = 16][slot = 16][8 bf16].
+// V: [page][g = 2][d = 128][slots 4g..4g+3 | slots 8+4g..8+4g+3] -- the 16 bytes one lane
+// feeds to the PV MFMA as its A operand.
+constexpr int K_PAGE = 4096;
+constexpr int K_TILE = PAGES * K_PAGE;
+constexpr int V_G = 2048;
+constexpr int V_PAGE = 2 * V_G;
+constexpr int V_TILE = PAGES * V_PAGE;
+constexpr int LDS_BYTES = 2 * (K_TILE + V_TILE);   // double buffered: 64 KB
+
+enum { TILE_FULL = 0, TILE_EDGE = 1, TILE_NEW = 2 };
 
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
-// value of x in the partner lane (lane ^ 32) of a 64-wide wave, via v_permlane32_swap.
-// The two operands are kept distinct registers on purpose.
-__device__ __forceinline__ float partner32(float x) {
-    uint32_t a = __float_as_uint(x), b = a;
-    asm volatile("" : "+v"(b));
-    auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
-    // r[0] = {a.lo, b.lo}, r[1] = {a.hi, b.hi}: lanes < 32 want r[1], lanes >= 32 want r[0]
-    return __uint_as_float((threadIdx.x & 32) ? r[0] : r[1]);
-}
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
     f32x2_t f = {a, b};
     bf16x2_t h = __builtin_convertvector(f, bf16x2_t);   // v_cvt_pk_bf16_f32, RNE
     return *reinterpret_cast<uint32_t *>(&h);
 }
+// value of x in the partner lane (lane ^ 32) of the wave, via v_permlane32_swap
+__device__ __forceinline__ float partner32(float x, bool upper) {
+    uint32_t a = __float_as_uint(x), b = a;
+    asm volatile("" : "+v"(b));      // two distinct registers for the swap
+    auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+    // r[0] = {a.lo, b.lo}, r[1] = {a.hi, b.hi}
+    return __uint_as_float(upper ? r[0] : r[1]);
+}
+__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
 
-// 8 consecutive table entries as floats
+__device__ __forceinline__ uint4 ldg16(const uint8_t *base, uint32_t off) {
+    return *reinterpret_cast<const uint4 *>(base + off);
+}
+__device__ __forceinline__ uint2 ldg8(const uint8_t *base, uint32_t off) {
+    return *reinterpret_cast<const uint2 *>(base + off);
+}
+
+// 8 consecutive cos (or sin) table entries
 template <typename TT> struct TabVec;
 template <> struct TabVec<bf16_t> {
     uint4 v;
-    __device__ __forceinline__ void load(const void *p) { v = *reinterpret_cast<const uint4 *>(p); }
-    __device__ __forceinline__ void identity(bool cosine) {
-        const uint32_t w = cosine ? 0x3f803f80u : 0u;
-        v = make_uint4(w, w, w, w);
+    __device__ __forceinline__ void load(const uint8_t *base, uint32_t off) { v = ldg16(base, off); }
+    __device__ __forceinline__ void fill(float w) {
+        const uint32_t u = __float_as_uint(w) >> 16;
+        v = make_uint4(u | (u << 16), u | (u << 16), u | (u << 16), u | (u << 16));
     }
-    __device__ __forceinline__ float get(int i) const {
-        const uint32_t w = (&v.x)[i >> 1];
-        return (i & 1) ? bf16_hi(w) : bf16_lo(w);
+    __device__ __forceinline__ void get(float *f) const {
+        f[0] = bf16_lo(v.x); f[1] = bf16_hi(v.x); f[2] = bf16_lo(v.y); f[3] = bf16_hi(v.y);
+        f[4] = bf16_lo(v.z); f[5] = bf16_hi(v.z); f[6] = bf16_lo(v.w); f[7] = bf16_hi(v.w);
     }
 };
 template <> struct TabVec<float> {
     float4 a, b;
-    __device__ __forceinline__ void load(const void *p) {
-        a = reinterpret_cast<const float4 *>(p)[0];
-        b = reinterpret_cast<const float4 *>(p)[1];
+    __device__ __forceinline__ void load(const uint8_t *base, uint32_t off) {
+        a = *reinterpret_cast<const float4 *>(base + off);
+        b = *reinterpret_cast<const float4 *>(base + off + 16);
     }
-    __device__ __forceinline__ void identity(bool cosine) {
-        const float w = cosine ? 1.f : 0.f;
-        a = make_float4(w, w, w, w); b = a;
+    __device__ __forceinline__ void fill(float w) { a = make_float4(w, w, w, w); b = a; }
+    __device__ __forceinline__ void get(float *f) const {
+        f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
     }
-    __device__ __forceinline__ float get(int i) const { return i < 4 ? (&a.x)[i] : (&b.x)[i - 4]; }
 };
 
-// one K work item: 8 (d, d+64) pairs of one key
-template <typename TT> struct KItem {
-    uint4 k1, k2;        // raw: 8 bf16 each, or 8 fp8 in .x/.y
+__device__ __forceinline__ void unpack8(const uint4 &w, float *f) {
+    f[0] = bf16_lo(w.x); f[1] = bf16_hi(w.x); f[2] = bf16_lo(w.y); f[3] = bf16_hi(w.y);
+    f[4] = bf16_lo(w.z); f[5] = bf16_hi(w.z); f[6] = bf16_lo(w.w); f[7] = bf16_hi(w.w);
+}
+// 8 fp8 e4m3 bytes -> (float * scale) rounded to bf16, as floats  (old_ops:239-241)
+__device__ __forceinline__ void unpack8_fp8(uint32_t lo, uint32_t hi, float scale, float *f) {
+    const f32x2_t a = __builtin_amdgcn_cvt_pk_f32_fp8(lo, false), b = __builtin_amdgcn_cvt_pk_f32_fp8(lo >> 16, false);
+    const f32x2_t c = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false), d = __builtin_amdgcn_cvt_pk_f32_fp8(hi >> 16, false);
+    const float t[8] = {a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = round_to<bf16_t>(t[i] * scale);
+}
+
+// one K item in flight: 8 (d, d+64) pairs of one key
+template <typename TT> struct KRegs {
+    uint4 k1, k2;
     TabVec<TT> c, s;
-    int lds_off;         // byte offset of chunk d8 inside the K tile; chunk d8+8 is +8*256
-    int kind;            // 0 = zero fill, 1 = bf16, 2 = fp8 e4m3
+    uint32_t lds_off;
 };
-struct VItem {
-    uint4 v;             // ctx bf16: 8 slots of one d; ctx fp8: 16 slots of one d; new: 8 d of one key
-    int a0, a1;          // ctx: LDS byte offsets; new: (page, slot) packed
-    int lim;             // valid slots in the page (ctx) / 1 = valid (new)
-    int kind;            // -1 no item, 1 ctx bf16, 2 ctx fp8, 3 new-token row
-};
-
-struct Ctx {
-    const lazyattn_prefill_params *p;
-    int b, g;
-    int64_t qs, q_len, ctx_len;
-    int n_pages;         // pages holding context keys
-    int pos_mode;
-    bool vanilla, rot_new;
-    float k_scale, v_scale;
-    int t_end;           // new-token keys this workgroup can see: [0, t_end)
-};
-
-// valid slots of context page j: slot < lim
-__device__ __forceinline__ int page_limit(const Ctx &c, int j) {
-    if (j >= c.n_pages) return 0;
-    int64_t lim = c.ctx_len - (int64_t)j * BS;
-    if (lim > BS) lim = BS;
-    if (!c.vanilla && c.p->q_mask) {
-        const int qm = c.p->q_mask[c.b * c.p->qm_stride[0] + j * c.p->qm_stride[1]];   // old_ops:165-167
-        if (BS - qm < lim) lim = BS - qm;
-    }
-    return lim < 0 ? 0 : (int)lim;
-}
-
-template <typename TT>
-__device__ __forceinline__ void load_table(const Ctx &c, KItem<TT> &it, int64_t pos, int cp) {
-    const TT *tab = (const TT *)c.p->cos_sin_cache + pos * c.p->table_stride + cp * 8;
-    it.c.load(tab);
-    it.s.load(tab + HALF);
-}
-
-// ---- issue the global loads of one K item of tile `tile` ----
-template <bool FP8, typename TT>
-__device__ __forceinline__ void load_k_item(const Ctx &c, KItem<TT> &it, int tile, int n_ctx_tiles, int idx) {
-    const lazyattn_prefill_params &p = *c.p;
-    it.kind = 0;
-    it.k1 = make_uint4(0, 0, 0, 0); it.k2 = it.k1;
-    if (tile < n_ctx_tiles) {
-        const int o = idx & 15, cp = (idx >> 4) & 7, pg = idx >> 7;
-        const int j = tile * PAGES + pg;
-        it.lds_off = pg * K_PAGE + cp * 256 + o * 16;
-        if (j >= c.n_pages) return;
-        const int64_t pb = p.block_table[c.b * p.bt_stride[0] + j * p.bt_stride[1]];
-        int64_t pos = -1;
-        if (!c.vanilla) {
-            if (c.pos_mode == LAZYATTN_POS_NATURAL) {
-                pos = (int64_t)j * BS + o;                                          // old_ops:183-184
-            } else {
-                const int qo = p.q_offset[c.b * p.qo_stride[0] + j * p.qo_stride[1]];
-                if (c.pos_mode == LAZYATTN_POS_OFFSET) pos = qo ? (int64_t)qo - 1 + o : (int64_t)j * BS + o;
-                else pos = qo ? (int64_t)qo - 1 : 0;                                // ops:180-186
-            }
-        }
-        if (FP8) {
-            // [D/16][16 slots][16]: this item takes 8 bytes of chunk cp/2 and of chunk cp/2+4
-            const uint8_t *kc = (const uint8_t *)p.k_cache + pb * p.kc_stride[0] + (int64_t)c.g * p.kc_stride[1] +
-                                (cp >> 1) * p.kc_stride[2] + o * 16 + (cp & 1) * 8;
-            const uint2 a = *reinterpret_cast<const uint2 *>(kc);
-            const uint2 b2 = *reinterpret_cast<const uint2 *>(kc + 4 * p.kc_stride[2]);
-            it.k1.x = a.x; it.k1.y = a.y; it.k2.x = b2.x; it.k2.y = b2.y;
-            it.kind = 2;
-        } else {
-            const bf16_t *kc = (const bf16_t *)p.k_cache + pb * p.kc_stride[0] + (int64_t)c.g * p.kc_stride[1] +
-                               cp * p.kc_stride[2] + o * 8;
-            it.k1 = *reinterpret_cast<const uint4 *>(kc);
-            it.k2 = *reinterpret_cast<const uint4 *>(kc + 8 * p.kc_stride[2]);
-            it.kind = 1;
-        }
-        if (pos >= 0) load_table<TT>(c, it, pos, cp);
-        else { it.c.identity(true); it.s.identity(false); }
-    } else {
-        // new-token keys: [T, Hkv, D] rows
-        const int cp = idx & 7, kl = idx >> 3;
-        const int m = (tile - n_ctx_tiles) * NT + kl;
-        it.lds_off = (kl >> 4) * K_PAGE + cp * 256 + (kl & 15) * 16;
-        if (m >= c.t_end) return;
-        const bf16_t *kn = (const bf16_t *)p.k + (c.qs + m) * p.k_stride[0] + (int64_t)c.g * p.k_stride[1] + cp * 8;
-        it.k1 = *reinterpret_cast<const uint4 *>(kn);
-        it.k2 = *reinterpret_cast<const uint4 *>(kn + HALF);
-        it.kind = 1;
-        if (c.rot_new) load_table<TT>(c, it, c.ctx_len + m, cp);                    // old_ops:342-343
-        else { it.c.identity(true); it.s.identity(false); }
-    }
-}
-
-__device__ __forceinline__ void fp8x8_to_f32(uint32_t lo, uint32_t hi, float scale, float *out) {
-    // (the word-select form of the conversion crashes this compiler's copy propagation)
-    f32x2_t a = __builtin_amdgcn_cvt_pk_f32_fp8(lo, false), b = __builtin_amdgcn_cvt_pk_f32_fp8(lo >> 16, false);
-    f32x2_t c2 = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false), d2 = __builtin_amdgcn_cvt_pk_f32_fp8(hi >> 16, false);
-    out[0] = a[0] * scale; out[1] = a[1] * scale; out[2] = b[0] * scale; out[3] = b[1] * scale;
-    out[4] = c2[0] * scale; out[5] = c2[1] * scale; out[6] = d2[0] * scale; out[7] = d2[1] * scale;
-}
-
-// ---- rotate one K item in fp32 and write both chunks to the LDS tile ----
-template <typename TT>
-__device__ __forceinline__ void rotate_store_k(const KItem<TT> &it, uint8_t *ktile, float k_scale) {
-    uint4 r1, r2;
-    if (it.kind == 0) {
-        r1 = make_uint4(0, 0, 0, 0); r2 = r1;
-    } else {
-        float a[8], b[8];
-        if (it.kind == 2) {
-            fp8x8_to_f32(it.k1.x, it.k1.y, k_scale, a);
-            fp8x8_to_f32(it.k2.x, it.k2.y, k_scale, b);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {          // (x.f32 * k_scale).to(bf16): old_ops:239-241
-                a[i] = round_to<bf16_t>(a[i]);
-                b[i] = round_to<bf16_t>(b[i]);
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const uint32_t w1 = (&it.k1.x)[i], w2 = (&it.k2.x)[i];
-                a[2 * i] = bf16_lo(w1); a[2 * i + 1] = bf16_hi(w1);
-                b[2 * i] = bf16_lo(w2); b[2 * i + 1] = bf16_hi(w2);
-            }
-        }
-        float x[8], y[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const float cs = it.c.get(i), sn = it.s.get(i);
-            x[i] = a[i] * cs - b[i] * sn;                                           // old_ops:253
-            y[i] = a[i] * sn + b[i] * cs;                                           // old_ops:254
-        }
-        r1 = make_uint4(pack_bf16(x[0], x[1]), pack_bf16(x[2], x[3]), pack_bf16(x[4], x[5]), pack_bf16(x[6], x[7]));
-        r2 = make_uint4(pack_bf16(y[0], y[1]), pack_bf16(y[2], y[3]), pack_bf16(y[4], y[5]), pack_bf16(y[6], y[7]));
-    }
-    *reinterpret_cast<uint4 *>(ktile + it.lds_off) = r1;
-    *reinterpret_cast<uint4 *>(ktile + it.lds_off + 8 * 256) = r2;
-}
-
-// ---- V items ----
-template <bool FP8>
-__device__ __forceinline__ void load_v_item(const Ctx &c, VItem &it, int tile, int n_ctx_tiles, int idx) {
-    const lazyattn_prefill_params &p = *c.p;
-    it.kind = 0;
-    it.v = make_uint4(0, 0, 0, 0);
-    if (tile < n_ctx_tiles) {
-        if (FP8) {
-            // [D][16 slots] bytes: one item = all 16 slots of one d
-            const int d = idx & 127, pg = idx >> 7;
-            const int j = tile * PAGES + pg;
-            it.a0 = pg * V_PAGE + d * 8;
-            it.lim = page_limit(c, j);
-            it.kind = 2;
-            if (it.lim <= 0) return;                     // stored as zeros
-            const int64_t pb = p.block_table[c.b * p.bt_stride[0] + j * p.bt_stride[1]];
-            const uint8_t *vc = (const uint8_t *)p.v_cache + pb * p.vc_stride[0] + (int64_t)c.g * p.vc_stride[1] + d * 16;
-            it.v = *reinterpret_cast<const uint4 *>(vc);
-            it.kind = 2;
-        } else {
-            // [D][16 slots] bf16: one item = 8 slots (half a row) of one d
-            const int d = idx & 127, hf = (idx >> 7) & 1, pg = idx >> 8;
-            const int j = tile * PAGES + pg;
-            it.a0 = pg * V_PAGE + (2 * hf) * V_SG + d * 8;
-            it.a1 = hf;
-            it.lim = page_limit(c, j);
-            it.kind = 1;
-            if (it.lim <= 0) return;                     // stored as zeros
-            const int64_t pb = p.block_table[c.b * p.bt_stride[0] + j * p.bt_stride[1]];
-            const bf16_t *vc = (const bf16_t *)p.v_cache + pb * p.vc_stride[0] + (int64_t)c.g * p.vc_stride[1] +
-                               d * 16 + hf * 8;
-            it.v = *reinterpret_cast<const uint4 *>(vc);
-            it.kind = 1;
-        }
-    } else {
-        const int dc = idx & 15, kl = idx >> 4;          // 8 d of one new-token key
-        const int m = (tile - n_ctx_tiles) * NT + kl;
-        it.a0 = (kl >> 4) * V_PAGE + ((kl & 15) >> 2) * V_SG + (dc * 8) * 8 + (kl & 3) * 2;
-        it.kind = 3;
-        if (m >= c.t_end) return;                        // stays zero
-        const bf16_t *vn = (const bf16_t *)p.v + (c.qs + m) * p.v_stride[0] + (int64_t)c.g * p.v_stride[1] + dc * 8;
-        it.v = *reinterpret_cast<const uint4 *>(vn);
-    }
-}
-
-__device__ __forceinline__ void store_v_item(const VItem &it, uint8_t *vtile, float v_scale) {
-    if (it.kind == 3) {
-        // one key, 8 d: scatter 2-byte entries into [sg][d][slot%4]
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const uint32_t w = (&it.v.x)[i];
-            *reinterpret_cast<uint16_t *>(vtile + it.a0 + (2 * i) * 8) = (uint16_t)(w & 0xffffu);
-            *reinterpret_cast<uint16_t *>(vtile + it.a0 + (2 * i + 1) * 8) = (uint16_t)(w >> 16);
-        }
-        return;
-    }
-    if (it.kind == 2) {
-        // 16 fp8 slots of one d -> bf16, four 8-byte groups of 4 slots
-        const uint32_t *w = &it.v.x;
-#pragma unroll
-        for (int sg = 0; sg < 4; ++sg) {
-            f32x2_t lo = __builtin_amdgcn_cvt_pk_f32_fp8(w[sg], false), hi = __builtin_amdgcn_cvt_pk_f32_fp8(w[sg] >> 16, false);
-            float f[4] = {lo[0] * v_scale, lo[1] * v_scale, hi[0] * v_scale, hi[1] * v_scale};
-#pragma unroll
-            for (int s = 0; s < 4; ++s)
-                if (sg * 4 + s >= it.lim) f[s] = 0.f;    // masked slots contribute nothing, whatever they hold
-            uint2 out = make_uint2(pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]));
-            *reinterpret_cast<uint2 *>(vtile + it.a0 + sg * V_SG) = out;
-        }
-        return;
-    }
-    uint4 v = it.v;
-    if (it.lim < BS) {
-        const int first = it.a1 * 8;                     // slot of element 0
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            uint32_t w = (&v.x)[i];
-            if (first + 2 * i >= it.lim) w &= 0xffff0000u;
-            if (first + 2 * i + 1 >= it.lim) w &= 0x0000ffffu;
-            (&v.x)[i] = w;
-        }
-    }
-    *reinterpret_cast<uint2 *>(vtile + it.a0) = make_uint2(v.x, v.y);
-    *reinterpret_cast<uint2 *>(vtile + it.a0 + V_SG) = make_uint2(v.z, v.w);
-}
 
 }  // namespace
 
-template <int NW, bool FP8, typename TT>
-__global__ void __launch_bounds__(NW * 64)
+// Workgroup = 8 waves: waves 0-3 compute (32 query rows each), waves 4-7 gather.  The
+// hardware places wave w on SIMD w % 4, so every SIMD hosts one computing and one
+// gathering wave: the gather's address arithmetic, fp32 rotation and LDS writes run in
+// the shadow of the other wave's MFMAs, and neither role ever waits for the other's
+// memory latency -- they only meet at one barrier per tile.
+constexpr int NC = 4;                    // computing waves = units per workgroup
+constexpr int LT = 256;                  // gathering threads
+constexpr int KI = (NT * 8) / LT;        // K items per gathering thread and tile (512 per tile)
+constexpr int VI = (NT * 16) / LT;       // V items per gathering thread and tile (1024 of 16 bytes)
+
+template <bool FP8, typename TT>
+__global__ void __launch_bounds__(512)
 prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int n_mt) {
-    constexpr int NTHREADS = NW * 64;
-    constexpr int K_ITEMS = (NT * 8) / NTHREADS;                 // 512 K items per tile
-    constexpr int V_TOTAL = FP8 ? PAGES * D : PAGES * D * 2;     // ctx V items per tile
-    constexpr int V_ITEMS = (PAGES * D * 2) / NTHREADS;          // new-token tiles: 64 keys x 16 chunks
-    static_assert(K_ITEMS >= 1 && V_ITEMS >= 1, "tile too small for the workgroup");
+    constexpr int VI_CTX = FP8 ? VI / 2 : VI;        // an fp8 page row of 16 slots is one 16-byte item
+    constexpr uint32_t TSZ = sizeof(TT);
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int l32 = lane & 31, gh = lane >> 5;
+    const bool gatherer = wave >= NC;
 
-    // ---- which work item: consecutive m-tiles of one (request, kv-head, split) share an XCD ----
+    // ---- work item: the m-tiles of one (request, kv-head, split) land on the same XCD ----
     const int n_groups = p.batch * p.num_kv_heads * nsplit;
     int mt, kvgrp;
     {
@@ -357,43 +165,364 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     const int b = kvgrp / (nsplit * p.num_kv_heads);
     const int group = p.num_q_heads / p.num_kv_heads;
 
-    Ctx c;
-    c.p = &p; c.b = b; c.g = g;
-    c.qs = load_index(p.b_start_loc, b, p.index_bits);
-    c.q_len = load_index(p.b_start_loc, b + 1, p.index_bits) - c.qs;
-    c.ctx_len = load_index(p.b_seq_len, b, p.index_bits) - c.q_len;
-    if (c.q_len <= 0 || c.ctx_len < 0) return;
-    if (p.skip_decode && c.q_len == 1) return;                   // old_ops:109-110
-    const int n_chunks = (int)((c.q_len + UNIT - 1) / UNIT);
+    const int64_t qs = load_index(p.b_start_loc, b, p.index_bits);
+    const int q_len = (int)(load_index(p.b_start_loc, b + 1, p.index_bits) - qs);
+    const int ctx_len = (int)(load_index(p.b_seq_len, b, p.index_bits) - q_len);
+    if (q_len <= 0 || ctx_len < 0) return;
+    if (p.skip_decode && q_len == 1) return;                     // old_ops:109-110
+    const int n_chunks = (q_len + UNIT - 1) / UNIT;
     const int n_units = n_chunks * group;
-    if (mt * NW >= n_units) return;                              // block_mask, old_ops:322-328
+    if (mt * NC >= n_units) return;                              // block_mask, old_ops:322-328
     const bool lazy_b = p.is_lazy ? p.is_lazy[b] != 0 : true;
-    c.pos_mode = p.pos_mode;
-    c.vanilla = p.pos_mode == LAZYATTN_POS_BLOCK_UNIFORM && !lazy_b;   // ops:398
-    c.rot_new = p.rotate_new_k && !c.vanilla;
-    c.n_pages = (int)((c.ctx_len + BS - 1) / BS);
-    c.k_scale = FP8 ? *p.k_scale : 1.f;
-    c.v_scale = FP8 ? *p.v_scale : 1.f;
+    const int pos_mode = p.pos_mode;
+    const bool vanilla = pos_mode == LAZYATTN_POS_BLOCK_UNIFORM && !lazy_b;   // ops:398
+    const bool use_qmask = !vanilla && p.q_mask != nullptr;
+    const int n_pages = (ctx_len + BS - 1) / BS;
+    int t_end;                                                   // new-token keys [0, t_end) are visible here
     {
-        int last_unit = mt * NW + NW - 1;
+        int last_unit = mt * NC + NC - 1;
         if (last_unit > n_units - 1) last_unit = n_units - 1;
-        int64_t te = (int64_t)(last_unit / group + 1) * UNIT;
-        c.t_end = (int)(te < c.q_len ? te : c.q_len);
+        const int te = (last_unit / group + 1) * UNIT;
+        t_end = te < q_len ? te : q_len;
+    }
+    const int n_ctx_tiles = (n_pages + PAGES - 1) / PAGES;
+    const int n_new_tiles = (t_end + NT - 1) / NT;
+    const int n_tiles = n_ctx_tiles + n_new_tiles;
+    const int tile_begin = (int)((int64_t)n_tiles * split / nsplit);
+    const int tile_end = (int)((int64_t)n_tiles * (split + 1) / nsplit);
+
+    // ---- page metadata of a tile, fetched ahead of its use ----
+    // lane l holds the entries of page (l & 3) of the tile: physical block, q_offset, and
+    // the number of valid slots (pad mask and end of context folded together).
+    // Branch-free on purpose (a branch around a load makes the compiler drain every
+    // outstanding load at the join): pages past the context read entry n_pages-1 and get
+    // limit 0; an absent q_offset / q_mask array is replaced by the block table, masked to 0.
+    struct Meta { int bt[PAGES], qo[PAGES], lim[PAGES]; };
+    // Read through the scalar unit (constant address space): the values are wave-uniform,
+    // they land in SGPRs, and waiting for them never drains the vector loads in flight.
+    typedef const int32_t __attribute__((address_space(4))) *sptr_i32;
+    const bool use_qo = !vanilla && pos_mode != LAZYATTN_POS_NATURAL;
+    const sptr_i32 bt_row = (sptr_i32)(p.block_table + b * p.bt_stride[0]);
+    const sptr_i32 qo_row = use_qo ? (sptr_i32)(p.q_offset + b * p.qo_stride[0]) : bt_row;
+    const sptr_i32 qm_row = use_qmask ? (sptr_i32)(p.q_mask + b * p.qm_stride[0]) : bt_row;
+    const int64_t bt_s1 = p.bt_stride[1];
+    const int64_t qo_s1 = use_qo ? p.qo_stride[1] : p.bt_stride[1];
+    const int64_t qm_s1 = use_qmask ? p.qm_stride[1] : p.bt_stride[1];
+    const int qo_and = use_qo ? -1 : 0, qm_and = use_qmask ? -1 : 0;
+    auto load_meta = [&](int tile) -> Meta {
+        Meta m;
+#pragma unroll
+        for (int pg = 0; pg < PAGES; ++pg) {
+            const int j = tile * PAGES + pg;
+            int jc = j < n_pages ? j : n_pages - 1;
+            jc = jc < 0 ? 0 : jc;
+            m.bt[pg] = bt_row[jc * bt_s1];
+            m.qo[pg] = qo_row[jc * qo_s1] & qo_and;
+            const int qm = qm_row[jc * qm_s1] & qm_and;                              // old_ops:165-167
+            int lim = ctx_len - j * BS;
+            lim = lim < BS - qm ? lim : BS - qm;
+            lim = lim > BS ? BS : lim;
+            m.lim[pg] = lim < 0 ? 0 : lim;
+        }
+        return m;
+    };
+    auto sel4 = [](const int *a, int pg) { return pg < 2 ? (pg == 0 ? a[0] : a[1]) : (pg == 2 ? a[2] : a[3]); };
+    auto page_bt = [&](const Meta &m, int pg) { return sel4(m.bt, pg); };
+    auto page_qo = [&](const Meta &m, int pg) { return sel4(m.qo, pg); };
+    auto page_lim = [&](const Meta &m, int pg) { return sel4(m.lim, pg); };
+
+    // ---- descriptor of a tile: kind and which of its 64 keys exist ----
+    struct TileDesc { int kind; uint32_t vlo, vhi; };
+    auto describe = [&](int tile, const Meta &m) -> TileDesc {
+        TileDesc t{TILE_FULL, ~0u, ~0u};
+        if (tile >= n_ctx_tiles) {
+            t.kind = TILE_NEW;
+            const int n = t_end - (tile - n_ctx_tiles) * NT;
+            const uint64_t valid = n >= 64 ? ~0ull : (n <= 0 ? 0ull : ((1ull << n) - 1ull));
+            t.vlo = (uint32_t)valid; t.vhi = (uint32_t)(valid >> 32);
+        } else {
+            t.vlo = ((1u << page_lim(m, 0)) - 1u) | (((1u << page_lim(m, 1)) - 1u) << BS);
+            t.vhi = ((1u << page_lim(m, 2)) - 1u) | (((1u << page_lim(m, 3)) - 1u) << BS);
+            t.kind = (t.vlo & t.vhi) == ~0u ? TILE_FULL : TILE_EDGE;
+        }
+        return t;
+    };
+
+    if (gatherer) {
+        // ====================================================================== gather
+        const int lt = tid - NC * 64;
+        const bool rot_new = p.rotate_new_k && !vanilla;
+        const float k_scale = FP8 ? *p.k_scale : 1.f;
+        const float v_scale = FP8 ? *p.v_scale : 1.f;
+        const uint8_t *kc_base = (const uint8_t *)p.k_cache + (int64_t)g * p.kc_stride[1] * (FP8 ? 1 : 2);
+        const uint8_t *vc_base = (const uint8_t *)p.v_cache + (int64_t)g * p.vc_stride[1] * (FP8 ? 1 : 2);
+        const int64_t kc_page_bytes = p.kc_stride[0] * (FP8 ? 1 : 2);
+        const int64_t vc_page_bytes = p.vc_stride[0] * (FP8 ? 1 : 2);
+        const uint8_t *tab_base = (const uint8_t *)p.cos_sin_cache;
+        const uint32_t row_bytes = (uint32_t)p.table_stride * TSZ;
+        // per-token rotation of context pages reads the packed table [2][D/16][rows][8]: the 16
+        // slots of a page are 16 consecutive 16-byte chunks there
+        const bool packed_tab = p.cos_sin_packed != nullptr && !vanilla && pos_mode != LAZYATTN_POS_BLOCK_UNIFORM;
+        const uint8_t *ctab_base = packed_tab ? (const uint8_t *)p.cos_sin_packed : tab_base;
+        const uint32_t pos_bytes = packed_tab ? 8 * TSZ : row_bytes;       // bytes per unit of position
+        const uint32_t sin_delta = packed_tab ? (uint32_t)(HALF / 8) * (uint32_t)p.packed_rows * 8 * TSZ : HALF * TSZ;
+        uint32_t k_goff[KI], k_toff[KI];
+        int k_pg[KI];
+#pragma unroll
+        for (int i = 0; i < KI; ++i) {
+            const int idx = lt + i * LT;
+            const int o = idx & 15, cp = (idx >> 4) & 7;
+            k_pg[i] = uniform(idx >> 7);
+            // bf16: [D/8][16][8] -> item (cp, o) at (cp*16 + o)*16 bytes, pair chunk +2048
+            // fp8 : [D/16][16][16] -> 8 bytes at chunk cp/2, half cp&1, pair chunk +4*256
+            k_goff[i] = FP8 ? (uint32_t)((cp >> 1) * 256 + o * 16 + (cp & 1) * 8) : (uint32_t)((idx & 127) * 16);
+            // block-uniform rotation and un-rotated requests use one table row for the whole page
+            k_toff[i] = packed_tab ? ((uint32_t)cp * (uint32_t)p.packed_rows + (uint32_t)o) * 8 * TSZ
+                      : ((pos_mode == LAZYATTN_POS_BLOCK_UNIFORM || vanilla) ? 0u : (uint32_t)o * row_bytes) +
+                            (uint32_t)cp * 8 * TSZ;
+        }
+        uint32_t v_goff[VI_CTX];
+        int v_pg[VI_CTX];
+#pragma unroll
+        for (int i = 0; i < VI_CTX; ++i) {
+            const int idx = lt + i * LT;
+            // bf16: 256 items of 16 bytes per page (d = idx/2, slots 8*(idx&1) ..); fp8: 128 items (d = idx)
+            v_pg[i] = uniform(FP8 ? idx >> 7 : idx >> 8);
+            v_goff[i] = (uint32_t)((idx & (FP8 ? 127 : 255)) * 16);
+        }
+        KRegs<TT> kr[KI];
+        uint4 vr[VI];
+        int v_lim[VI_CTX];
+
+        // ---- loads of a full context tile: no branch, no zero fill ----
+        auto issue_loads_full = [&](int tile, const Meta &meta) {
+#pragma unroll
+            for (int i = 0; i < KI; ++i) {
+                const int j = tile * PAGES + k_pg[i];
+                const int idx = lt + i * LT;
+                kr[i].lds_off = (uint32_t)(k_pg[i] * K_PAGE + (idx & 127) * 16);
+                const uint8_t *kb = kc_base + page_bt(meta, k_pg[i]) * kc_page_bytes;
+                if (FP8) {
+                    const uint2 a = ldg8(kb, k_goff[i]), a2 = ldg8(kb, k_goff[i] + 4 * 256);
+                    kr[i].k1 = make_uint4(a.x, a.y, 0, 0);
+                    kr[i].k2 = make_uint4(a2.x, a2.y, 0, 0);
+                } else {
+                    kr[i].k1 = ldg16(kb, k_goff[i]);
+                    kr[i].k2 = ldg16(kb, k_goff[i] + 2048);
+                }
+                // un-rotated requests read row 0 of the table (cos 1, sin 0): exact identity
+                const int qo = page_qo(meta, k_pg[i]);
+                const int nat = j * BS;                                              // old_ops:183-184
+                int pos0 = pos_mode == LAZYATTN_POS_NATURAL ? nat
+                         : pos_mode == LAZYATTN_POS_OFFSET ? (qo ? qo - 1 : nat)      // old_ops:186-191
+                                                           : (qo ? qo - 1 : 0);       // ops:180-186
+                pos0 = vanilla ? 0 : pos0;
+                const uint8_t *tb = ctab_base + (int64_t)pos0 * pos_bytes;
+                kr[i].c.load(tb, k_toff[i]);
+                kr[i].s.load(tb, k_toff[i] + sin_delta);
+            }
+#pragma unroll
+            for (int i = 0; i < VI_CTX; ++i) {
+                v_lim[i] = BS;
+                vr[i] = ldg16(vc_base + page_bt(meta, v_pg[i]) * vc_page_bytes, v_goff[i]);
+            }
+        };
+        // ---- loads of any tile: edge context tiles and new-token tiles ----
+        auto issue_loads = [&](int tile, int kind, const Meta &meta) {
+            if (kind == TILE_FULL) {
+                issue_loads_full(tile, meta);
+            } else if (kind == TILE_EDGE) {
+                issue_loads_full(tile, meta);          // pages past the context re-read the last page: harmless
+#pragma unroll
+                for (int i = 0; i < VI_CTX; ++i) v_lim[i] = page_lim(meta, v_pg[i]);
+#pragma unroll
+                for (int i = 0; i < KI; ++i)
+                    if (tile * PAGES + k_pg[i] >= n_pages) { kr[i].k1 = make_uint4(0, 0, 0, 0); kr[i].k2 = kr[i].k1; }
+            } else {
+                const int m0 = (tile - n_ctx_tiles) * NT;
+#pragma unroll
+                for (int i = 0; i < KI; ++i) {
+                    const int idx = lt + i * LT;
+                    const int cp = idx & 7, kl = idx >> 3, m = m0 + kl;
+                    kr[i].lds_off = (uint32_t)((kl >> 4) * K_PAGE + cp * 256 + (kl & 15) * 16);
+                    kr[i].k1 = make_uint4(0, 0, 0, 0); kr[i].k2 = kr[i].k1;
+                    kr[i].c.fill(1.f); kr[i].s.fill(0.f);
+                    if (m < t_end) {
+                        const bf16_t *kn = (const bf16_t *)p.k + (qs + m) * p.k_stride[0] + (int64_t)g * p.k_stride[1] + cp * 8;
+                        kr[i].k1 = *reinterpret_cast<const uint4 *>(kn);
+                        kr[i].k2 = *reinterpret_cast<const uint4 *>(kn + HALF);
+                        if (rot_new) {                                               // old_ops:342-343
+                            const uint8_t *tb = tab_base + (int64_t)(ctx_len + m) * row_bytes;
+                            kr[i].c.load(tb, (uint32_t)cp * 8 * TSZ);
+                            kr[i].s.load(tb, (uint32_t)cp * 8 * TSZ + HALF * TSZ);
+                        }
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < VI; ++i) {
+                    const int idx = lt + i * LT;
+                    const int dc = idx & 15, m = m0 + (idx >> 4);
+                    vr[i] = make_uint4(0, 0, 0, 0);
+                    if (m < t_end)
+                        vr[i] = *reinterpret_cast<const uint4 *>((const bf16_t *)p.v + (qs + m) * p.v_stride[0] +
+                                                                 (int64_t)g * p.v_stride[1] + dc * 8);
+                }
+            }
+        };
+        // ---- rotate the K items in fp32 and write them to a K tile ----
+        auto store_k = [&](uint8_t *ktile, int kind) {
+#pragma unroll
+            for (int i = 0; i < KI; ++i) {
+                float a[8], bb[8], cs[8], sn[8];
+                if (FP8 && kind != TILE_NEW) {
+                    unpack8_fp8(kr[i].k1.x, kr[i].k1.y, k_scale, a);
+                    unpack8_fp8(kr[i].k2.x, kr[i].k2.y, k_scale, bb);
+                } else {
+                    unpack8(kr[i].k1, a);
+                    unpack8(kr[i].k2, bb);
+                }
+                kr[i].c.get(cs);
+                kr[i].s.get(sn);
+                float x[8], y[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    x[e] = a[e] * cs[e] - bb[e] * sn[e];                             // old_ops:253
+                    y[e] = a[e] * sn[e] + bb[e] * cs[e];                             // old_ops:254
+                }
+                *reinterpret_cast<uint4 *>(ktile + kr[i].lds_off) = make_uint4(
+                    pack_bf16(x[0], x[1]), pack_bf16(x[2], x[3]), pack_bf16(x[4], x[5]), pack_bf16(x[6], x[7]));
+                *reinterpret_cast<uint4 *>(ktile + kr[i].lds_off + 8 * 256) = make_uint4(
+                    pack_bf16(y[0], y[1]), pack_bf16(y[2], y[3]), pack_bf16(y[4], y[5]), pack_bf16(y[6], y[7]));
+            }
+        };
+        // ---- write the V items to a V tile ----
+        auto store_v = [&](uint8_t *vtile, int kind) {
+            if (kind == TILE_NEW) {
+                // item = 8 d of one new-token key: scatter 2-byte entries
+#pragma unroll
+                for (int i = 0; i < VI; ++i) {
+                    const int idx = lt + i * LT;
+                    const int dc = idx & 15, kl = idx >> 4, slot = kl & 15;
+                    uint8_t *dst = vtile + (kl >> 4) * V_PAGE + ((slot >> 2) & 1) * V_G + (dc * 8) * 16 + (slot >> 3) * 8 +
+                                   (slot & 3) * 2;
+                    const uint32_t w[4] = {vr[i].x, vr[i].y, vr[i].z, vr[i].w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        *reinterpret_cast<uint16_t *>(dst + (2 * e) * 16) = (uint16_t)(w[e] & 0xffffu);
+                        *reinterpret_cast<uint16_t *>(dst + (2 * e + 1) * 16) = (uint16_t)(w[e] >> 16);
+                    }
+                }
+                return;
+            }
+#pragma unroll
+            for (int i = 0; i < VI_CTX; ++i) {
+                const int idx = lt + i * LT;
+                const int lim = v_lim[i];
+                if (FP8) {
+                    // 16 fp8 slots of one d: entry g=0 <- slots 0-3 | 8-11, entry g=1 <- slots 4-7 | 12-15
+                    const int d = idx & 127;
+                    const uint32_t w[4] = {vr[i].x, vr[i].y, vr[i].z, vr[i].w};
+                    uint32_t o2[4][2];
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; ++q4) {
+                        const f32x2_t lo = __builtin_amdgcn_cvt_pk_f32_fp8(w[q4], false);
+                        const f32x2_t hi = __builtin_amdgcn_cvt_pk_f32_fp8(w[q4] >> 16, false);
+                        float f[4] = {lo[0] * v_scale, lo[1] * v_scale, hi[0] * v_scale, hi[1] * v_scale};
+                        if (kind == TILE_EDGE) {
+#pragma unroll
+                            for (int s = 0; s < 4; ++s)
+                                if (q4 * 4 + s >= lim) f[s] = 0.f;   // masked slots contribute nothing, whatever they hold
+                        }
+                        o2[q4][0] = pack_bf16(f[0], f[1]);
+                        o2[q4][1] = pack_bf16(f[2], f[3]);
+                    }
+                    uint8_t *dst = vtile + v_pg[i] * V_PAGE + d * 16;
+                    *reinterpret_cast<uint4 *>(dst) = make_uint4(o2[0][0], o2[0][1], o2[2][0], o2[2][1]);
+                    *reinterpret_cast<uint4 *>(dst + V_G) = make_uint4(o2[1][0], o2[1][1], o2[3][0], o2[3][1]);
+                } else {
+                    // 8 bf16 slots (8*hf ..) of one d: slots +0..3 -> entry g=0, +4..7 -> entry g=1, half hf
+                    const int d = (idx >> 1) & 127, hf = idx & 1;
+                    uint4 v = vr[i];
+                    if (kind == TILE_EDGE && lim < BS) {
+                        uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            if (hf * 8 + 2 * e >= lim) w[e] &= 0xffff0000u;
+                            if (hf * 8 + 2 * e + 1 >= lim) w[e] &= 0x0000ffffu;
+                        }
+                        v = make_uint4(w[0], w[1], w[2], w[3]);
+                    }
+                    uint8_t *dst = vtile + v_pg[i] * V_PAGE + d * 16 + hf * 8;
+                    *reinterpret_cast<uint2 *>(dst) = make_uint2(v.x, v.y);
+                    *reinterpret_cast<uint2 *>(dst + V_G) = make_uint2(v.z, v.w);
+                }
+            }
+        };
+
+        // At the top of iteration `tile` the raw K/V of tile+1 sit in registers (loaded during
+        // the previous iteration); they are rotated into the other LDS buffer while the
+        // computing waves work on `tile`, then the loads of tile+2 are issued.
+        int nxt_kind = TILE_FULL;
+        Meta meta_pend = load_meta(tile_begin + 2);
+        if (tile_begin < tile_end) {
+            const Meta m0 = load_meta(tile_begin);
+            const Meta m1 = load_meta(tile_begin + 1);
+            const int k0 = describe(tile_begin, m0).kind;
+            issue_loads(tile_begin, k0, m0);
+            store_k(lds, k0);
+            store_v(lds + 2 * K_TILE, k0);
+            if (tile_begin + 1 < tile_end) {
+                nxt_kind = describe(tile_begin + 1, m1).kind;
+                issue_loads(tile_begin + 1, nxt_kind, m1);
+            }
+        }
+        __syncthreads();
+        int tile = tile_begin;
+        while (tile < tile_end) {
+            // steady state: tile+1 (in registers) and tile+2 (to load) are plain context tiles
+            while (tile + 2 < tile_end && nxt_kind == TILE_FULL && describe(tile + 2, meta_pend).kind == TILE_FULL) {
+                const int cur = (tile - tile_begin) & 1;
+                const Meta meta_new = load_meta(tile + 3);      // scalar loads, land during the rotation
+                store_k(lds + (cur ^ 1) * K_TILE, TILE_FULL);
+                store_v(lds + 2 * K_TILE + (cur ^ 1) * V_TILE, TILE_FULL);
+                issue_loads_full(tile + 2, meta_pend);
+                meta_pend = meta_new;
+                ++tile;
+                __syncthreads();
+            }
+            if (tile >= tile_end) break;
+            const int cur = (tile - tile_begin) & 1;
+            if (tile + 1 < tile_end) {
+                store_k(lds + (cur ^ 1) * K_TILE, nxt_kind);
+                store_v(lds + 2 * K_TILE + (cur ^ 1) * V_TILE, nxt_kind);
+            }
+            int new_kind = TILE_FULL;
+            if (tile + 2 < tile_end) {
+                new_kind = describe(tile + 2, meta_pend).kind;
+                issue_loads(tile + 2, new_kind, meta_pend);
+            }
+            nxt_kind = new_kind;
+            meta_pend = load_meta(tile + 3);
+            ++tile;
+            __syncthreads();
+        }
+        return;
     }
 
-    // ---- this wave's rows ----
-    const int unit = mt * NW + wave;
+    // ========================================================================== compute
+    const int l32 = lane & 31, gh = lane >> 5;
+    const int unit = mt * NC + wave;
     const bool active = unit < n_units;
     const int chunk = active ? unit / group : 0;
     const int h = g * group + (active ? unit % group : 0);
     const int t0 = chunk * UNIT;
-    const int64_t row = t0 + l32;                                // token index of this lane's query row
-    const bool row_ok = active && row < c.q_len;
+    const int row = t0 + l32;                                    // token index of this lane's query row
+    const bool row_ok = active && row < q_len;
 
     // Q^T fragments: B operand of S^T = K.Q^T, lane = (row l32, d = ks*16 + gh*8 .. +8)
     bf16x8_t qf[8];
     {
-        const bf16_t *qp = (const bf16_t *)p.q + (c.qs + row) * p.q_stride[0] + (int64_t)h * p.q_stride[1] + gh * 8;
+        const bf16_t *qp = (const bf16_t *)p.q + (qs + row) * p.q_stride[0] + (int64_t)h * p.q_stride[1] + gh * 8;
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
             uint4 v = make_uint4(0, 0, 0, 0);
@@ -401,14 +530,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             qf[ks] = *reinterpret_cast<bf16x8_t *>(&v);
         }
     }
-
-    const int n_ctx_tiles = (c.n_pages + PAGES - 1) / PAGES;
-    const int n_new_tiles = (c.t_end + NT - 1) / NT;
-    const int n_tiles = n_ctx_tiles + n_new_tiles;
-    const int tile_begin = (int)((int64_t)n_tiles * split / nsplit);
-    const int tile_end = (int)((int64_t)n_tiles * (split + 1) / nsplit);
-
-    const float cs2 = p.sm_scale * 1.4426950408889634f;          // scores to log2 units
+    const float cs2 = p.sm_scale * 1.4426950408889634f;          // scores -> log2 units
     float m_run = -INFINITY, l_run = 0.f;
     f32x16_t acc[4];
 #pragma unroll
@@ -416,184 +538,146 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[dt][i] = 0.f;
 
-    KItem<TT> kit[K_ITEMS];
-    VItem vit[V_ITEMS];
-
-    if (tile_begin < tile_end) {
-        // ---- prologue: first tile into buffer 0 ----
+    // ---- S^T = K . Q^T for one 64-key tile: two independent 32-key accumulation chains ----
+    // The LDS reads of the A fragments run six ahead of the MFMAs that consume them, so the
+    // matrix pipe does not wait for an LDS round trip between instructions.
+    auto qk_tile = [&](const uint8_t *ktile, f32x16_t &s0, f32x16_t &s1) {
 #pragma unroll
-        for (int i = 0; i < K_ITEMS; ++i) load_k_item<FP8, TT>(c, kit[i], tile_begin, n_ctx_tiles, tid + i * NTHREADS);
-        {
-            const bool ctx_t = tile_begin < n_ctx_tiles;
+        for (int i = 0; i < 16; ++i) { s0[i] = 0.f; s1[i] = 0.f; }
+        const uint8_t *kp = ktile + (l32 >> 4) * K_PAGE + gh * 256 + (l32 & 15) * 16;
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int i = 0; i < V_ITEMS; ++i) {
-                const int idx = tid + i * NTHREADS;
-                if (!ctx_t || idx < V_TOTAL) load_v_item<FP8>(c, vit[i], tile_begin, n_ctx_tiles, idx);
-                else vit[i] = VItem{make_uint4(0, 0, 0, 0), 0, 0, 0, -1};
-            }
+        for (int ks = 0; ks < 8; ++ks) {
+            const bf16x8_t a0 = *reinterpret_cast<const bf16x8_t *>(kp + ks * 512);
+            const bf16x8_t a1 = *reinterpret_cast<const bf16x8_t *>(kp + 2 * K_PAGE + ks * 512);
+            s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, qf[ks], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, qf[ks], s1, 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);            // 6 DS reads up front
+#pragma unroll
+        for (int i = 0; i < 10; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);        // 1 MFMA
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);        // 1 DS read
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 6, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // ---- masks: register i of half `sub` holds key sub*32 + 8*(i/4) + 4*gh + i%4 ----
+    auto mask_half = [&](f32x16_t &s, uint32_t vbits, int sub, int kind, int m0) {
+        const uint32_t w = vbits >> (4 * gh);
+        // causal: key m0 + kk <= row  <=>  8*(i/4) + i%4 <= row - m0 - sub*32 - 4*gh   (old_ops:371-372)
+        const int lim = kind == TILE_NEW ? row - m0 - sub * 32 - 4 * gh : 64;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int kb = 8 * (i >> 2) + (i & 3);
+            const bool ok = ((w >> kb) & 1u) && kb <= lim;
+            s[i] = ok ? s[i] : -INFINITY;
+        }
+    };
+    // ---- running max over the tile, rescale of the accumulators when it grew (old_ops:287-291) ----
+    auto update_max = [&](const f32x16_t &s0, const f32x16_t &s1) -> float {
+        float mx = fmaxf(fmaxf(s0[0], s0[1]), fmaxf(s1[0], s1[1]));
+#pragma unroll
+        for (int i = 2; i < 16; i += 2) mx = fmaxf(mx, fmaxf(fmaxf(s0[i], s0[i + 1]), fmaxf(s1[i], s1[i + 1])));
+        mx = fmaxf(mx, partner32(mx, gh != 0));
+        const float m_new = fmaxf(m_run, mx);
+        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f((m_run - m_safe) * cs2);          // m_run = -inf -> 0
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt) acc[dt] *= alpha;
+            l_run *= alpha;
+        }
+        m_run = m_new;
+        return m_safe * cs2;
+    };
+    // ---- P = exp2(S*cs2 - mc) for 32 keys, packed as the two B operands of the PV steps ----
+    auto exp_half = [&](const f32x16_t &s, float mc, bf16x8_t &p0, bf16x8_t &p1) {
+        float pr[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) pr[i] = __builtin_amdgcn_exp2f(fmaf(s[i], cs2, -mc));
+        float la = 0.f, lb = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) { la += pr[i]; lb += pr[i + 1]; }
+        l_run += la + lb;                                                            // old_ops:312
+        uint4 w0 = make_uint4(pack_bf16(pr[0], pr[1]), pack_bf16(pr[2], pr[3]), pack_bf16(pr[4], pr[5]), pack_bf16(pr[6], pr[7]));
+        uint4 w1 = make_uint4(pack_bf16(pr[8], pr[9]), pack_bf16(pr[10], pr[11]), pack_bf16(pr[12], pr[13]), pack_bf16(pr[14], pr[15]));
+        p0 = *reinterpret_cast<bf16x8_t *>(&w0);
+        p1 = *reinterpret_cast<bf16x8_t *>(&w1);
+    };
+    // ---- O^T += V^T . P^T for 32 keys (pages 2*sub, 2*sub+1 of the tile) ----
+    // k index j of a 16-key step <-> slot 4*gh + j (j < 4), 8 + 4*gh + j - 4 (j >= 4)
+    auto pv_half = [&](const uint8_t *vtile, int sub, const bf16x8_t &p0, const bf16x8_t &p1) {
+        const uint8_t *vp = vtile + (sub * 2) * V_PAGE + gh * V_G + l32 * 16;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) {
+            const bf16x8_t a = *reinterpret_cast<const bf16x8_t *>(vp + dt * 512);
+            acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, p0, acc[dt], 0, 0, 0);
         }
 #pragma unroll
-        for (int i = 0; i < K_ITEMS; ++i) rotate_store_k<TT>(kit[i], lds, c.k_scale);
-#pragma unroll
-        for (int i = 0; i < V_ITEMS; ++i)
-            if (vit[i].kind >= 0) store_v_item(vit[i], lds + 2 * K_TILE, c.v_scale);
-    }
-    __syncthreads();
+        for (int dt = 0; dt < 4; ++dt) {
+            const bf16x8_t a = *reinterpret_cast<const bf16x8_t *>(vp + V_PAGE + dt * 512);
+            acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, p1, acc[dt], 0, 0, 0);
+        }
+    };
+    auto attend = [&](const uint8_t *vtile, const f32x16_t &s0, const f32x16_t &s1) {
+        const float mc = update_max(s0, s1);
+        bf16x8_t p0, p1, p2, p3;
+        exp_half(s0, mc, p0, p1);
+        pv_half(vtile, 0, p0, p1);
+        exp_half(s1, mc, p2, p3);
+        pv_half(vtile, 1, p2, p3);
+    };
 
+    Meta m_cur = load_meta(tile_begin), m_nxt = load_meta(tile_begin + 1);
+    __syncthreads();
     for (int tile = tile_begin; tile < tile_end; ++tile) {
         const int cur = (tile - tile_begin) & 1;
         const uint8_t *ktile = lds + cur * K_TILE;
         const uint8_t *vtile = lds + 2 * K_TILE + cur * V_TILE;
-        uint8_t *ktile_n = lds + (cur ^ 1) * K_TILE;
-        uint8_t *vtile_n = lds + 2 * K_TILE + (cur ^ 1) * V_TILE;
-        const bool has_next = tile + 1 < tile_end;
-        const bool is_ctx = tile < n_ctx_tiles;
-        const bool next_ctx = tile + 1 < n_ctx_tiles;
-
-        if (has_next) {
-#pragma unroll
-            for (int i = 0; i < K_ITEMS; ++i) load_k_item<FP8, TT>(c, kit[i], tile + 1, n_ctx_tiles, tid + i * NTHREADS);
-#pragma unroll
-            for (int i = 0; i < V_ITEMS; ++i) {
-                const int idx = tid + i * NTHREADS;
-                if (!next_ctx || idx < V_TOTAL) load_v_item<FP8>(c, vit[i], tile + 1, n_ctx_tiles, idx);
-                else vit[i] = VItem{make_uint4(0, 0, 0, 0), 0, 0, 0, -1};
-            }
-        }
-
-        // keys of this tile that exist: bit kk of `valid`
-        uint64_t valid;
-        int m0 = 0;
-        if (is_ctx) {
-            valid = 0;
-#pragma unroll
-            for (int pg = 0; pg < PAGES; ++pg) {
-                const int lim = page_limit(c, tile * PAGES + pg);
-                valid |= (uint64_t)((1u << lim) - 1u) << (pg * BS);
-            }
+        const TileDesc td = describe(tile, m_cur);
+        const Meta m_new = load_meta(tile + 2);
+        if (td.kind == TILE_FULL) {
+            // rows of an idle wave are all-zero queries: harmless, never stored
+            f32x16_t s0, s1;
+            qk_tile(ktile, s0, s1);
+            attend(vtile, s0, s1);
         } else {
-            m0 = (tile - n_ctx_tiles) * NT;
-            const int n = c.t_end - m0;
-            valid = n >= 64 ? ~0ull : ((1ull << n) - 1ull);
+            const int m0 = td.kind == TILE_NEW ? (tile - n_ctx_tiles) * NT : 0;
+            // a new-token tile entirely in this wave's future contributes nothing (causal)
+            if (active && (td.kind != TILE_NEW || m0 <= t0 + UNIT - 1)) {
+                f32x16_t s0, s1;
+                qk_tile(ktile, s0, s1);
+                mask_half(s0, td.vlo, 0, td.kind, m0);
+                mask_half(s1, td.vhi, 1, td.kind, m0);
+                attend(vtile, s0, s1);
+            }
         }
-        // a new-token tile entirely in this wave's future contributes nothing (causal)
-        const bool compute = active && (is_ctx || m0 <= t0 + UNIT - 1);
-
-        if (compute) {
-            // ---- S^T = K . Q^T ----
-            f32x16_t s[2];
-#pragma unroll
-            for (int sub = 0; sub < 2; ++sub) {
-#pragma unroll
-                for (int i = 0; i < 16; ++i) s[sub][i] = 0.f;
-                const uint8_t *kp = ktile + (sub * 2 + (l32 >> 4)) * K_PAGE + gh * 256 + (l32 & 15) * 16;
-#pragma unroll
-                for (int ks = 0; ks < 8; ++ks) {
-                    const bf16x8_t a = *reinterpret_cast<const bf16x8_t *>(kp + ks * 512);
-                    s[sub] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[ks], s[sub], 0, 0, 0);
-                }
-            }
-            // ---- masks: register i of sub-tile `sub` holds key sub*32 + 8*(i/4) + 4*gh + i%4 ----
-            const bool need_mask = (valid != ~0ull) || (!is_ctx && m0 + NT - 1 > t0);
-            if (need_mask) {
-#pragma unroll
-                for (int sub = 0; sub < 2; ++sub)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const int kk = sub * 32 + 8 * (i >> 2) + 4 * gh + (i & 3);
-                        bool ok = (valid >> kk) & 1ull;
-                        if (!is_ctx) ok = ok && (m0 + kk <= row);                     // old_ops:371-372
-                        if (!ok) s[sub][i] = -INFINITY;
-                    }
-            }
-            // ---- online softmax (old_ops:287-291,312-313) ----
-            float mx = s[0][0];
-#pragma unroll
-            for (int sub = 0; sub < 2; ++sub)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[sub][i]);
-            mx = fmaxf(mx, partner32(mx));
-            const float m_new = fmaxf(m_run, mx);
-            const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-            const float alpha = __builtin_amdgcn_exp2f((m_run - m_safe) * cs2);      // -inf -> 0
-            if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
-#pragma unroll
-                for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) acc[dt][i] *= alpha;
-                l_run *= alpha;
-            }
-            m_run = m_new;
-            const float mc = m_safe * cs2;
-            float lsum = 0.f;
-            bf16x8_t pf[4];
-#pragma unroll
-            for (int sub = 0; sub < 2; ++sub) {
-                float pr[16];
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    pr[i] = __builtin_amdgcn_exp2f(fmaf(s[sub][i], cs2, -mc));
-                    lsum += pr[i];
-                }
-#pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    uint4 w = make_uint4(pack_bf16(pr[8 * t + 0], pr[8 * t + 1]), pack_bf16(pr[8 * t + 2], pr[8 * t + 3]),
-                                         pack_bf16(pr[8 * t + 4], pr[8 * t + 5]), pack_bf16(pr[8 * t + 6], pr[8 * t + 7]));
-                    pf[sub * 2 + t] = *reinterpret_cast<bf16x8_t *>(&w);
-                }
-            }
-            l_run += lsum;
-
-            if (has_next) {
-#pragma unroll
-                for (int i = 0; i < K_ITEMS; ++i) rotate_store_k<TT>(kit[i], ktile_n, c.k_scale);
-            }
-
-            // ---- O^T += V^T . P^T ; k index j of step kt <-> slots 4*gh + j (j<4), 8 + 4*gh + j-4 ----
-#pragma unroll
-            for (int kt = 0; kt < 4; ++kt) {
-                const uint8_t *vp = vtile + kt * V_PAGE + gh * V_SG + l32 * 8;
-#pragma unroll
-                for (int dt = 0; dt < 4; ++dt) {
-                    const uint2 lo = *reinterpret_cast<const uint2 *>(vp + dt * 256);
-                    const uint2 hi = *reinterpret_cast<const uint2 *>(vp + dt * 256 + 2 * V_SG);
-                    uint4 w = make_uint4(lo.x, lo.y, hi.x, hi.y);
-                    const bf16x8_t a = *reinterpret_cast<bf16x8_t *>(&w);
-                    acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pf[kt], acc[dt], 0, 0, 0);
-                }
-            }
-        } else if (has_next) {
-#pragma unroll
-            for (int i = 0; i < K_ITEMS; ++i) rotate_store_k<TT>(kit[i], ktile_n, c.k_scale);
-        }
-        if (has_next) {
-#pragma unroll
-            for (int i = 0; i < V_ITEMS; ++i)
-                if (vit[i].kind >= 0) store_v_item(vit[i], vtile_n, c.v_scale);
-        }
+        m_cur = m_nxt;
+        m_nxt = m_new;
         __syncthreads();
     }
 
     // ---- epilogue ----
-    l_run += partner32(l_run);
+    l_run += partner32(l_run, gh != 0);
     if (!row_ok) return;
     const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
     if (nsplit == 1) {
-        bf16_t *op = (bf16_t *)p.o + (c.qs + row) * p.o_stride[0] + (int64_t)h * p.o_stride[1];
+        bf16_t *op = (bf16_t *)p.o + (qs + row) * p.o_stride[0] + (int64_t)h * p.o_stride[1];
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) {
                 const int d = dt * 32 + 8 * i4 + 4 * gh;
-                uint2 w = make_uint2(pack_bf16(acc[dt][4 * i4] * inv, acc[dt][4 * i4 + 1] * inv),
-                                     pack_bf16(acc[dt][4 * i4 + 2] * inv, acc[dt][4 * i4 + 3] * inv));
-                *reinterpret_cast<uint2 *>(op + d) = w;
+                *reinterpret_cast<uint2 *>(op + d) =
+                    make_uint2(pack_bf16(acc[dt][4 * i4] * inv, acc[dt][4 * i4 + 1] * inv),
+                               pack_bf16(acc[dt][4 * i4 + 2] * inv, acc[dt][4 * i4 + 3] * inv));
             }
     } else {
         const int64_t T = p.num_tokens;
         float *wo = (float *)p.workspace;
         float *wl = wo + (int64_t)nsplit * T * p.num_q_heads * D;
-        const int64_t r_idx = ((int64_t)split * T + (c.qs + row)) * p.num_q_heads + h;
+        const int64_t r_idx = ((int64_t)split * T + (qs + row)) * p.num_q_heads + h;
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
@@ -641,17 +725,12 @@ prefill_combine_kernel(const lazyattn_prefill_params p, const int nsplit) {
 }
 
 // ------------------------------------------------------------------ host side
+static int mfma_waves(const lazyattn_prefill_params &) { return NC; }   // units per workgroup
+
 static int mfma_mtiles(const lazyattn_prefill_params &p, int nw) {
     const int group = p.num_q_heads / p.num_kv_heads;
     const int units = ((p.max_q_len + UNIT - 1) / UNIT) * group;
     return (units + nw - 1) / nw;
-}
-
-static int mfma_waves(const lazyattn_prefill_params &p) {
-    if (p.cache_dtype == LAZYATTN_FP8_E4M3 && p.table_dtype == LAZYATTN_F32) return 8;
-    const int group = p.num_q_heads / p.num_kv_heads;
-    const int units = ((p.max_q_len + UNIT - 1) / UNIT) * group;
-    return units >= 8 ? 8 : 4;
 }
 
 static int mfma_splits(const lazyattn_prefill_params &p, int nw) {
@@ -678,7 +757,7 @@ bool mfma_supports(const lazyattn_prefill_params &p) {
                           p.o_stride[0], p.o_stride[1], p.kc_stride[0], p.kc_stride[1], p.vc_stride[0], p.vc_stride[1],
                           p.table_stride};
     for (int64_t s : al)
-        if (s % 8) return false;
+        if (s % 16) return false;
     const void *ptrs[] = {p.q, p.k, p.v, p.o, p.k_cache, p.v_cache, p.cos_sin_cache};
     for (const void *q : ptrs)
         if (((uintptr_t)q) & 15) return false;
@@ -693,9 +772,9 @@ size_t mfma_workspace_bytes(const lazyattn_prefill_params &p) {
     return (size_t)ns * (size_t)p.num_tokens * p.num_q_heads * (D + 1) * sizeof(float);
 }
 
-template <int NW, bool FP8, typename TT>
+template <bool FP8, typename TT>
 static int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt, hipStream_t stream) {
-    auto kern = prefill_mfma_kernel<NW, FP8, TT>;
+    auto kern = prefill_mfma_kernel<FP8, TT>;
     static bool attr_set = false;
     if (!attr_set) {
         if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
@@ -703,24 +782,17 @@ static int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt,
         attr_set = true;
     }
     const unsigned nblocks = (unsigned)(p.batch * p.num_kv_heads * nsplit * n_mt);
-    hipLaunchKernelGGL(kern, dim3(nblocks), dim3(NW * 64), LDS_BYTES, stream, p, nsplit, n_mt);
+    hipLaunchKernelGGL(kern, dim3(nblocks), dim3(512), LDS_BYTES, stream, p, nsplit, n_mt);
     return hipGetLastError() == hipSuccess ? LAZYATTN_OK : LAZYATTN_E_LAUNCH;
 }
 
-template <int NW>
-static int launch_mfma_nw(const lazyattn_prefill_params &p, int nsplit, int n_mt, hipStream_t stream) {
+static int launch_mfma_any(const lazyattn_prefill_params &p, int nsplit, int n_mt, hipStream_t stream) {
     const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3;
     const bool t32 = p.table_dtype == LAZYATTN_F32;
-    if (fp8) {
-        // <4 waves, fp8 cache, f32 table> is not instantiated (it crashes this compiler);
-        // launch_prefill_mfma() routes that combination to the 8-wave kernel.
-        if constexpr (NW == 8) {
-            if (t32) return launch_mfma_t<8, true, float>(p, nsplit, n_mt, stream);
-        }
-        return launch_mfma_t<NW, true, bf16_t>(p, nsplit, n_mt, stream);
-    }
-    return t32 ? launch_mfma_t<NW, false, float>(p, nsplit, n_mt, stream)
-               : launch_mfma_t<NW, false, bf16_t>(p, nsplit, n_mt, stream);
+    if (fp8) return t32 ? launch_mfma_t<true, float>(p, nsplit, n_mt, stream)
+                        : launch_mfma_t<true, bf16_t>(p, nsplit, n_mt, stream);
+    return t32 ? launch_mfma_t<false, float>(p, nsplit, n_mt, stream)
+               : launch_mfma_t<false, bf16_t>(p, nsplit, n_mt, stream);
 }
 
 int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
@@ -734,7 +806,7 @@ int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
         if (((uintptr_t)p.workspace) & 15) return LAZYATTN_E_WORKSPACE;
     }
     if (phases & LAZYATTN_PHASE_MAIN) {
-        const int rc = nw == 8 ? launch_mfma_nw<8>(p, nsplit, n_mt, stream) : launch_mfma_nw<4>(p, nsplit, n_mt, stream);
+        const int rc = launch_mfma_any(p, nsplit, n_mt, stream);
         if (rc != LAZYATTN_OK) return rc;
     }
     if (nsplit > 1 && (phases & LAZYATTN_PHASE_COMBINE)) {

@@ -58,4 +58,39 @@ int launch_cos_sin_table(void *out, int out_dtype, int64_t row_stride, int max_p
     return hipGetLastError() == hipSuccess ? LAZYATTN_OK : LAZYATTN_E_LAUNCH;
 }
 
+// packed[h][c][p][e] = table[p, h*R/2 + c*8 + e]: one thread moves one 8-element chunk
+template <typename T>
+__global__ void __launch_bounds__(256)
+pack_cos_sin_kernel(const T *table, T *packed, int64_t row_stride, int rows, int rotary_dim) {
+    const int chunks = rotary_dim / 8;               // per row: R/16 cos chunks then R/16 sin chunks
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)rows * chunks) return;
+    const int hc = (int)(idx % chunks);              // h * (R/16) + c
+    const int64_t pos = idx / chunks;
+    const T *src = table + pos * row_stride + hc * 8;
+    T *dst = packed + ((int64_t)hc * rows + pos) * 8;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) dst[e] = src[e];
+}
+
+int launch_pack_cos_sin(const void *table, void *packed, int dtype, int64_t row_stride, int rows,
+                        int rotary_dim, hipStream_t stream) {
+    const int64_t n = (int64_t)rows * (rotary_dim / 8);
+    if (n <= 0) return LAZYATTN_OK;
+    dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    switch (dtype) {
+        case LAZYATTN_F32:
+            hipLaunchKernelGGL(pack_cos_sin_kernel<float>, grid, block, 0, stream, (const float *)table,
+                               (float *)packed, row_stride, rows, rotary_dim);
+            break;
+        case LAZYATTN_BF16:
+        case LAZYATTN_F16:
+            hipLaunchKernelGGL(pack_cos_sin_kernel<uint16_t>, grid, block, 0, stream, (const uint16_t *)table,
+                               (uint16_t *)packed, row_stride, rows, rotary_dim);
+            break;
+        default: return LAZYATTN_E_DTYPE;
+    }
+    return hipGetLastError() == hipSuccess ? LAZYATTN_OK : LAZYATTN_E_LAUNCH;
+}
+
 }  // namespace lazyattn

@@ -22,6 +22,7 @@ PHASE_MAIN, PHASE_COMBINE, PHASE_ALL = 1, 2, 3
 ERRORS = {-1: "NULL", -2: "SHAPE", -3: "DTYPE", -4: "UNSUPPORTED", -5: "WORKSPACE", -6: "LAUNCH"}
 EXPORTS = ("lazyattn_prefill_workspace_bytes", "lazyattn_prefix_prefill",
            "lazyattn_paged_decode_rotary", "lazyattn_build_cos_sin_cache",
+           "lazyattn_pack_cos_sin_cache",
            "lazyattn_error_string", "lazyattn_abi_version")
 
 _DTYPE = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
@@ -31,7 +32,7 @@ class PrefillParams(C.Structure):
     _fields_ = (
         [(n, C.c_void_p) for n in ("q", "k", "v", "o", "k_cache", "v_cache", "block_table",
                                    "q_offset", "q_mask", "is_lazy", "b_start_loc", "b_seq_len",
-                                   "cos_sin_cache", "k_scale", "v_scale", "workspace")]
+                                   "cos_sin_cache", "cos_sin_packed", "k_scale", "v_scale", "workspace")]
         + [("workspace_bytes", C.c_int64),
            ("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3),
            ("v_stride", C.c_int64 * 3), ("o_stride", C.c_int64 * 3),
@@ -44,7 +45,7 @@ class PrefillParams(C.Structure):
                                     "rotate_new_k", "skip_decode", "fp32_rotary", "kernel",
                                     "num_splits", "phases")]
         + [("sm_scale", C.c_float), ("num_tokens", C.c_int32), ("max_seq_len", C.c_int32),
-           ("reserved", C.c_int32)])
+           ("packed_rows", C.c_int32)])
 
 
 def lib() -> C.CDLL:
@@ -66,6 +67,9 @@ def lib() -> C.CDLL:
         L.lazyattn_build_cos_sin_cache.argtypes = [
             C.c_void_p, C.c_int32, C.c_int64, C.c_int32, C.c_int32, C.c_double, C.c_int32,
             C.c_double, C.c_double, C.c_double, C.c_int32, C.c_void_p]
+        L.lazyattn_pack_cos_sin_cache.restype = C.c_int
+        L.lazyattn_pack_cos_sin_cache.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int32,
+                                                  C.c_int32, C.c_void_p]
         L.lazyattn_error_string.restype = C.c_char_p
         L.lazyattn_error_string.argtypes = [C.c_int]
         L.lazyattn_abi_version.restype = C.c_int
@@ -103,6 +107,29 @@ def workspace(device: torch.device, nbytes: int) -> Optional[torch.Tensor]:
     return buf
 
 
+_packed_tables: dict = {}
+
+
+def packed_cos_sin(table: torch.Tensor) -> Optional[torch.Tensor]:
+    """The table in the gather-friendly layout, built once per table (and again if the
+    caller writes to it) by the library's pack kernel."""
+    if table.dim() != 2 or table.shape[1] % 16 or table.stride(1) != 1:
+        return None
+    key = (table.data_ptr(), tuple(table.shape), table.stride(0), table.dtype, table.device)
+    hit = _packed_tables.get(key)
+    if hit is not None and hit[0] == table._version:
+        return hit[1]
+    if len(_packed_tables) > 16:
+        _packed_tables.clear()
+    packed = torch.empty(table.shape[0] * table.shape[1], dtype=table.dtype, device=table.device)
+    rc = lib().lazyattn_pack_cos_sin_cache(table.data_ptr(), packed.data_ptr(), dtype_code(table.dtype),
+                                           table.stride(0), table.shape[0], table.shape[1],
+                                           torch.cuda.current_stream(table.device).cuda_stream)
+    check(rc, "lazyattn_pack_cos_sin_cache")
+    _packed_tables[key] = (table._version, packed)
+    return packed
+
+
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return None if t is None else t.data_ptr()
 
@@ -112,13 +139,16 @@ def fill_params(*, q, k, v, o, k_cache, v_cache, block_table, b_start_loc, b_seq
                 max_q_len: int, rotary_dim: int, sliding_window: int, sm_scale: float,
                 pos_mode: int, rotate_new_k: bool, skip_decode: bool, fp32_rotary: bool = False,
                 kernel: int = KERNEL_AUTO, num_splits: int = 0, phases: int = PHASE_ALL,
-                max_seq_len: int = 0) -> PrefillParams:
+                max_seq_len: int = 0, packed_table=None) -> PrefillParams:
     p = PrefillParams()
     p.q, p.k, p.v, p.o = _ptr(q), _ptr(k), _ptr(v), _ptr(o)
     p.k_cache, p.v_cache = _ptr(k_cache), _ptr(v_cache)
     p.block_table, p.q_offset, p.q_mask, p.is_lazy = _ptr(block_table), _ptr(q_offset), _ptr(q_mask), _ptr(is_lazy)
     p.b_start_loc, p.b_seq_len = _ptr(b_start_loc), _ptr(b_seq_len)
     p.cos_sin_cache, p.k_scale, p.v_scale = _ptr(cos_sin_cache), _ptr(k_scale), _ptr(v_scale)
+    if packed_table is not None:
+        p.cos_sin_packed = packed_table.data_ptr()
+        p.packed_rows = cos_sin_cache.shape[0]
     p.q_stride[:] = q.stride()
     p.k_stride[:] = k.stride() if k is not None else (0, 0, 0)
     p.v_stride[:] = v.stride() if v is not None else (0, 0, 0)

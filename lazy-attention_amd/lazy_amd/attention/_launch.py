@@ -49,7 +49,7 @@ def launch_prefill(*, q, k, v, o, kv_cache_dtype, k_cache, v_cache, b_loc, b_sta
                    skip_decode, cos_sin_cache, rotary_dim, is_neox_style, is_lazy, q_offset, q_mask,
                    pos_mode: int, rotate_new_k: bool, fp32_rotary: bool = False,
                    kernel: int = _ffi.KERNEL_AUTO, num_splits: int = 0,
-                   phases: int = _ffi.PHASE_ALL, decode: bool = False) -> None:
+                   phases: int = _ffi.PHASE_ALL, decode: bool = False, _return_plan: bool = False):
     lib = _ffi.lib()
     cache_code = _cache_code(kv_cache_dtype, k_cache, v_cache, q.dtype)
     if not decode:
@@ -86,21 +86,45 @@ def launch_prefill(*, q, k, v, o, kv_cache_dtype, k_cache, v_cache, b_loc, b_sta
             v_scale.device != dev or v_scale.dtype != torch.float32) else v_scale
     else:
         k_scale = v_scale = None
+    b_loc, q_offset, q_mask = _i32(b_loc), _i32(q_offset), _i32(q_mask)
+    packed = None
+    if not decode and q.dtype == torch.bfloat16 and pos_mode != _ffi.POS_BLOCK_UNIFORM:
+        packed = _ffi.packed_cos_sin(cos_sin_cache)      # built once per table
     p = _ffi.fill_params(
-        q=q, k=k, v=v, o=o, k_cache=k_cache, v_cache=v_cache, block_table=_i32(b_loc),
+        q=q, k=k, v=v, o=o, k_cache=k_cache, v_cache=v_cache, block_table=b_loc,
         b_start_loc=b_start_loc, b_seq_len=b_seq_len, cos_sin_cache=cos_sin_cache,
-        k_scale=k_scale, v_scale=v_scale, q_offset=_i32(q_offset), q_mask=_i32(q_mask),
+        k_scale=k_scale, v_scale=v_scale, q_offset=q_offset, q_mask=q_mask,
         is_lazy=is_lazy, cache_code=cache_code, max_q_len=max_input_len, rotary_dim=rotary_dim,
         sliding_window=sliding_window, sm_scale=sm_scale, pos_mode=pos_mode,
         rotate_new_k=rotate_new_k, skip_decode=skip_decode, fp32_rotary=fp32_rotary,
-        kernel=kernel, num_splits=num_splits, phases=phases, max_seq_len=max_seq_len)
-    stream = torch.cuda.current_stream(dev).cuda_stream
-    if decode:
-        _ffi.check(lib.lazyattn_paged_decode_rotary(p, stream), "lazyattn_paged_decode_rotary")
-        return
-    nbytes = lib.lazyattn_prefill_workspace_bytes(p)
-    ws = _ffi.workspace(dev, nbytes)
-    if ws is not None:
-        p.workspace = ws.data_ptr()
-        p.workspace_bytes = ws.numel()
-    _ffi.check(lib.lazyattn_prefix_prefill(p, stream), "lazyattn_prefix_prefill")
+        kernel=kernel, num_splits=num_splits, phases=phases, max_seq_len=max_seq_len, packed_table=packed)
+    plan = PrefillPlan(p, dev, decode, keep=(q, k, v, o, k_cache, v_cache, b_loc, b_start_loc, b_seq_len,
+                                            cos_sin_cache, q_offset, q_mask, is_lazy, k_scale, v_scale, packed))
+    if _return_plan:
+        return plan
+    plan.run()
+
+
+class PrefillPlan:
+    """A validated call: the filled C struct plus references that keep its tensors alive.
+    ``run()`` enqueues it on torch's current stream; calling it again repeats the call
+    on the same operands (a serving loop re-uses the plan while shapes stay fixed)."""
+
+    def __init__(self, params, device, decode, keep):
+        self.params, self.device, self.decode, self._keep = params, device, decode, keep
+        self._lib = _ffi.lib()
+        self._ws = None
+        if not decode:
+            nbytes = self._lib.lazyattn_prefill_workspace_bytes(params)
+            self._ws = _ffi.workspace(device, nbytes)
+            if self._ws is not None:
+                params.workspace = self._ws.data_ptr()
+                params.workspace_bytes = self._ws.numel()
+
+    def run(self) -> None:
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        if self.decode:
+            _ffi.check(self._lib.lazyattn_paged_decode_rotary(self.params, stream),
+                       "lazyattn_paged_decode_rotary")
+        else:
+            _ffi.check(self._lib.lazyattn_prefix_prefill(self.params, stream), "lazyattn_prefix_prefill")

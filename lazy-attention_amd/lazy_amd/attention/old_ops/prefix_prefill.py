@@ -21,10 +21,10 @@ def context_attention_fwd(q, k, v, o, kv_cache_dtype: str, k_cache, v_cache, b_l
                           sm_scale=None, skip_decode=False, cos_sin_cache=None, rotary_dim=None,
                           is_neox_style=True, q_mask=None, q_offset=None, is_mepic: bool = True,
                           force_fp32_rotary: bool = False, *, _kernel: int = _ffi.KERNEL_AUTO,
-                          _num_splits: int = 0, _phases: int = _ffi.PHASE_ALL):
+                          _num_splits: int = 0, _phases: int = _ffi.PHASE_ALL, _return_plan: bool = False):
     if not is_mepic and q_offset is None:
         raise ValueError("q_offset is required when is_mepic is False")
-    _launch.launch_prefill(
+    plan = _launch.launch_prefill(
         q=q, k=k, v=v, o=o, kv_cache_dtype=kv_cache_dtype, k_cache=k_cache, v_cache=v_cache,
         b_loc=b_loc, b_start_loc=b_start_loc, b_seq_len=b_seq_len, max_input_len=max_input_len, max_seq_len=max_seq_len,
         k_scale=k_scale, v_scale=v_scale, alibi_slopes=alibi_slopes, sliding_window=sliding_window,
@@ -32,5 +32,5 @@ def context_attention_fwd(q, k, v, o, kv_cache_dtype: str, k_cache, v_cache, b_l
         rotary_dim=rotary_dim, is_neox_style=is_neox_style, is_lazy=None,
         q_offset=None if is_mepic else q_offset, q_mask=q_mask,
         pos_mode=_ffi.POS_NATURAL if is_mepic else _ffi.POS_OFFSET, rotate_new_k=True,
-        fp32_rotary=force_fp32_rotary, kernel=_kernel, num_splits=_num_splits, phases=_phases)
-    return
+        fp32_rotary=force_fp32_rotary, kernel=_kernel, num_splits=_num_splits, phases=_phases, _return_plan=_return_plan)
+    return plan

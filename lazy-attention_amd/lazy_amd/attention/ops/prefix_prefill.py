@@ -22,22 +22,23 @@ def context_attention_fwd(q, k, v, o, kv_cache_dtype: str, k_cache, v_cache, b_l
                           sm_scale=None, skip_decode=False, cos_sin_cache=None, rotary_dim=None,
                           is_neox_style=True, is_lazy=None, q_offset=None, q_mask=None, *,
                           _kernel: int = _ffi.KERNEL_AUTO, _num_splits: int = 0,
-                          _phases: int = _ffi.PHASE_ALL):
+                          _phases: int = _ffi.PHASE_ALL, _return_plan: bool = False):
     if is_lazy is None:
         is_lazy = torch.zeros(b_seq_len.shape[0], dtype=torch.bool, device=q.device)
         if cos_sin_cache is None:
-            cos_sin_cache = q.new_zeros((1, q.shape[-1]))
+            half = q.shape[-1] // 2                      # one row: cos 1, sin 0
+            cos_sin_cache = torch.cat([q.new_ones(half), q.new_zeros(half)])[None]
             rotary_dim = q.shape[-1]
         if q_offset is None:
             q_offset = torch.zeros_like(b_loc, dtype=torch.int32)
     elif q_offset is None:
         raise ValueError("q_offset is required when is_lazy is given")
-    _launch.launch_prefill(
+    plan = _launch.launch_prefill(
         q=q, k=k, v=v, o=o, kv_cache_dtype=kv_cache_dtype, k_cache=k_cache, v_cache=v_cache,
         b_loc=b_loc, b_start_loc=b_start_loc, b_seq_len=b_seq_len, max_input_len=max_input_len, max_seq_len=max_seq_len,
         k_scale=k_scale, v_scale=v_scale, alibi_slopes=alibi_slopes, sliding_window=sliding_window,
         sm_scale=sm_scale, skip_decode=skip_decode, cos_sin_cache=cos_sin_cache,
         rotary_dim=rotary_dim, is_neox_style=is_neox_style, is_lazy=is_lazy, q_offset=q_offset,
         q_mask=q_mask, pos_mode=_ffi.POS_BLOCK_UNIFORM, rotate_new_k=False, kernel=_kernel,
-        num_splits=_num_splits, phases=_phases)
-    return
+        num_splits=_num_splits, phases=_phases, _return_plan=_return_plan)
+    return plan
