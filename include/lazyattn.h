@@ -35,7 +35,9 @@ enum {
 enum {
     LAZYATTN_KERNEL_AUTO = 0,
     LAZYATTN_KERNEL_GENERIC = 1, /* fp32 arithmetic, any geometry */
-    LAZYATTN_KERNEL_MFMA = 2     /* bf16 MFMA, head_dim 128 / 64, 16-token pages */
+    LAZYATTN_KERNEL_MFMA = 2,    /* bf16 MFMA, head_dim 128, 16-token pages; workgroup shape chosen */
+    LAZYATTN_KERNEL_MFMA4 = 3,   /* ... with 4 x 32 query rows per workgroup */
+    LAZYATTN_KERNEL_MFMA8 = 4    /* ... with 8 x 32 query rows per workgroup */
 };
 
 /* which launches of a call to enqueue (profiling aid; default = both) */

@@ -67,7 +67,7 @@ extern "C" int lazyattn_prefix_prefill(const lazyattn_prefill_params *p, void *s
     int kernel = p->kernel;
     if (kernel == LAZYATTN_KERNEL_AUTO)
         kernel = mfma_supports(*p) ? LAZYATTN_KERNEL_MFMA : LAZYATTN_KERNEL_GENERIC;
-    if (kernel == LAZYATTN_KERNEL_MFMA) {
+    if (kernel == LAZYATTN_KERNEL_MFMA || kernel == LAZYATTN_KERNEL_MFMA4 || kernel == LAZYATTN_KERNEL_MFMA8) {
         if (!mfma_supports(*p)) return LAZYATTN_E_UNSUPPORTED;
         return launch_prefill_mfma(*p, s);
     }

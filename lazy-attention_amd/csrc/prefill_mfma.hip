@@ -50,7 +50,7 @@ constexpr int K_TILE = PAGES * K_PAGE;
 constexpr int V_G = 2048;
 constexpr int V_PAGE = 2 * V_G;
 constexpr int V_TILE = PAGES * V_PAGE;
-constexpr int LDS_BYTES = 2 * (K_TILE + V_TILE);   // double buffered: 64 KB
+constexpr int KV_BYTES = 2 * (K_TILE + V_TILE);    // double buffered: 64 KB
 
 enum { TILE_FULL = 0, TILE_EDGE = 1, TILE_NEW = 2 };
 
@@ -131,13 +131,16 @@ template <typename TT> struct KRegs {
 // gathering wave: the gather's address arithmetic, fp32 rotation and LDS writes run in
 // the shadow of the other wave's MFMAs, and neither role ever waits for the other's
 // memory latency -- they only meet at one barrier per tile.
-constexpr int NC = 4;                    // computing waves = units per workgroup
+// NC = computing waves = 32-row units per workgroup: 8 (12 waves, three per SIMD) for long
+// key ranges, 4 (8 waves) when the call is small and more, lighter workgroups fill the chip
+// with fewer key-axis splits.
+constexpr int lds_bytes(int nc) { return KV_BYTES + nc * 8 * 1024; }   // + Q^T fragments, re-read every tile
 constexpr int LT = 256;                  // gathering threads
 constexpr int KI = (NT * 8) / LT;        // K items per gathering thread and tile (512 per tile)
 constexpr int VI = (NT * 16) / LT;       // V items per gathering thread and tile (1024 of 16 bytes)
 
-template <bool FP8, typename TT>
-__global__ void __launch_bounds__(512)
+template <int NC, bool FP8, typename TT>
+__global__ void __launch_bounds__((NC + 4) * 64)
 prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int n_mt) {
     constexpr int VI_CTX = FP8 ? VI / 2 : VI;        // an fp8 page row of 16 slots is one 16-byte item
     constexpr uint32_t TSZ = sizeof(TT);
@@ -197,7 +200,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     // Branch-free on purpose (a branch around a load makes the compiler drain every
     // outstanding load at the join): pages past the context read entry n_pages-1 and get
     // limit 0; an absent q_offset / q_mask array is replaced by the block table, masked to 0.
-    struct Meta { int bt[PAGES], qo[PAGES], lim[PAGES]; };
+    struct Meta { int bt0, bt1, bt2, bt3, qo0, qo1, qo2, qo3, lim0, lim1, lim2, lim3; };
     // Read through the scalar unit (constant address space): the values are wave-uniform,
     // they land in SGPRs, and waiting for them never drains the vector loads in flight.
     typedef const int32_t __attribute__((address_space(4))) *sptr_i32;
@@ -209,27 +212,30 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     const int64_t qo_s1 = use_qo ? p.qo_stride[1] : p.bt_stride[1];
     const int64_t qm_s1 = use_qmask ? p.qm_stride[1] : p.bt_stride[1];
     const int qo_and = use_qo ? -1 : 0, qm_and = use_qmask ? -1 : 0;
+    auto load_page = [&](int j, int &bt, int &qo, int &lim) {
+        int jc = j < n_pages ? j : n_pages - 1;
+        jc = jc < 0 ? 0 : jc;
+        bt = bt_row[jc * bt_s1];
+        qo = qo_row[jc * qo_s1] & qo_and;
+        const int qm = qm_row[jc * qm_s1] & qm_and;                                  // old_ops:165-167
+        int l = ctx_len - j * BS;
+        l = l < BS - qm ? l : BS - qm;
+        l = l > BS ? BS : l;
+        lim = l < 0 ? 0 : l;
+    };
     auto load_meta = [&](int tile) -> Meta {
         Meta m;
-#pragma unroll
-        for (int pg = 0; pg < PAGES; ++pg) {
-            const int j = tile * PAGES + pg;
-            int jc = j < n_pages ? j : n_pages - 1;
-            jc = jc < 0 ? 0 : jc;
-            m.bt[pg] = bt_row[jc * bt_s1];
-            m.qo[pg] = qo_row[jc * qo_s1] & qo_and;
-            const int qm = qm_row[jc * qm_s1] & qm_and;                              // old_ops:165-167
-            int lim = ctx_len - j * BS;
-            lim = lim < BS - qm ? lim : BS - qm;
-            lim = lim > BS ? BS : lim;
-            m.lim[pg] = lim < 0 ? 0 : lim;
-        }
+        load_page(tile * PAGES + 0, m.bt0, m.qo0, m.lim0);
+        load_page(tile * PAGES + 1, m.bt1, m.qo1, m.lim1);
+        load_page(tile * PAGES + 2, m.bt2, m.qo2, m.lim2);
+        load_page(tile * PAGES + 3, m.bt3, m.qo3, m.lim3);
         return m;
     };
-    auto sel4 = [](const int *a, int pg) { return pg < 2 ? (pg == 0 ? a[0] : a[1]) : (pg == 2 ? a[2] : a[3]); };
-    auto page_bt = [&](const Meta &m, int pg) { return sel4(m.bt, pg); };
-    auto page_qo = [&](const Meta &m, int pg) { return sel4(m.qo, pg); };
-    auto page_lim = [&](const Meta &m, int pg) { return sel4(m.lim, pg); };
+    // by value on purpose: taking the address of a member array would push the struct to scratch memory
+    auto sel4 = [](int a0, int a1, int a2, int a3, int pg) { return pg < 2 ? (pg == 0 ? a0 : a1) : (pg == 2 ? a2 : a3); };
+    auto page_bt = [&](const Meta &m, int pg) { return sel4(m.bt0, m.bt1, m.bt2, m.bt3, pg); };
+    auto page_qo = [&](const Meta &m, int pg) { return sel4(m.qo0, m.qo1, m.qo2, m.qo3, pg); };
+    auto page_lim = [&](const Meta &m, int pg) { return sel4(m.lim0, m.lim1, m.lim2, m.lim3, pg); };
 
     // ---- descriptor of a tile: kind and which of its 64 keys exist ----
     struct TileDesc { int kind; uint32_t vlo, vhi; };
@@ -519,15 +525,17 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     const int row = t0 + l32;                                    // token index of this lane's query row
     const bool row_ok = active && row < q_len;
 
-    // Q^T fragments: B operand of S^T = K.Q^T, lane = (row l32, d = ks*16 + gh*8 .. +8)
-    bf16x8_t qf[8];
+    // Q^T fragments: B operand of S^T = K.Q^T, lane = (row l32, d = ks*16 + gh*8 .. +8).
+    // They live in this wave's own LDS slice (not in registers: three waves share a SIMD's
+    // register file) and are re-read for every tile.
+    uint8_t *qlds = lds + KV_BYTES + wave * 8192 + lane * 16;
     {
         const bf16_t *qp = (const bf16_t *)p.q + (qs + row) * p.q_stride[0] + (int64_t)h * p.q_stride[1] + gh * 8;
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
             uint4 v = make_uint4(0, 0, 0, 0);
             if (row_ok) v = *reinterpret_cast<const uint4 *>(qp + ks * 16);
-            qf[ks] = *reinterpret_cast<bf16x8_t *>(&v);
+            *reinterpret_cast<uint4 *>(qlds + ks * 1024) = v;
         }
     }
     const float cs2 = p.sm_scale * 1.4426950408889634f;          // scores -> log2 units
@@ -539,28 +547,18 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         for (int i = 0; i < 16; ++i) acc[dt][i] = 0.f;
 
     // ---- S^T = K . Q^T for one 64-key tile: two independent 32-key accumulation chains ----
-    // The LDS reads of the A fragments run six ahead of the MFMAs that consume them, so the
-    // matrix pipe does not wait for an LDS round trip between instructions.
     auto qk_tile = [&](const uint8_t *ktile, f32x16_t &s0, f32x16_t &s1) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) { s0[i] = 0.f; s1[i] = 0.f; }
         const uint8_t *kp = ktile + (l32 >> 4) * K_PAGE + gh * 256 + (l32 & 15) * 16;
-        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
             const bf16x8_t a0 = *reinterpret_cast<const bf16x8_t *>(kp + ks * 512);
             const bf16x8_t a1 = *reinterpret_cast<const bf16x8_t *>(kp + 2 * K_PAGE + ks * 512);
-            s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, qf[ks], s0, 0, 0, 0);
-            s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, qf[ks], s1, 0, 0, 0);
+            const bf16x8_t q = *reinterpret_cast<const bf16x8_t *>(qlds + ks * 1024);
+            s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, q, s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, q, s1, 0, 0, 0);
         }
-        __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);            // 6 DS reads up front
-#pragma unroll
-        for (int i = 0; i < 10; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);        // 1 MFMA
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);        // 1 DS read
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, 6, 0);
-        __builtin_amdgcn_sched_barrier(0);
     };
     // ---- masks: register i of half `sub` holds key sub*32 + 8*(i/4) + 4*gh + i%4 ----
     auto mask_half = [&](f32x16_t &s, uint32_t vbits, int sub, int kind, int m0) {
@@ -725,13 +723,23 @@ prefill_combine_kernel(const lazyattn_prefill_params p, const int nsplit) {
 }
 
 // ------------------------------------------------------------------ host side
-static int mfma_waves(const lazyattn_prefill_params &) { return NC; }   // units per workgroup
-
-static int mfma_mtiles(const lazyattn_prefill_params &p, int nw) {
+static int mfma_units(const lazyattn_prefill_params &p) {
     const int group = p.num_q_heads / p.num_kv_heads;
-    const int units = ((p.max_q_len + UNIT - 1) / UNIT) * group;
-    return (units + nw - 1) / nw;
+    return ((p.max_q_len + UNIT - 1) / UNIT) * group;
 }
+// units (computing waves) per workgroup
+static int mfma_waves(const lazyattn_prefill_params &p) {
+    if (p.kernel == LAZYATTN_KERNEL_MFMA4) return 4;
+    if (p.kernel == LAZYATTN_KERNEL_MFMA8) return 8;
+    const int units = mfma_units(p);
+    if (units <= 4) return 4;
+    // 64-key tiles of work per CU if the 8-unit kernel is used: small calls take the lighter one
+    const int64_t wgs8 = (int64_t)p.batch * p.num_kv_heads * ((units + 7) / 8);
+    const int64_t tiles = p.max_seq_len > 0 ? (p.max_seq_len + NT - 1) / NT : 64;
+    return wgs8 * tiles >= 16 * 256 ? 8 : 4;
+}
+
+static int mfma_mtiles(const lazyattn_prefill_params &p, int nw) { return (mfma_units(p) + nw - 1) / nw; }
 
 static int mfma_splits(const lazyattn_prefill_params &p, int nw) {
     if (p.num_splits > 0) return p.num_splits > 64 ? 64 : p.num_splits;
@@ -772,9 +780,10 @@ size_t mfma_workspace_bytes(const lazyattn_prefill_params &p) {
     return (size_t)ns * (size_t)p.num_tokens * p.num_q_heads * (D + 1) * sizeof(float);
 }
 
-template <bool FP8, typename TT>
+template <int NC, bool FP8, typename TT>
 static int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt, hipStream_t stream) {
-    auto kern = prefill_mfma_kernel<FP8, TT>;
+    auto kern = prefill_mfma_kernel<NC, FP8, TT>;
+    constexpr int LDS_BYTES = lds_bytes(NC);
     static bool attr_set = false;
     if (!attr_set) {
         if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
@@ -782,17 +791,18 @@ static int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt,
         attr_set = true;
     }
     const unsigned nblocks = (unsigned)(p.batch * p.num_kv_heads * nsplit * n_mt);
-    hipLaunchKernelGGL(kern, dim3(nblocks), dim3(512), LDS_BYTES, stream, p, nsplit, n_mt);
+    hipLaunchKernelGGL(kern, dim3(nblocks), dim3((NC + 4) * 64), LDS_BYTES, stream, p, nsplit, n_mt);
     return hipGetLastError() == hipSuccess ? LAZYATTN_OK : LAZYATTN_E_LAUNCH;
 }
 
-static int launch_mfma_any(const lazyattn_prefill_params &p, int nsplit, int n_mt, hipStream_t stream) {
+template <int NC>
+static int launch_mfma_nc(const lazyattn_prefill_params &p, int nsplit, int n_mt, hipStream_t stream) {
     const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3;
     const bool t32 = p.table_dtype == LAZYATTN_F32;
-    if (fp8) return t32 ? launch_mfma_t<true, float>(p, nsplit, n_mt, stream)
-                        : launch_mfma_t<true, bf16_t>(p, nsplit, n_mt, stream);
-    return t32 ? launch_mfma_t<false, float>(p, nsplit, n_mt, stream)
-               : launch_mfma_t<false, bf16_t>(p, nsplit, n_mt, stream);
+    if (fp8) return t32 ? launch_mfma_t<NC, true, float>(p, nsplit, n_mt, stream)
+                        : launch_mfma_t<NC, true, bf16_t>(p, nsplit, n_mt, stream);
+    return t32 ? launch_mfma_t<NC, false, float>(p, nsplit, n_mt, stream)
+               : launch_mfma_t<NC, false, bf16_t>(p, nsplit, n_mt, stream);
 }
 
 int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
@@ -806,7 +816,7 @@ int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
         if (((uintptr_t)p.workspace) & 15) return LAZYATTN_E_WORKSPACE;
     }
     if (phases & LAZYATTN_PHASE_MAIN) {
-        const int rc = launch_mfma_any(p, nsplit, n_mt, stream);
+        const int rc = nw == 8 ? launch_mfma_nc<8>(p, nsplit, n_mt, stream) : launch_mfma_nc<4>(p, nsplit, n_mt, stream);
         if (rc != LAZYATTN_OK) return rc;
     }
     if (nsplit > 1 && (phases & LAZYATTN_PHASE_COMBINE)) {

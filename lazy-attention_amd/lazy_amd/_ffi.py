@@ -16,7 +16,7 @@ _lib = None
 
 F32, BF16, F16, FP8_E4M3, FP8_E5M2 = 0, 1, 2, 3, 4
 POS_NATURAL, POS_OFFSET, POS_BLOCK_UNIFORM = 0, 1, 2
-KERNEL_AUTO, KERNEL_GENERIC, KERNEL_MFMA = 0, 1, 2
+KERNEL_AUTO, KERNEL_GENERIC, KERNEL_MFMA, KERNEL_MFMA4, KERNEL_MFMA8 = 0, 1, 2, 3, 4
 PHASE_MAIN, PHASE_COMBINE, PHASE_ALL = 1, 2, 3
 
 ERRORS = {-1: "NULL", -2: "SHAPE", -3: "DTYPE", -4: "UNSUPPORTED", -5: "WORKSPACE", -6: "LAUNCH"}
