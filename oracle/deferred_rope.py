@@ -286,13 +286,19 @@ def prefix_prefill(q, k, v, k_cache, v_cache, block_table, b_start_loc, b_seq_le
 
 
 def paged_decode(q, k_cache, v_cache, block_table, query_start_loc, seq_lens,
-                 cos_sin_cache, q_mask=None, *, kv_cache_dtype="auto",
+                 cos_sin_cache, q_mask=None, *, q_offset=None, is_lazy=None,
+                 pos_mode: int = POS_NATURAL, kv_cache_dtype="auto",
                  k_scale=1.0, v_scale=1.0, sm_scale=None, sliding_window: int = 0,
                  out=None, compute_dtype=torch.float32):
-    """q_len==1 rows of the un-rotated-cache variant
-    (old_ops/chunked_prefill_paged_decode.py:68-280): all seq_len keys come from the
-    paged cache (the new token was written there by the caller), each rotated at its
-    natural position j*BS+o; pad slots masked by q_mask; requests with q_len>1 skipped."""
+    """q_len==1 rows: all seq_len keys come from the paged cache (the new token was
+    written there by the caller); requests with q_len>1 are skipped.
+
+    pos_mode=POS_NATURAL: un-rotated cache, key n rotated at n
+      (old_ops/chunked_prefill_paged_decode.py:68-280).
+    pos_mode=POS_BLOCK_UNIFORM: the reference de-rotates Q by q_offset-1 once per distinct
+      offset (ops/models/llama_v1.py:231-262); rotating the page's keys forward by the same
+      angle gives the same scores, which is how it is stated here.  Requests with
+      is_lazy[b]==0 are not rotated and ignore q_mask."""
     cdt = compute_dtype
     hq, d = q.shape[1], q.shape[2]
     hkv = k_cache.shape[1]
@@ -314,11 +320,19 @@ def paged_decode(q, k_cache, v_cache, block_table, query_start_loc, seq_lens,
         kg, vg = gather_pages(kc, vc, block_table[b, :npages])
         kg = kg[:seq_len].to(cdt); vg = vg[:seq_len].to(cdt)
         n = torch.arange(seq_len)
+        lazy_b = True if is_lazy is None else bool(is_lazy[b])
+        vanilla = pos_mode == POS_BLOCK_UNIFORM and not lazy_b
         valid = torch.ones(seq_len, dtype=torch.bool)
-        if q_mask is not None:
+        if q_mask is not None and not vanilla:
             valid = (n % bs) < (bs - q_mask[b, :npages].long()[n // bs])
-        rows = table[n]
-        kg = neox_rotate(kg, rows[:, None, :half], rows[:, None, half:])
+        if not vanilla:
+            if pos_mode == POS_NATURAL:
+                pos = n
+            else:
+                qo = q_offset[b, :npages].long()[n // bs]
+                pos = torch.where(qo != 0, qo - 1, torch.zeros_like(qo))
+            rows = table[pos]
+            kg = neox_rotate(kg, rows[:, None, :half], rows[:, None, half:])
         kg = torch.where(valid[:, None, None], kg, torch.zeros_like(kg))
         vg = torch.where(valid[:, None, None], vg, torch.zeros_like(vg))
         fill = None

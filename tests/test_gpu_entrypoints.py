@@ -1,0 +1,73 @@
+"""GPU parity of the entry points the attention backend calls
+(``chunked_prefill_paged_decode`` of both variants): a mixed batch of prefill requests
+and q_len==1 requests, checked against the CPU oracle."""
+import pytest
+import torch
+
+from oracle import deferred_rope as orc
+from lazy_amd import workloads as wl
+from lazy_amd.attention.old_ops.chunked_prefill_paged_decode import chunked_prefill_paged_decode as entry_unrotated
+from lazy_amd.attention.ops.chunked_prefill_paged_decode import chunked_prefill_paged_decode as entry_block_uniform
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _mixed(variant, dtype, d, seed=41):
+    w = wl.make_workload("mixed", dtype=dtype, hq=8, hkv=2, d=d, theta=500000.0, block_size=16,
+                         doc_lens=[40, 16, 33, 70, 5], requests=[[3, 1, 0], [2], [0, 2, 3, 1], [4, 0]],
+                         q_lens=[70, 1, 9, 1], variant=variant, seed=seed)
+    # the attention backend writes the new tokens into the paged cache before the call
+    # (backends/triton_attn.py:100-109); the q_len==1 kernels read them from there
+    x = w.k_cache.shape[4]
+    for b in range(4):
+        qs, qe = int(w.b_start_loc[b]), int(w.b_start_loc[b + 1])
+        ctx = int(w.b_seq_len[b]) - (qe - qs)
+        for t in range(qe - qs):
+            n = ctx + t
+            pb = int(w.block_table[b, n // 16]); o_ = n % 16
+            w.k_cache[pb, :, :, o_, :] = w.k[qs + t].view(2, d // x, x)
+            w.v_cache[pb, :, :, o_] = w.v[qs + t]
+    return w
+
+
+def _expected(w, lazy=None):
+    ref = torch.full_like(w.q, 5.0)
+    orc.prefix_prefill(w.q, w.k, w.v, w.k_cache, w.v_cache, w.block_table, w.b_start_loc, w.b_seq_len,
+                       w.cos_sin_cache, w.q_offset, w.q_mask, pos_mode=w.pos_mode,
+                       rotate_new_k=w.rotate_new_k, is_lazy=lazy, skip_decode=True, out=ref)
+    orc.paged_decode(w.q, w.k_cache, w.v_cache, w.block_table, w.b_start_loc, w.b_seq_len,
+                     w.cos_sin_cache, w.q_mask, q_offset=w.q_offset, is_lazy=lazy,
+                     pos_mode=orc.POS_NATURAL if w.pos_mode != orc.POS_BLOCK_UNIFORM else w.pos_mode, out=ref)
+    return ref
+
+
+@pytest.mark.parametrize("dtype,d,tol", [(torch.float32, 64, 1e-5), (torch.bfloat16, 128, 2e-2)])
+def test_entry_unrotated_cache_mixed_batch(dtype, d, tol):
+    print(f"case: entry old_ops {dtype}", flush=True)
+    w = _mixed("natural", dtype, d)
+    ref = _expected(w)
+    g = w.to(DEV)
+    out = torch.full_like(g.q, 5.0)
+    entry_unrotated(g.q, g.k, g.v, out, "auto", g.k_cache, g.v_cache, g.block_table, g.b_start_loc, g.b_seq_len,
+                    g.max_seq_len, g.max_query_len, g.k_scale, g.v_scale, sm_scale=d ** -0.5, rotary_dim=d,
+                    cos_sin_cache=g.cos_sin_cache, q_mask=g.q_mask)
+    err = (out.cpu().float() - ref.float()).abs().max().item()
+    assert err < tol, err
+
+
+@pytest.mark.parametrize("dtype,d,tol", [(torch.float32, 64, 1e-5), (torch.bfloat16, 128, 2e-2)])
+def test_entry_block_uniform_mixed_batch_with_packed_table(dtype, d, tol):
+    print(f"case: entry ops {dtype}", flush=True)
+    w = _mixed("block_uniform", dtype, d)
+    lazy = torch.tensor([True, True, False, False])
+    ref = _expected(w, lazy)
+    g = w.to(DEV)
+    out = torch.full_like(g.q, 5.0)
+    packed = (g.block_table.long() << 32) | (g.q_offset.long() << 16) | g.q_mask.long()
+    entry_block_uniform(g.q, g.k, g.v, out, "auto", g.k_cache, g.v_cache, g.block_table, g.b_start_loc,
+                        g.b_seq_len, g.max_seq_len, g.max_query_len, g.k_scale, g.v_scale, sm_scale=d ** -0.5,
+                        rotary_dim=d, cos_sin_cache=g.cos_sin_cache, is_lazy=lazy.to(DEV), q_offset=None,
+                        q_mask=None, packed_block_table=packed)
+    err = (out.cpu().float() - ref.float()).abs().max().item()
+    assert err < tol, err

@@ -329,3 +329,38 @@ def test_decode_oracle_equals_prefill_with_token_in_cache():
     dec = orc.paged_decode(w.q, w.k_cache, w.v_cache, w.block_table, w.b_start_loc, w.b_seq_len,
                            w.cos_sin_cache, w.q_mask, compute_dtype=torch.float64)
     assert (dec - pre).abs().max() < 1e-6
+
+
+def test_lazy_decode_rotating_keys_equals_derotating_query():
+    """ops/models/llama_v1.py:231-262 rotates Q backwards by q_offset-1 per page; the oracle
+    rotates the page's keys forwards.  Both give the same scores: check on one request by
+    brute force over pages."""
+    w = wl.make_workload("ldec", dtype=torch.float32, hq=4, hkv=2, d=8, theta=10000.0, block_size=4,
+                         doc_lens=[7, 8], requests=[[1, 0]], q_lens=[1], variant="block_uniform", seed=13)
+    ctx = int(w.b_seq_len[0]) - 1
+    pb = int(w.block_table[0, ctx // 4])
+    w.k_cache[pb, :, :, ctx % 4, :] = w.k[0].view(2, 2, 4)
+    w.v_cache[pb, :, :, ctx % 4] = w.v[0]
+    got = orc.paged_decode(w.q, w.k_cache, w.v_cache, w.block_table, w.b_start_loc, w.b_seq_len,
+                           w.cos_sin_cache, w.q_mask, q_offset=w.q_offset, pos_mode=orc.POS_BLOCK_UNIFORM,
+                           compute_dtype=torch.float64)
+    tab = w.cos_sin_cache.double()
+    seq = ctx + 1
+    scores = torch.full((4, seq), float("-inf"), dtype=torch.float64)
+    vals = torch.zeros(seq, 2, 8, dtype=torch.float64)
+    for n in range(seq):
+        j, o_ = divmod(n, 4)
+        if o_ >= 4 - int(w.q_mask[0, j]):
+            continue
+        blk = int(w.block_table[0, j])
+        kvec = w.k_cache[blk, :, :, o_, :].reshape(2, 8).double()
+        vals[n] = w.v_cache[blk, :, :, o_].double()
+        qo = int(w.q_offset[0, j])
+        rows = tab[qo - 1] if qo > 1 else tab[0]
+        c, s_ = rows[:4], rows[4:]
+        qrot = orc.neox_rotate(w.q[0].double(), c, -s_)           # rotate Q backwards
+        for h in range(4):
+            scores[h, n] = (qrot[h] * kvec[h // 2]).sum() / math.sqrt(8)
+    p = torch.softmax(scores, dim=-1)
+    ref = torch.stack([(p[h][:, None] * vals[:, h // 2]).sum(0) for h in range(4)])
+    assert (got[0].double() - ref).abs().max() < 1e-6
