@@ -76,6 +76,8 @@ def main():
     ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5])
     ap.add_argument("--num-splits", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a 256 MiB device-to-device copy (known traffic, for scaling profiler counters)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU: the operator has no multi-GPU path "
@@ -109,6 +111,12 @@ def main():
     main_ms = statistics.median(reps)
     plan.run()
     torch.cuda.synchronize()
+    if a.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
 
     tflops = w.flops / (ms * 1e-3) / 1e12
     main_tflops = w.flops / (main_ms * 1e-3) / 1e12
