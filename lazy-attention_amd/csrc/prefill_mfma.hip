@@ -62,6 +62,17 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
     return *reinterpret_cast<uint32_t *>(&h);
 }
 // value of x in the partner lane (lane ^ 32) of the wave, via v_permlane32_swap
+// IEEE-754 maximum of three (v_maximum3_f32): NaN-propagating, so no canonicalising pre-pass
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    return __builtin_elementwise_maximum(__builtin_elementwise_maximum(a, b), c);
+}
+// acc + lo(w) + hi(w) for a packed bf16 pair (v_dot2c_f32_bf16 against (1, 1))
+__device__ __forceinline__ float dot2_ones(uint32_t w, float acc) {
+    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+    const uint32_t one = 0x3f803f80u;
+    return __builtin_amdgcn_fdot2_f32_bf16(*reinterpret_cast<const bf16x2_t *>(&w),
+                                           *reinterpret_cast<const bf16x2_t *>(&one), acc, false);
+}
 __device__ __forceinline__ float partner32(float x, bool upper) {
     uint32_t a = __float_as_uint(x), b = a;
     asm volatile("" : "+v"(b));      // two distinct registers for the swap
@@ -539,7 +550,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         }
     }
     const float cs2 = p.sm_scale * 1.4426950408889634f;          // scores -> log2 units
-    float m_run = -INFINITY, l_run = 0.f;
+    float m_run = -INFINITY, l_run = 0.f, l_alt = 0.f;              // row sum kept as two chains
     f32x16_t acc[4];
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt)
@@ -574,10 +585,13 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     };
     // ---- running max over the tile, rescale of the accumulators when it grew (old_ops:287-291) ----
     auto update_max = [&](const f32x16_t &s0, const f32x16_t &s1) -> float {
-        float mx = fmaxf(fmaxf(s0[0], s0[1]), fmaxf(s1[0], s1[1]));
+        // v_maximum3_f32: no quieting pre-pass over the MFMA results, NaN scores stay NaN
+        float ma = max3(s0[0], s0[1], s0[2]), mb = max3(s1[0], s1[1], s1[2]);
 #pragma unroll
-        for (int i = 2; i < 16; i += 2) mx = fmaxf(mx, fmaxf(fmaxf(s0[i], s0[i + 1]), fmaxf(s1[i], s1[i + 1])));
-        mx = fmaxf(mx, partner32(mx, gh != 0));
+        for (int i = 3; i < 15; i += 2) { ma = max3(ma, s0[i], s0[i + 1]); mb = max3(mb, s1[i], s1[i + 1]); }
+        float mx = max3(ma, mb, s0[15]);
+        mx = max3(mx, s1[15], s1[15]);
+        mx = max3(mx, partner32(mx, gh != 0), mx);
         const float m_new = fmaxf(m_run, mx);
         const float m_safe = m_new == -INFINITY ? 0.f : m_new;
         const float alpha = __builtin_amdgcn_exp2f((m_run - m_safe) * cs2);          // m_run = -inf -> 0
@@ -585,6 +599,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt) acc[dt] *= alpha;
             l_run *= alpha;
+            l_alt *= alpha;
         }
         m_run = m_new;
         return m_safe * cs2;
@@ -594,12 +609,14 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         float pr[16];
 #pragma unroll
         for (int i = 0; i < 16; ++i) pr[i] = __builtin_amdgcn_exp2f(fmaf(s[i], cs2, -mc));
-        float la = 0.f, lb = 0.f;
+        uint32_t w[8];
 #pragma unroll
-        for (int i = 0; i < 16; i += 2) { la += pr[i]; lb += pr[i + 1]; }
-        l_run += la + lb;                                                            // old_ops:312
-        uint4 w0 = make_uint4(pack_bf16(pr[0], pr[1]), pack_bf16(pr[2], pr[3]), pack_bf16(pr[4], pr[5]), pack_bf16(pr[6], pr[7]));
-        uint4 w1 = make_uint4(pack_bf16(pr[8], pr[9]), pack_bf16(pr[10], pr[11]), pack_bf16(pr[12], pr[13]), pack_bf16(pr[14], pr[15]));
+        for (int i = 0; i < 8; ++i) w[i] = pack_bf16(pr[2 * i], pr[2 * i + 1]);
+        // row sum of the rounded probabilities, two per instruction (old_ops:312 sums them unrounded)
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) { l_run = dot2_ones(w[i], l_run); l_alt = dot2_ones(w[i + 1], l_alt); }
+        uint4 w0 = make_uint4(w[0], w[1], w[2], w[3]);
+        uint4 w1 = make_uint4(w[4], w[5], w[6], w[7]);
         p0 = *reinterpret_cast<bf16x8_t *>(&w0);
         p1 = *reinterpret_cast<bf16x8_t *>(&w1);
     };
@@ -635,21 +652,18 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         const uint8_t *vtile = lds + 2 * K_TILE + cur * V_TILE;
         const TileDesc td = describe(tile, m_cur);
         const Meta m_new = load_meta(tile + 2);
-        if (td.kind == TILE_FULL) {
-            // rows of an idle wave are all-zero queries: harmless, never stored
+        const int m0 = td.kind == TILE_NEW ? (tile - n_ctx_tiles) * NT : 0;
+        // One call site for the tile body: the accumulators keep their registers round the loop.
+        // Rows of an idle wave are all-zero queries (harmless, never stored); a new-token tile
+        // entirely in this wave's future contributes nothing (causal) and is skipped.
+        if (td.kind != TILE_NEW || m0 <= t0 + UNIT - 1) {
             f32x16_t s0, s1;
             qk_tile(ktile, s0, s1);
-            attend(vtile, s0, s1);
-        } else {
-            const int m0 = td.kind == TILE_NEW ? (tile - n_ctx_tiles) * NT : 0;
-            // a new-token tile entirely in this wave's future contributes nothing (causal)
-            if (active && (td.kind != TILE_NEW || m0 <= t0 + UNIT - 1)) {
-                f32x16_t s0, s1;
-                qk_tile(ktile, s0, s1);
+            if (td.kind != TILE_FULL) {
                 mask_half(s0, td.vlo, 0, td.kind, m0);
                 mask_half(s1, td.vhi, 1, td.kind, m0);
-                attend(vtile, s0, s1);
             }
+            attend(vtile, s0, s1);
         }
         m_cur = m_nxt;
         m_nxt = m_new;
@@ -657,6 +671,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     }
 
     // ---- epilogue ----
+    l_run += l_alt;
     l_run += partner32(l_run, gh != 0);
     if (!row_ok) return;
     const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
