@@ -145,10 +145,9 @@ template <typename TT> struct KRegs {
 // NC = computing waves = 32-row units per workgroup: 8 (12 waves, three per SIMD) for long
 // key ranges, 4 (8 waves) when the call is small and more, lighter workgroups fill the chip
 // with fewer key-axis splits.
-constexpr int lds_bytes(int nc) { return KV_BYTES + nc * 8 * 1024; }   // + Q^T fragments, re-read every tile
-constexpr int LT = 256;                  // gathering threads
-constexpr int KI = (NT * 8) / LT;        // K items per gathering thread and tile (512 per tile)
-constexpr int VI = (NT * 16) / LT;       // V items per gathering thread and tile (1024 of 16 bytes)
+constexpr int lds_bytes(int nc) { return KV_BYTES + nc * 8 * 1024 + 2 * PAGES * 4; }   // + Q^T fragments (re-read every tile) + page limits
+constexpr int KI = 2;                    // K items per gathering lane and tile: a page has 128 (8 chunks x 16 slots)
+constexpr int VI = 4;                    // V items per gathering lane and tile: a page has 256 of 16 bytes
 
 template <int NC, bool FP8, typename TT>
 __global__ void __launch_bounds__((NC + 4) * 64)
@@ -205,15 +204,14 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     const int tile_begin = (int)((int64_t)n_tiles * split / nsplit);
     const int tile_end = (int)((int64_t)n_tiles * (split + 1) / nsplit);
 
-    // ---- page metadata of a tile, fetched ahead of its use ----
-    // lane l holds the entries of page (l & 3) of the tile: physical block, q_offset, and
-    // the number of valid slots (pad mask and end of context folded together).
-    // Branch-free on purpose (a branch around a load makes the compiler drain every
-    // outstanding load at the join): pages past the context read entry n_pages-1 and get
-    // limit 0; an absent q_offset / q_mask array is replaced by the block table, masked to 0.
-    struct Meta { int bt0, bt1, bt2, bt3, qo0, qo1, qo2, qo3, lim0, lim1, lim2, lim3; };
-    // Read through the scalar unit (constant address space): the values are wave-uniform,
-    // they land in SGPRs, and waiting for them never drains the vector loads in flight.
+    // ---- page metadata, fetched ahead of its use ----
+    // Gathering wave w owns page w of every tile, so it needs one block-table entry, one
+    // q_offset and one q_mask per tile.  They are read through the scalar unit (constant address
+    // space): the values are wave-uniform, land in SGPRs, and waiting for them never drains the
+    // vector loads in flight.  Branch-free on purpose (a branch around a load makes the compiler
+    // drain every outstanding load at the join): pages past the context read entry n_pages-1
+    // and get limit 0; an absent q_offset / q_mask array is replaced by the block table, masked to 0.
+    struct PageMeta { int bt, qo, lim; };      // physical block, q_offset, number of valid slots
     typedef const int32_t __attribute__((address_space(4))) *sptr_i32;
     const bool use_qo = !vanilla && pos_mode != LAZYATTN_POS_NATURAL;
     const sptr_i32 bt_row = (sptr_i32)(p.block_table + b * p.bt_stride[0]);
@@ -223,51 +221,26 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     const int64_t qo_s1 = use_qo ? p.qo_stride[1] : p.bt_stride[1];
     const int64_t qm_s1 = use_qmask ? p.qm_stride[1] : p.bt_stride[1];
     const int qo_and = use_qo ? -1 : 0, qm_and = use_qmask ? -1 : 0;
-    auto load_page = [&](int j, int &bt, int &qo, int &lim) {
+    auto load_page = [&](int j) -> PageMeta {
+        PageMeta m;
         int jc = j < n_pages ? j : n_pages - 1;
         jc = jc < 0 ? 0 : jc;
-        bt = bt_row[jc * bt_s1];
-        qo = qo_row[jc * qo_s1] & qo_and;
+        m.bt = bt_row[jc * bt_s1];
+        m.qo = qo_row[jc * qo_s1] & qo_and;
         const int qm = qm_row[jc * qm_s1] & qm_and;                                  // old_ops:165-167
         int l = ctx_len - j * BS;
         l = l < BS - qm ? l : BS - qm;
         l = l > BS ? BS : l;
-        lim = l < 0 ? 0 : l;
-    };
-    auto load_meta = [&](int tile) -> Meta {
-        Meta m;
-        load_page(tile * PAGES + 0, m.bt0, m.qo0, m.lim0);
-        load_page(tile * PAGES + 1, m.bt1, m.qo1, m.lim1);
-        load_page(tile * PAGES + 2, m.bt2, m.qo2, m.lim2);
-        load_page(tile * PAGES + 3, m.bt3, m.qo3, m.lim3);
+        m.lim = l < 0 ? 0 : l;
         return m;
     };
-    // by value on purpose: taking the address of a member array would push the struct to scratch memory
-    auto sel4 = [](int a0, int a1, int a2, int a3, int pg) { return pg < 2 ? (pg == 0 ? a0 : a1) : (pg == 2 ? a2 : a3); };
-    auto page_bt = [&](const Meta &m, int pg) { return sel4(m.bt0, m.bt1, m.bt2, m.bt3, pg); };
-    auto page_qo = [&](const Meta &m, int pg) { return sel4(m.qo0, m.qo1, m.qo2, m.qo3, pg); };
-    auto page_lim = [&](const Meta &m, int pg) { return sel4(m.lim0, m.lim1, m.lim2, m.lim3, pg); };
-
-    // ---- descriptor of a tile: kind and which of its 64 keys exist ----
-    struct TileDesc { int kind; uint32_t vlo, vhi; };
-    auto describe = [&](int tile, const Meta &m) -> TileDesc {
-        TileDesc t{TILE_FULL, ~0u, ~0u};
-        if (tile >= n_ctx_tiles) {
-            t.kind = TILE_NEW;
-            const int n = t_end - (tile - n_ctx_tiles) * NT;
-            const uint64_t valid = n >= 64 ? ~0ull : (n <= 0 ? 0ull : ((1ull << n) - 1ull));
-            t.vlo = (uint32_t)valid; t.vhi = (uint32_t)(valid >> 32);
-        } else {
-            t.vlo = ((1u << page_lim(m, 0)) - 1u) | (((1u << page_lim(m, 1)) - 1u) << BS);
-            t.vhi = ((1u << page_lim(m, 2)) - 1u) | (((1u << page_lim(m, 3)) - 1u) << BS);
-            t.kind = (t.vlo & t.vhi) == ~0u ? TILE_FULL : TILE_EDGE;
-        }
-        return t;
-    };
+    // Valid-slot counts of the four pages of a context tile, one int per page and LDS buffer:
+    // written by the gathering waves with the tile, read by the computing waves for the masks.
+    int *page_lims = reinterpret_cast<int *>(lds + KV_BYTES + NC * 8192);
 
     if (gatherer) {
         // ====================================================================== gather
-        const int lt = tid - NC * 64;
+        const int gw = wave - NC;                                // this wave's page of every tile
         const bool rot_new = p.rotate_new_k && !vanilla;
         const float k_scale = FP8 ? *p.k_scale : 1.f;
         const float v_scale = FP8 ? *p.v_scale : 1.f;
@@ -279,46 +252,41 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         const uint32_t row_bytes = (uint32_t)p.table_stride * TSZ;
         // per-token rotation of context pages reads the packed table [2][D/16][rows][8]: the 16
         // slots of a page are 16 consecutive 16-byte chunks there
-        const bool packed_tab = p.cos_sin_packed != nullptr && !vanilla && pos_mode != LAZYATTN_POS_BLOCK_UNIFORM;
+        const bool per_token = !vanilla && pos_mode != LAZYATTN_POS_BLOCK_UNIFORM;
+        const bool packed_tab = p.cos_sin_packed != nullptr && per_token;
         const uint8_t *ctab_base = packed_tab ? (const uint8_t *)p.cos_sin_packed : tab_base;
         const uint32_t pos_bytes = packed_tab ? 8 * TSZ : row_bytes;       // bytes per unit of position
         const uint32_t sin_delta = packed_tab ? (uint32_t)(HALF / 8) * (uint32_t)p.packed_rows * 8 * TSZ : HALF * TSZ;
+        // K items of a page: 128 = (8 chunks of 8 (d, d+64) pairs) x 16 slots, two per lane
         uint32_t k_goff[KI], k_toff[KI];
-        int k_pg[KI];
 #pragma unroll
         for (int i = 0; i < KI; ++i) {
-            const int idx = lt + i * LT;
-            const int o = idx & 15, cp = (idx >> 4) & 7;
-            k_pg[i] = uniform(idx >> 7);
+            const int idx = lane + i * 64;
+            const int o = idx & 15, cp = idx >> 4;
             // bf16: [D/8][16][8] -> item (cp, o) at (cp*16 + o)*16 bytes, pair chunk +2048
             // fp8 : [D/16][16][16] -> 8 bytes at chunk cp/2, half cp&1, pair chunk +4*256
-            k_goff[i] = FP8 ? (uint32_t)((cp >> 1) * 256 + o * 16 + (cp & 1) * 8) : (uint32_t)((idx & 127) * 16);
+            k_goff[i] = FP8 ? (uint32_t)((cp >> 1) * 256 + o * 16 + (cp & 1) * 8) : (uint32_t)(idx * 16);
             // block-uniform rotation and un-rotated requests use one table row for the whole page
             k_toff[i] = packed_tab ? ((uint32_t)cp * (uint32_t)p.packed_rows + (uint32_t)o) * 8 * TSZ
-                      : ((pos_mode == LAZYATTN_POS_BLOCK_UNIFORM || vanilla) ? 0u : (uint32_t)o * row_bytes) +
-                            (uint32_t)cp * 8 * TSZ;
-        }
-        uint32_t v_goff[VI_CTX];
-        int v_pg[VI_CTX];
-#pragma unroll
-        for (int i = 0; i < VI_CTX; ++i) {
-            const int idx = lt + i * LT;
-            // bf16: 256 items of 16 bytes per page (d = idx/2, slots 8*(idx&1) ..); fp8: 128 items (d = idx)
-            v_pg[i] = uniform(FP8 ? idx >> 7 : idx >> 8);
-            v_goff[i] = (uint32_t)((idx & (FP8 ? 127 : 255)) * 16);
+                                   : (per_token ? (uint32_t)o * row_bytes : 0u) + (uint32_t)cp * 8 * TSZ;
         }
         KRegs<TT> kr[KI];
         uint4 vr[VI];
-        int v_lim[VI_CTX];
 
-        // ---- loads of a full context tile: no branch, no zero fill ----
-        auto issue_loads_full = [&](int tile, const Meta &meta) {
+        // ---- loads of a context page: no branch, no zero fill ----
+        auto issue_loads_ctx = [&](int tile, const PageMeta &pm) {
+            const int j = tile * PAGES + gw;
+            const uint8_t *kb = kc_base + pm.bt * kc_page_bytes;
+            // un-rotated requests read row 0 of the table (cos 1, sin 0): exact identity
+            const int nat = j * BS;                                                  // old_ops:183-184
+            int pos0 = pos_mode == LAZYATTN_POS_NATURAL ? nat
+                     : pos_mode == LAZYATTN_POS_OFFSET ? (pm.qo ? pm.qo - 1 : nat)      // old_ops:186-191
+                                                       : (pm.qo ? pm.qo - 1 : 0);       // ops:180-186
+            pos0 = vanilla ? 0 : pos0;
+            const uint8_t *tb = ctab_base + (int64_t)pos0 * pos_bytes;
 #pragma unroll
             for (int i = 0; i < KI; ++i) {
-                const int j = tile * PAGES + k_pg[i];
-                const int idx = lt + i * LT;
-                kr[i].lds_off = (uint32_t)(k_pg[i] * K_PAGE + (idx & 127) * 16);
-                const uint8_t *kb = kc_base + page_bt(meta, k_pg[i]) * kc_page_bytes;
+                kr[i].lds_off = (uint32_t)(gw * K_PAGE + (lane + i * 64) * 16);
                 if (FP8) {
                     const uint2 a = ldg8(kb, k_goff[i]), a2 = ldg8(kb, k_goff[i] + 4 * 256);
                     kr[i].k1 = make_uint4(a.x, a.y, 0, 0);
@@ -327,64 +295,54 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                     kr[i].k1 = ldg16(kb, k_goff[i]);
                     kr[i].k2 = ldg16(kb, k_goff[i] + 2048);
                 }
-                // un-rotated requests read row 0 of the table (cos 1, sin 0): exact identity
-                const int qo = page_qo(meta, k_pg[i]);
-                const int nat = j * BS;                                              // old_ops:183-184
-                int pos0 = pos_mode == LAZYATTN_POS_NATURAL ? nat
-                         : pos_mode == LAZYATTN_POS_OFFSET ? (qo ? qo - 1 : nat)      // old_ops:186-191
-                                                           : (qo ? qo - 1 : 0);       // ops:180-186
-                pos0 = vanilla ? 0 : pos0;
-                const uint8_t *tb = ctab_base + (int64_t)pos0 * pos_bytes;
                 kr[i].c.load(tb, k_toff[i]);
                 kr[i].s.load(tb, k_toff[i] + sin_delta);
             }
+            const uint8_t *vb = vc_base + pm.bt * vc_page_bytes;
 #pragma unroll
-            for (int i = 0; i < VI_CTX; ++i) {
-                v_lim[i] = BS;
-                vr[i] = ldg16(vc_base + page_bt(meta, v_pg[i]) * vc_page_bytes, v_goff[i]);
-            }
+            for (int i = 0; i < VI_CTX; ++i) vr[i] = ldg16(vb, (uint32_t)((lane + i * 64) * 16));
         };
-        // ---- loads of any tile: edge context tiles and new-token tiles ----
-        auto issue_loads = [&](int tile, int kind, const Meta &meta) {
-            if (kind == TILE_FULL) {
-                issue_loads_full(tile, meta);
-            } else if (kind == TILE_EDGE) {
-                issue_loads_full(tile, meta);          // pages past the context re-read the last page: harmless
+        // ---- loads of this wave's 16 keys of a new-token tile ----
+        auto issue_loads_new = [&](int tile) {
+            const int m0 = (tile - n_ctx_tiles) * NT + gw * BS;
 #pragma unroll
-                for (int i = 0; i < VI_CTX; ++i) v_lim[i] = page_lim(meta, v_pg[i]);
-#pragma unroll
-                for (int i = 0; i < KI; ++i)
-                    if (tile * PAGES + k_pg[i] >= n_pages) { kr[i].k1 = make_uint4(0, 0, 0, 0); kr[i].k2 = kr[i].k1; }
-            } else {
-                const int m0 = (tile - n_ctx_tiles) * NT;
-#pragma unroll
-                for (int i = 0; i < KI; ++i) {
-                    const int idx = lt + i * LT;
-                    const int cp = idx & 7, kl = idx >> 3, m = m0 + kl;
-                    kr[i].lds_off = (uint32_t)((kl >> 4) * K_PAGE + cp * 256 + (kl & 15) * 16);
-                    kr[i].k1 = make_uint4(0, 0, 0, 0); kr[i].k2 = kr[i].k1;
-                    kr[i].c.fill(1.f); kr[i].s.fill(0.f);
-                    if (m < t_end) {
-                        const bf16_t *kn = (const bf16_t *)p.k + (qs + m) * p.k_stride[0] + (int64_t)g * p.k_stride[1] + cp * 8;
-                        kr[i].k1 = *reinterpret_cast<const uint4 *>(kn);
-                        kr[i].k2 = *reinterpret_cast<const uint4 *>(kn + HALF);
-                        if (rot_new) {                                               // old_ops:342-343
-                            const uint8_t *tb = tab_base + (int64_t)(ctx_len + m) * row_bytes;
-                            kr[i].c.load(tb, (uint32_t)cp * 8 * TSZ);
-                            kr[i].s.load(tb, (uint32_t)cp * 8 * TSZ + HALF * TSZ);
-                        }
+            for (int i = 0; i < KI; ++i) {
+                const int idx = lane + i * 64;
+                const int cp = idx & 7, kl = idx >> 3, m = m0 + kl;
+                kr[i].lds_off = (uint32_t)(gw * K_PAGE + cp * 256 + kl * 16);
+                kr[i].k1 = make_uint4(0, 0, 0, 0); kr[i].k2 = kr[i].k1;
+                kr[i].c.fill(1.f); kr[i].s.fill(0.f);
+                if (m < t_end) {
+                    const bf16_t *kn = (const bf16_t *)p.k + (qs + m) * p.k_stride[0] + (int64_t)g * p.k_stride[1] + cp * 8;
+                    kr[i].k1 = *reinterpret_cast<const uint4 *>(kn);
+                    kr[i].k2 = *reinterpret_cast<const uint4 *>(kn + HALF);
+                    if (rot_new) {                                               // old_ops:342-343
+                        const uint8_t *tb = tab_base + (int64_t)(ctx_len + m) * row_bytes;
+                        kr[i].c.load(tb, (uint32_t)cp * 8 * TSZ);
+                        kr[i].s.load(tb, (uint32_t)cp * 8 * TSZ + HALF * TSZ);
                     }
                 }
-#pragma unroll
-                for (int i = 0; i < VI; ++i) {
-                    const int idx = lt + i * LT;
-                    const int dc = idx & 15, m = m0 + (idx >> 4);
-                    vr[i] = make_uint4(0, 0, 0, 0);
-                    if (m < t_end)
-                        vr[i] = *reinterpret_cast<const uint4 *>((const bf16_t *)p.v + (qs + m) * p.v_stride[0] +
-                                                                 (int64_t)g * p.v_stride[1] + dc * 8);
-                }
             }
+#pragma unroll
+            for (int i = 0; i < VI; ++i) {
+                const int idx = lane + i * 64;
+                const int dc = idx & 15, m = m0 + (idx >> 4);
+                vr[i] = make_uint4(0, 0, 0, 0);
+                if (m < t_end)
+                    vr[i] = *reinterpret_cast<const uint4 *>((const bf16_t *)p.v + (qs + m) * p.v_stride[0] +
+                                                             (int64_t)g * p.v_stride[1] + dc * 8);
+            }
+        };
+        // kind of this wave's part of a tile, and its loads
+        auto issue_loads = [&](int tile, const PageMeta &pm) -> int {
+            if (tile >= n_ctx_tiles) { issue_loads_new(tile); return TILE_NEW; }
+            issue_loads_ctx(tile, pm);                     // pages past the context re-read the last page: harmless
+            if (pm.lim == BS) return TILE_FULL;
+            if (tile * PAGES + gw >= n_pages) {
+#pragma unroll
+                for (int i = 0; i < KI; ++i) { kr[i].k1 = make_uint4(0, 0, 0, 0); kr[i].k2 = kr[i].k1; }
+            }
+            return TILE_EDGE;
         };
         // ---- rotate the K items in fp32 and write them to a K tile ----
         auto store_k = [&](uint8_t *ktile, int kind) {
@@ -412,15 +370,15 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                     pack_bf16(y[0], y[1]), pack_bf16(y[2], y[3]), pack_bf16(y[4], y[5]), pack_bf16(y[6], y[7]));
             }
         };
-        // ---- write the V items to a V tile ----
-        auto store_v = [&](uint8_t *vtile, int kind) {
+        // ---- write the V items to a V tile; lim = valid slots of the page ----
+        auto store_v = [&](uint8_t *vtile, int kind, int lim) {
             if (kind == TILE_NEW) {
                 // item = 8 d of one new-token key: scatter 2-byte entries
 #pragma unroll
                 for (int i = 0; i < VI; ++i) {
-                    const int idx = lt + i * LT;
-                    const int dc = idx & 15, kl = idx >> 4, slot = kl & 15;
-                    uint8_t *dst = vtile + (kl >> 4) * V_PAGE + ((slot >> 2) & 1) * V_G + (dc * 8) * 16 + (slot >> 3) * 8 +
+                    const int idx = lane + i * 64;
+                    const int dc = idx & 15, slot = idx >> 4;
+                    uint8_t *dst = vtile + gw * V_PAGE + ((slot >> 2) & 1) * V_G + (dc * 8) * 16 + (slot >> 3) * 8 +
                                    (slot & 3) * 2;
                     const uint32_t w[4] = {vr[i].x, vr[i].y, vr[i].z, vr[i].w};
 #pragma unroll
@@ -433,11 +391,10 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             }
 #pragma unroll
             for (int i = 0; i < VI_CTX; ++i) {
-                const int idx = lt + i * LT;
-                const int lim = v_lim[i];
+                const int idx = lane + i * 64;
                 if (FP8) {
                     // 16 fp8 slots of one d: entry g=0 <- slots 0-3 | 8-11, entry g=1 <- slots 4-7 | 12-15
-                    const int d = idx & 127;
+                    const int d = idx;
                     const uint32_t w[4] = {vr[i].x, vr[i].y, vr[i].z, vr[i].w};
                     uint32_t o2[4][2];
 #pragma unroll
@@ -453,14 +410,14 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                         o2[q4][0] = pack_bf16(f[0], f[1]);
                         o2[q4][1] = pack_bf16(f[2], f[3]);
                     }
-                    uint8_t *dst = vtile + v_pg[i] * V_PAGE + d * 16;
+                    uint8_t *dst = vtile + gw * V_PAGE + d * 16;
                     *reinterpret_cast<uint4 *>(dst) = make_uint4(o2[0][0], o2[0][1], o2[2][0], o2[2][1]);
                     *reinterpret_cast<uint4 *>(dst + V_G) = make_uint4(o2[1][0], o2[1][1], o2[3][0], o2[3][1]);
                 } else {
                     // 8 bf16 slots (8*hf ..) of one d: slots +0..3 -> entry g=0, +4..7 -> entry g=1, half hf
-                    const int d = (idx >> 1) & 127, hf = idx & 1;
+                    const int d = idx >> 1, hf = idx & 1;
                     uint4 v = vr[i];
-                    if (kind == TILE_EDGE && lim < BS) {
+                    if (kind == TILE_EDGE) {
                         uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
@@ -469,57 +426,55 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                         }
                         v = make_uint4(w[0], w[1], w[2], w[3]);
                     }
-                    uint8_t *dst = vtile + v_pg[i] * V_PAGE + d * 16 + hf * 8;
+                    uint8_t *dst = vtile + gw * V_PAGE + d * 16 + hf * 8;
                     *reinterpret_cast<uint2 *>(dst) = make_uint2(v.x, v.y);
                     *reinterpret_cast<uint2 *>(dst + V_G) = make_uint2(v.z, v.w);
                 }
             }
         };
+        // tile + its page limit -> LDS buffer `buf`
+        auto store_tile = [&](int buf, int kind, int lim) {
+            store_k(lds + buf * K_TILE, kind);
+            store_v(lds + 2 * K_TILE + buf * V_TILE, kind, lim);
+            if (lane == 0) page_lims[buf * PAGES + gw] = lim;
+        };
 
         // At the top of iteration `tile` the raw K/V of tile+1 sit in registers (loaded during
         // the previous iteration); they are rotated into the other LDS buffer while the
         // computing waves work on `tile`, then the loads of tile+2 are issued.
-        int nxt_kind = TILE_FULL;
-        Meta meta_pend = load_meta(tile_begin + 2);
+        int nxt_kind = TILE_FULL, nxt_lim = BS;
+        PageMeta pm_pend = load_page((tile_begin + 2) * PAGES + gw);
         if (tile_begin < tile_end) {
-            const Meta m0 = load_meta(tile_begin);
-            const Meta m1 = load_meta(tile_begin + 1);
-            const int k0 = describe(tile_begin, m0).kind;
-            issue_loads(tile_begin, k0, m0);
-            store_k(lds, k0);
-            store_v(lds + 2 * K_TILE, k0);
+            const PageMeta pm0 = load_page(tile_begin * PAGES + gw);
+            const PageMeta pm1 = load_page((tile_begin + 1) * PAGES + gw);
+            const int k0 = issue_loads(tile_begin, pm0);
+            store_tile(0, k0, pm0.lim);
             if (tile_begin + 1 < tile_end) {
-                nxt_kind = describe(tile_begin + 1, m1).kind;
-                issue_loads(tile_begin + 1, nxt_kind, m1);
+                nxt_kind = issue_loads(tile_begin + 1, pm1);
+                nxt_lim = pm1.lim;
             }
         }
         __syncthreads();
         int tile = tile_begin;
         while (tile < tile_end) {
-            // steady state: tile+1 (in registers) and tile+2 (to load) are plain context tiles
-            while (tile + 2 < tile_end && nxt_kind == TILE_FULL && describe(tile + 2, meta_pend).kind == TILE_FULL) {
+            // steady state: this wave's pages of tile+1 (in registers) and tile+2 (to load) are full context pages
+            while (tile + 2 < n_ctx_tiles && tile + 2 < tile_end && nxt_kind == TILE_FULL && pm_pend.lim == BS) {
                 const int cur = (tile - tile_begin) & 1;
-                const Meta meta_new = load_meta(tile + 3);      // scalar loads, land during the rotation
-                store_k(lds + (cur ^ 1) * K_TILE, TILE_FULL);
-                store_v(lds + 2 * K_TILE + (cur ^ 1) * V_TILE, TILE_FULL);
-                issue_loads_full(tile + 2, meta_pend);
-                meta_pend = meta_new;
+                const PageMeta pm_new = load_page((tile + 3) * PAGES + gw);      // scalar loads, land during the rotation
+                store_tile(cur ^ 1, TILE_FULL, BS);
+                issue_loads_ctx(tile + 2, pm_pend);
+                pm_pend = pm_new;
                 ++tile;
                 __syncthreads();
             }
             if (tile >= tile_end) break;
             const int cur = (tile - tile_begin) & 1;
-            if (tile + 1 < tile_end) {
-                store_k(lds + (cur ^ 1) * K_TILE, nxt_kind);
-                store_v(lds + 2 * K_TILE + (cur ^ 1) * V_TILE, nxt_kind);
-            }
+            if (tile + 1 < tile_end) store_tile(cur ^ 1, nxt_kind, nxt_lim);
             int new_kind = TILE_FULL;
-            if (tile + 2 < tile_end) {
-                new_kind = describe(tile + 2, meta_pend).kind;
-                issue_loads(tile + 2, new_kind, meta_pend);
-            }
+            if (tile + 2 < tile_end) new_kind = issue_loads(tile + 2, pm_pend);
             nxt_kind = new_kind;
-            meta_pend = load_meta(tile + 3);
+            nxt_lim = pm_pend.lim;
+            pm_pend = load_page((tile + 3) * PAGES + gw);
             ++tile;
             __syncthreads();
         }
@@ -644,15 +599,30 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         pv_half(vtile, 1, p2, p3);
     };
 
-    Meta m_cur = load_meta(tile_begin), m_nxt = load_meta(tile_begin + 1);
     __syncthreads();
     for (int tile = tile_begin; tile < tile_end; ++tile) {
         const int cur = (tile - tile_begin) & 1;
         const uint8_t *ktile = lds + cur * K_TILE;
         const uint8_t *vtile = lds + 2 * K_TILE + cur * V_TILE;
-        const TileDesc td = describe(tile, m_cur);
-        const Meta m_new = load_meta(tile + 2);
-        const int m0 = td.kind == TILE_NEW ? (tile - n_ctx_tiles) * NT : 0;
+        // which of the tile's 64 keys exist: new-token tiles from the token count, context tiles
+        // from the page limits the gathering waves left beside the tile
+        struct { int kind; uint32_t vlo, vhi; } td{TILE_FULL, ~0u, ~0u};
+        int m0 = 0;
+        if (tile >= n_ctx_tiles) {
+            td.kind = TILE_NEW;
+            m0 = (tile - n_ctx_tiles) * NT;
+            const int n = t_end - m0;
+            const uint64_t valid = n >= 64 ? ~0ull : (n <= 0 ? 0ull : ((1ull << n) - 1ull));
+            td.vlo = (uint32_t)valid; td.vhi = (uint32_t)(valid >> 32);
+        } else {
+            const int4 lims = *reinterpret_cast<const int4 *>(page_lims + cur * PAGES);
+            const int l0 = uniform(lims.x), l1 = uniform(lims.y), l2 = uniform(lims.z), l3 = uniform(lims.w);
+            if ((l0 & l1 & l2 & l3) != BS) {
+                td.kind = TILE_EDGE;
+                td.vlo = ((1u << l0) - 1u) | (((1u << l1) - 1u) << BS);
+                td.vhi = ((1u << l2) - 1u) | (((1u << l3) - 1u) << BS);
+            }
+        }
         // One call site for the tile body: the accumulators keep their registers round the loop.
         // Rows of an idle wave are all-zero queries (harmless, never stored); a new-token tile
         // entirely in this wave's future contributes nothing (causal) and is skipped.
@@ -665,8 +635,6 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             }
             attend(vtile, s0, s1);
         }
-        m_cur = m_nxt;
-        m_nxt = m_new;
         __syncthreads();
     }
 
