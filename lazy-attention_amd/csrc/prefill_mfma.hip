@@ -156,7 +156,8 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     constexpr uint32_t TSZ = sizeof(TT);
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = uniform(tid >> 6);              // in an SGPR: everything derived from it stays scalar
     const bool gatherer = wave >= NC;
 
     // ---- work item: the m-tiles of one (request, kv-head, split) land on the same XCD ----
