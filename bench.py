@@ -23,6 +23,11 @@ for _p in (ROOT, os.path.join(ROOT, "lazy-attention_amd")):
         sys.path.insert(0, _p)
 
 PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
+# HBM bytes one launch of the dominant kernel moves, from hardware counters (rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE, each scaled by what the same counter reads for a 256 MiB copy; summary under profiles/).
+# Counters cannot be read from inside this script, so the figure is the committed measurement of the
+# named workload; workloads without one report null.
+MEASURED_TRAFFIC_BYTES = {"c2_8b_bf16_10x512_q128": 49_600_000}
 PEAK_HBM_GBS = 8000.0
 
 
@@ -131,7 +136,8 @@ def main():
                    "query_tokens": int(w.max_query_len), "kv_cache": w.kv_cache_dtype,
                    "gflop_per_call": round(w.flops / 1e9, 3), "mb_per_call": round(w.bytes / 1e6, 2)},
         "roofline": {"bound": "mfma", "achieved": round(main_tflops, 2), "peak": PEAK_BF16_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(main_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "unit": "TFLOP/s", "frac": round(main_tflops / PEAK_BF16_TFLOPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(w.name), "traffic_unit": "HBM bytes per launch",
                      "kernel": "prefill_mfma_kernel", "kernel_ms": round(main_ms, 5),
                      "hbm_gbs_algorithmic": round(w.bytes / (main_ms * 1e-3) / 1e9, 1)},
     }
