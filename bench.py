@@ -73,6 +73,68 @@ def cpu_baseline(w, reps):
     return statistics.median(once() for _ in range(reps))
 
 
+def bench_decode(a):
+    """The q_len==1 path: 32 requests x 5 120 context keys, one new token each.  HBM-bound: value and
+    roofline are bytes of K/V (each read once) per second."""
+    import torch
+    from lazy_amd import _ffi, workloads as wl
+    from lazy_amd.attention import _launch
+    w = wl.decode_config()
+    g = w.to("cuda:0")
+    o = torch.zeros_like(g.q)
+
+    def plan(phases):
+        return _launch.launch_prefill(
+            q=g.q, k=g.k, v=g.v, o=o, kv_cache_dtype="auto", k_cache=g.k_cache, v_cache=g.v_cache,
+            b_loc=g.block_table, b_start_loc=g.b_start_loc, b_seq_len=g.b_seq_len, max_input_len=1,
+            max_seq_len=g.max_seq_len, k_scale=g.k_scale, v_scale=g.v_scale, alibi_slopes=None,
+            sliding_window=0, sm_scale=g.q.shape[-1] ** -0.5, skip_decode=False, cos_sin_cache=g.cos_sin_cache,
+            rotary_dim=g.q.shape[-1], is_neox_style=True, is_lazy=None, q_offset=None, q_mask=g.q_mask,
+            pos_mode=_ffi.POS_NATURAL, rotate_new_k=True, decode=True, num_splits=a.num_splits, phases=phases,
+            _return_plan=True)
+    full, main_only = plan(_ffi.PHASE_ALL), plan(_ffi.PHASE_MAIN)
+    for _ in range(a.warmup):
+        full.run()
+    torch.cuda.synchronize()
+    ms = time_calls(full, a.steps)
+    for _ in range(a.warmup):
+        main_only.run()
+    torch.cuda.synchronize()
+    main_ms = statistics.median([time_calls(main_only, max(a.steps // 4, 10)) for _ in range(7)])
+    full.run()
+    torch.cuda.synchronize()
+    gbs = w.bytes / (ms * 1e-3) / 1e9
+    main_gbs = w.bytes / (main_ms * 1e-3) / 1e9
+    out = {
+        "metric": "fused-rotary paged decode (q_len==1): K/V GB/s, 8B geometry, 32 requests x 5K context",
+        "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": w.name, "hq": 32, "hkv": 8, "head_dim": 128, "page": 16,
+                   "requests": int(w.b_seq_len.numel()), "keys_per_request": int(w.b_seq_len[0]),
+                   "mb_per_call": round(w.bytes / 1e6, 2)},
+        "roofline": {"bound": "hbm", "achieved": round(main_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(main_gbs / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(w.name),
+                     "traffic_unit": "HBM bytes per launch", "kernel": "paged_decode_kernel",
+                     "kernel_ms": round(main_ms, 5)},
+    }
+    if not a.no_cpu:
+        from oracle import deferred_rope as orc
+        torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))
+        ws = wl.decode_config(nreq=4)
+        ts = []
+        for _ in range(3):
+            t = time.perf_counter()
+            orc.paged_decode(ws.q, ws.k_cache, ws.v_cache, ws.block_table, ws.b_start_loc, ws.b_seq_len,
+                             ws.cos_sin_cache, ws.q_mask, pos_mode=orc.POS_NATURAL)
+            ts.append(time.perf_counter() - t)
+        sec = statistics.median(ts)
+        out["cpu_baseline"] = {"value": round(ws.bytes / sec / 1e9, 3), "unit": "GB/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"{ws.name}: 3 calls of 4 requests, median {sec * 1e3:.1f} ms/call"}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -81,6 +143,8 @@ def main():
     ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5])
     ap.add_argument("--num-splits", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--path", choices=["prefill", "decode"], default="prefill",
+                    help="prefill: the headline prefix-prefill call (default); decode: the q_len==1 kernel, an HBM-bound path")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a 256 MiB device-to-device copy (known traffic, for scaling profiler counters)")
     a = ap.parse_args()
@@ -96,6 +160,8 @@ def main():
         sys.exit(2)
     _ffi.lib()
     torch.cuda.set_device(0)
+    if a.path == "decode":
+        return bench_decode(a)
     w = wl.config(a.config)
     g = w.to("cuda:0")
     plan, o = make_plan(g, a.num_splits, _ffi.PHASE_ALL)

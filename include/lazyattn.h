@@ -131,6 +131,12 @@ int lazyattn_prefix_prefill(const lazyattn_prefill_params *p, void *stream);
  * skipped (old_ops/chunked_prefill_paged_decode.py:72-79). */
 int lazyattn_paged_decode_rotary(const lazyattn_prefill_params *p, void *stream);
 
+/* Bytes of workspace lazyattn_paged_decode_rotary() can use for these sizes: partials of the
+ * slices one request's pages are cut into so that few requests still fill the GPU (0 = none).
+ * Without (enough) workspace the call runs unsliced.  Pure host arithmetic; no reference
+ * counterpart (the Triton kernel is one program per (sequence, kv head)). */
+size_t lazyattn_paged_decode_workspace_bytes(const lazyattn_prefill_params *p);
+
 /* cos/sin table builder on the device: out[p, i] = cos(p*inv[i]), out[p, R/2+i] = sin(..),
  * inv = base^(-2i/R), optionally Llama-3 smoothed.  Restates
  * lazy_attn/lazy/model_executor/rope/cos_sin.py:24-66 and the third-party table layout

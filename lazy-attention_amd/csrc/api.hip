@@ -6,6 +6,9 @@ int launch_prefill_generic(const lazyattn_prefill_params &p, int decode, hipStre
 int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream);
 bool mfma_supports(const lazyattn_prefill_params &p);
 size_t mfma_workspace_bytes(const lazyattn_prefill_params &p);
+int launch_decode_mfma(const lazyattn_prefill_params &p, hipStream_t stream);
+bool decode_mfma_supports(const lazyattn_prefill_params &p);
+size_t decode_workspace_bytes(const lazyattn_prefill_params &p);
 int launch_cos_sin_table(void *out, int out_dtype, int64_t row_stride, int max_position,
                          int rotary_dim, double base, int rope_type, double factor, double low,
                          double high, int orig_max, hipStream_t stream);
@@ -80,7 +83,15 @@ extern "C" int lazyattn_paged_decode_rotary(const lazyattn_prefill_params *p, vo
     if (rc != LAZYATTN_OK) return rc;
     if (p->pos_mode == LAZYATTN_POS_OFFSET) return LAZYATTN_E_UNSUPPORTED;
     if (p->batch == 0) return LAZYATTN_OK;
+    if (p->kernel != LAZYATTN_KERNEL_GENERIC && decode_mfma_supports(*p)) return launch_decode_mfma(*p, (hipStream_t)stream);
+    if (p->kernel != LAZYATTN_KERNEL_AUTO && p->kernel != LAZYATTN_KERNEL_GENERIC) return LAZYATTN_E_UNSUPPORTED;
     return launch_prefill_generic(*p, 1, (hipStream_t)stream);
+}
+
+extern "C" size_t lazyattn_paged_decode_workspace_bytes(const lazyattn_prefill_params *p) {
+    if (!p || check_common(p, true) != LAZYATTN_OK) return 0;
+    if (p->kernel == LAZYATTN_KERNEL_GENERIC || !decode_mfma_supports(*p)) return 0;
+    return decode_workspace_bytes(*p);
 }
 
 extern "C" int lazyattn_build_cos_sin_cache(void *out, int32_t out_dtype, int64_t row_stride,

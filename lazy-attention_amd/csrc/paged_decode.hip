@@ -1,0 +1,401 @@
+// q_len == 1 rows with the rotation fused in: bf16, head_dim 128, 16-token pages, gfx950.
+//
+// Follows old_ops/chunked_prefill_paged_decode.py:23-280 (un-rotated cache, key n rotated
+// at position n) and ops/models/llama_v1.py:18-637 (block-uniform rotation by q_offset-1,
+// un-rotated branch for is_lazy == 0).  Every key, the new token included, is read from the
+// paged cache (backends/triton_attn.py:100-109 writes it there before the call).
+//
+// The work is HBM-bound (each K/V byte is used by `group` query rows only), so the kernel is
+// built around plain streaming: one wave owns one (request, kv head, slice of the pages) and
+// walks its pages two at a time, entirely in registers -- no LDS, no barrier:
+//   * a K page [D/8][16][8] is read with one 16-byte load per (token, 8-d chunk); lane
+//     (token t = lane % 16, chunk group = lane / 16) receives exactly the A operand of
+//     v_mfma_f32_16x16x32_bf16 for S^T = K . Q^T, and holds both halves (d, d + 64) of its
+//     rotation pairs, so the rotation happens in place;
+//   * the query heads of the group are the 16 columns of the MFMA (heads beyond the group are
+//     zero columns): the matrix pipe is mostly idle here and that is fine;
+//   * S^T comes out as (4 tokens per lane) x (head = lane % 16): each lane runs the online
+//     softmax of one head, lanes 16 apart share a head and exchange the row max;
+//   * P^T (two pages = 32 tokens) is the B operand of O^T += V^T . P^T as it stands if the
+//     contraction index is ordered (page X tokens 4g..4g+3 | page Y tokens 4g..4g+3) per lane
+//     group g, which is how the V rows [D][16] are read: 8 bytes per page, row and lane.
+// Slices of one request are merged by paged_decode_merge_kernel.
+#include "common.hpp"
+
+namespace lazyattn {
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+
+constexpr int D = 128;
+constexpr int HALF = 64;
+constexpr int BS = 16;
+constexpr int WAVES = 4;            // independent waves per workgroup
+
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+    f32x2_t f = {a, b};
+    bf16x2_t h = __builtin_convertvector(f, bf16x2_t);   // v_cvt_pk_bf16_f32, RNE
+    return *reinterpret_cast<uint32_t *>(&h);
+}
+__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
+__device__ __forceinline__ void unpack8(const uint4 &w, float *f) {
+    f[0] = bf16_lo(w.x); f[1] = bf16_hi(w.x); f[2] = bf16_lo(w.y); f[3] = bf16_hi(w.y);
+    f[4] = bf16_lo(w.z); f[5] = bf16_hi(w.z); f[6] = bf16_lo(w.w); f[7] = bf16_hi(w.w);
+}
+
+// 8 consecutive cos (or sin) entries of one table row
+template <typename TT> struct Tab8;
+template <> struct Tab8<bf16_t> {
+    uint4 v;
+    __device__ __forceinline__ void load(const uint8_t *row, int elem) { v = *reinterpret_cast<const uint4 *>(row + elem * 2); }
+    __device__ __forceinline__ void get(float *f) const { unpack8(v, f); }
+};
+template <> struct Tab8<float> {
+    float4 a, b;
+    __device__ __forceinline__ void load(const uint8_t *row, int elem) {
+        a = *reinterpret_cast<const float4 *>(row + elem * 4);
+        b = *reinterpret_cast<const float4 *>(row + elem * 4 + 16);
+    }
+    __device__ __forceinline__ void get(float *f) const {
+        f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+    }
+};
+
+// what one page contributes, as loaded: the key side and the value side travel separately
+template <typename TT> struct KeyRegs {
+    uint4 k[4];                 // chunks grp, 4 + grp, 8 + grp, 12 + grp of token t
+    Tab8<TT> c0, s0, c1, s1;    // cos / sin for d = 8 grp .. (pair k[0], k[2]) and d = 32 + 8 grp .. (pair k[1], k[3])
+    int lim;                    // valid slots
+};
+struct ValRegs {
+    uint2 v[8];                 // V[d = 16 blk + t][tokens 4 grp .. 4 grp + 3]
+};
+
+}  // namespace
+
+template <typename TT>
+__global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2)))
+paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
+    constexpr int TSZ = sizeof(TT);
+    const int lane = threadIdx.x & 63;
+    const int wave = uniform(threadIdx.x >> 6);
+    const int W = blockIdx.x * WAVES + wave;
+    if (W >= p.batch * p.num_kv_heads * nsplit) return;
+    // kv heads vary fastest: the waves of a workgroup walk the same pages, whose heads are
+    // adjacent 4 KB pieces of one cache block
+    const int g = W % p.num_kv_heads;
+    const int split = (W / p.num_kv_heads) % nsplit;
+    const int b = W / (nsplit * p.num_kv_heads);
+    const int group = p.num_q_heads / p.num_kv_heads;
+
+    const int64_t qs = load_index(p.b_start_loc, b, p.index_bits);
+    const int q_len = (int)(load_index(p.b_start_loc, b + 1, p.index_bits) - qs);
+    if (q_len != 1) return;                                      // old_ops/chunked_prefill_paged_decode.py:72-79
+    const int seq_len = (int)load_index(p.b_seq_len, b, p.index_bits);
+    const bool lazy_b = p.is_lazy ? p.is_lazy[b] != 0 : true;
+    const bool vanilla = p.pos_mode == LAZYATTN_POS_BLOCK_UNIFORM && !lazy_b;
+    const bool per_token = !vanilla && p.pos_mode == LAZYATTN_POS_NATURAL;
+    const bool use_qmask = !vanilla && p.q_mask != nullptr;
+    const bool use_qo = !vanilla && p.pos_mode == LAZYATTN_POS_BLOCK_UNIFORM;
+    const int n_pages = seq_len > 0 ? (seq_len + BS - 1) / BS : 0;
+    const int n_pairs = (n_pages + 1) / 2;
+    const int pair_begin = (int)((int64_t)n_pairs * split / nsplit);
+    const int pair_end = (int)((int64_t)n_pairs * (split + 1) / nsplit);
+
+    const int t = lane & 15, grp = lane >> 4;
+
+    // page metadata through the scalar unit
+    typedef const int32_t __attribute__((address_space(4))) *sptr_i32;
+    const sptr_i32 bt_row = (sptr_i32)(p.block_table + b * p.bt_stride[0]);
+    const sptr_i32 qo_row = use_qo ? (sptr_i32)(p.q_offset + b * p.qo_stride[0]) : bt_row;
+    const sptr_i32 qm_row = use_qmask ? (sptr_i32)(p.q_mask + b * p.qm_stride[0]) : bt_row;
+    const int64_t bt_s1 = p.bt_stride[1];
+    const int64_t qo_s1 = use_qo ? p.qo_stride[1] : p.bt_stride[1];
+    const int64_t qm_s1 = use_qmask ? p.qm_stride[1] : p.bt_stride[1];
+    const int qo_and = use_qo ? -1 : 0, qm_and = use_qmask ? -1 : 0;
+
+    const uint8_t *kc_base = (const uint8_t *)p.k_cache + (int64_t)g * p.kc_stride[1] * 2;
+    const uint8_t *vc_base = (const uint8_t *)p.v_cache + (int64_t)g * p.vc_stride[1] * 2;
+    const int64_t kc_page_bytes = p.kc_stride[0] * 2, vc_page_bytes = p.vc_stride[0] * 2;
+    const uint8_t *tab = (const uint8_t *)p.cos_sin_cache;
+    const int64_t row_bytes = p.table_stride * TSZ;
+    const uint32_t k_off = (uint32_t)(grp * 256 + t * 16);       // + m * 1024 for chunk 4 m + grp
+    const uint32_t v_off = (uint32_t)(t * 32 + grp * 8);         // + blk * 512 for d = 16 blk + t
+
+    auto page_block = [&](int j) -> int {
+        int jc = j < n_pages ? j : n_pages - 1;
+        jc = jc < 0 ? 0 : jc;
+        return bt_row[jc * bt_s1];
+    };
+    auto load_keys = [&](int j, KeyRegs<TT> &r) {
+        int jc = j < n_pages ? j : n_pages - 1;
+        jc = jc < 0 ? 0 : jc;
+        const int bt = bt_row[jc * bt_s1];
+        const int qo = qo_row[jc * qo_s1] & qo_and;
+        const int qm = qm_row[jc * qm_s1] & qm_and;                                  // old_ops/chunked...:165-167 analogue
+        int l = seq_len - j * BS;
+        l = l < BS - qm ? l : BS - qm;
+        l = l > BS ? BS : l;
+        r.lim = l < 0 ? 0 : l;
+        const uint8_t *kb = kc_base + bt * kc_page_bytes;
+#pragma unroll
+        for (int m = 0; m < 4; ++m) r.k[m] = *reinterpret_cast<const uint4 *>(kb + k_off + m * 1024);
+        // position of this lane's token: its index in the sequence (un-rotated cache), or one
+        // angle for the whole page (block-uniform), or row 0 = identity (un-rotated request)
+        int pos = qo ? qo - 1 : 0;                                                   // ops/models/llama_v1.py:231-262
+        if (per_token) {
+            pos = j * BS + t;                                                        // old_ops/chunked...:203-233
+            pos = pos < seq_len ? pos : seq_len - 1;     // slots past the end are masked; stay inside the table
+            pos = pos < 0 ? 0 : pos;
+        }
+        const uint8_t *row = tab + (int64_t)pos * row_bytes;
+        r.c0.load(row, 8 * grp);
+        r.s0.load(row, HALF + 8 * grp);
+        r.c1.load(row, 32 + 8 * grp);
+        r.s1.load(row, HALF + 32 + 8 * grp);
+    };
+    auto load_values = [&](int j, ValRegs &r) {
+        const uint8_t *vb = vc_base + page_block(j) * vc_page_bytes;
+#pragma unroll
+        for (int blk = 0; blk < 8; ++blk) r.v[blk] = *reinterpret_cast<const uint2 *>(vb + v_off + blk * 512);
+    };
+    // rotate the pair (lo, hi) = (d, d + 64) in fp32, one rounding to bf16
+    auto rotate = [&](const uint4 &lo, const uint4 &hi, const Tab8<TT> &c, const Tab8<TT> &s, bf16x8_t &xo, bf16x8_t &yo) {
+        float a[8], bb[8], cs[8], sn[8], x[8], y[8];
+        unpack8(lo, a);
+        unpack8(hi, bb);
+        c.get(cs);
+        s.get(sn);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            x[e] = a[e] * cs[e] - bb[e] * sn[e];
+            y[e] = a[e] * sn[e] + bb[e] * cs[e];
+        }
+        uint4 xw = make_uint4(pack_bf16(x[0], x[1]), pack_bf16(x[2], x[3]), pack_bf16(x[4], x[5]), pack_bf16(x[6], x[7]));
+        uint4 yw = make_uint4(pack_bf16(y[0], y[1]), pack_bf16(y[2], y[3]), pack_bf16(y[4], y[5]), pack_bf16(y[6], y[7]));
+        xo = *reinterpret_cast<bf16x8_t *>(&xw);
+        yo = *reinterpret_cast<bf16x8_t *>(&yw);
+    };
+
+    // Q^T: column = head = t, contraction d = 32 m + 8 grp ..
+    bf16x8_t qf[4];
+    {
+        const bool head_ok = t < group;
+        const bf16_t *qp = (const bf16_t *)p.q + qs * p.q_stride[0] + (int64_t)(g * group + (head_ok ? t : 0)) * p.q_stride[1] + 8 * grp;
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+            uint4 w = make_uint4(0, 0, 0, 0);
+            if (head_ok) w = *reinterpret_cast<const uint4 *>(qp + 32 * m);
+            qf[m] = *reinterpret_cast<bf16x8_t *>(&w);
+        }
+    }
+    const float cs2 = p.sm_scale * 1.4426950408889634f;
+    float m_run = -INFINITY, l_run = 0.f;
+    f32x4_t acc[8];
+#pragma unroll
+    for (int blk = 0; blk < 8; ++blk) acc[blk] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    // scores of one page: S^T[token 4 grp + i][head t], masked
+    auto scores = [&](const KeyRegs<TT> &r) -> f32x4_t {
+        bf16x8_t k0, k1, k2, k3;
+        rotate(r.k[0], r.k[2], r.c0, r.s0, k0, k2);
+        rotate(r.k[1], r.k[3], r.c1, r.s1, k1, k3);
+        f32x4_t s = {0.f, 0.f, 0.f, 0.f};
+        s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0, qf[0], s, 0, 0, 0);
+        s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1, qf[1], s, 0, 0, 0);
+        s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k2, qf[2], s, 0, 0, 0);
+        s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k3, qf[3], s, 0, 0, 0);
+        if (r.lim < BS) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s[i] = 4 * grp + i < r.lim ? s[i] : -INFINITY;
+        }
+        return s;
+    };
+    // V words of a page with the masked tokens zeroed (a masked slot may hold anything)
+    auto masked_v = [&](const ValRegs &r, int lim, int blk) -> uint2 {
+        uint2 w = r.v[blk];
+        if (lim < BS) {
+            if (4 * grp + 0 >= lim) w.x &= 0xffff0000u;
+            if (4 * grp + 1 >= lim) w.x &= 0x0000ffffu;
+            if (4 * grp + 2 >= lim) w.y &= 0xffff0000u;
+            if (4 * grp + 3 >= lim) w.y &= 0x0000ffffu;
+        }
+        return w;
+    };
+
+    // The key side of pair i+1 is requested as soon as the scores of pair i have consumed the
+    // registers it lands in, the value side of pair i at the top of its iteration: every load has
+    // about half an iteration of other work between issue and use, at no extra registers.
+    KeyRegs<TT> KX, KY;
+    if (pair_begin < pair_end) {
+        load_keys(2 * pair_begin, KX);
+        load_keys(2 * pair_begin + 1, KY);
+    }
+    for (int pr = pair_begin; pr < pair_end; ++pr) {
+        ValRegs X, Y;
+        load_values(2 * pr, X);
+        load_values(2 * pr + 1, Y);
+        const f32x4_t sx = scores(KX), sy = scores(KY);
+        const int lim_x = KX.lim, lim_y = KY.lim;
+        if (pr + 1 < pair_end) {
+            load_keys(2 * pr + 2, KX);
+            load_keys(2 * pr + 3, KY);
+        }
+        // online softmax of head t over the 32 tokens; lanes t, t+16, t+32, t+48 share the head
+        float mx = fmaxf(fmaxf(fmaxf(sx[0], sx[1]), fmaxf(sx[2], sx[3])), fmaxf(fmaxf(sy[0], sy[1]), fmaxf(sy[2], sy[3])));
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run, mx);
+        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f((m_run - m_safe) * cs2);
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
+#pragma unroll
+            for (int blk = 0; blk < 8; ++blk) acc[blk] *= alpha;
+            l_run *= alpha;
+        }
+        m_run = m_new;
+        const float mc = m_safe * cs2;
+        float px[4], py[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            px[i] = __builtin_amdgcn_exp2f(fmaf(sx[i], cs2, -mc));
+            py[i] = __builtin_amdgcn_exp2f(fmaf(sy[i], cs2, -mc));
+        }
+        l_run += (px[0] + px[1]) + (px[2] + px[3]) + (py[0] + py[1]) + (py[2] + py[3]);
+        uint4 pw = make_uint4(pack_bf16(px[0], px[1]), pack_bf16(px[2], px[3]), pack_bf16(py[0], py[1]), pack_bf16(py[2], py[3]));
+        const bf16x8_t pf = *reinterpret_cast<bf16x8_t *>(&pw);
+#pragma unroll
+        for (int blk = 0; blk < 8; ++blk) {
+            const uint2 vx = masked_v(X, lim_x, blk), vy = masked_v(Y, lim_y, blk);
+            uint4 vw = make_uint4(vx.x, vx.y, vy.x, vy.y);
+            acc[blk] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<bf16x8_t *>(&vw), pf, acc[blk], 0, 0, 0);
+        }
+    }
+
+    // ---- epilogue: lane (head t, grp) holds O^T[d = 16 blk + 4 grp + i][head t] ----
+    l_run += __shfl_xor(l_run, 16);
+    l_run += __shfl_xor(l_run, 32);
+    if (t >= group) return;
+    const int h = g * group + t;
+    const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+    if (nsplit == 1) {
+        bf16_t *op = (bf16_t *)p.o + qs * p.o_stride[0] + (int64_t)h * p.o_stride[1] + 4 * grp;
+#pragma unroll
+        for (int blk = 0; blk < 8; ++blk)
+            *reinterpret_cast<uint2 *>(op + 16 * blk) =
+                make_uint2(pack_bf16(acc[blk][0] * inv, acc[blk][1] * inv), pack_bf16(acc[blk][2] * inv, acc[blk][3] * inv));
+        return;
+    }
+    // partial of this slice: normalised O and log2-sum-exp, indexed by (slice, request, head)
+    float *wo = (float *)p.workspace;
+    float *wl = wo + (int64_t)nsplit * p.batch * p.num_q_heads * D;
+    const int64_t r_idx = ((int64_t)split * p.batch + b) * p.num_q_heads + h;
+#pragma unroll
+    for (int blk = 0; blk < 8; ++blk)
+        *reinterpret_cast<float4 *>(wo + r_idx * D + 16 * blk + 4 * grp) =
+            make_float4(acc[blk][0] * inv, acc[blk][1] * inv, acc[blk][2] * inv, acc[blk][3] * inv);
+    if (grp == 0) wl[r_idx] = l_run > 0.f ? m_run * cs2 + __builtin_amdgcn_logf(l_run) : -INFINITY;
+}
+
+// merge of the slices: one 32-lane group per (request, q head)
+__global__ void __launch_bounds__(256)
+paged_decode_merge_kernel(const lazyattn_prefill_params p, const int nsplit) {
+    const int64_t r = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);
+    if (r >= (int64_t)p.batch * p.num_q_heads) return;
+    const int b = (int)(r / p.num_q_heads), h = (int)(r % p.num_q_heads);
+    const int64_t qs = load_index(p.b_start_loc, b, p.index_bits);
+    if (load_index(p.b_start_loc, b + 1, p.index_bits) - qs != 1) return;
+    const int d = (threadIdx.x & 31) * 4;
+    const float *wo = (const float *)p.workspace;
+    const float *wl = wo + (int64_t)nsplit * p.batch * p.num_q_heads * D;
+    const int64_t rows = (int64_t)p.batch * p.num_q_heads;
+    float mx = -INFINITY;
+    for (int s = 0; s < nsplit; ++s) mx = fmaxf(mx, wl[s * rows + r]);
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    float wsum = 0.f;
+    if (mx != -INFINITY) {
+        for (int s = 0; s < nsplit; ++s) {
+            const int64_t ri = s * rows + r;
+            const float w = __builtin_amdgcn_exp2f(wl[ri] - mx);
+            const float4 v = *reinterpret_cast<const float4 *>(wo + ri * D + d);
+            o.x = fmaf(w, v.x, o.x); o.y = fmaf(w, v.y, o.y); o.z = fmaf(w, v.z, o.z); o.w = fmaf(w, v.w, o.w);
+            wsum += w;
+        }
+    }
+    const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
+    bf16_t *op = (bf16_t *)p.o + qs * p.o_stride[0] + (int64_t)h * p.o_stride[1] + d;
+    *reinterpret_cast<uint2 *>(op) = make_uint2(pack_bf16(o.x * inv, o.y * inv), pack_bf16(o.z * inv, o.w * inv));
+}
+
+// ------------------------------------------------------------------ host side
+bool decode_mfma_supports(const lazyattn_prefill_params &p) {
+    if (p.dtype != LAZYATTN_BF16 || p.cache_dtype != LAZYATTN_BF16) return false;
+    if (p.table_dtype != LAZYATTN_BF16 && p.table_dtype != LAZYATTN_F32) return false;
+    if (p.head_dim != D || p.block_size != BS || p.x != 8) return false;
+    if (p.sliding_window > 0) return false;
+    if (p.pos_mode != LAZYATTN_POS_NATURAL && p.pos_mode != LAZYATTN_POS_BLOCK_UNIFORM) return false;
+    if (p.num_q_heads / p.num_kv_heads > 16) return false;
+    if (p.q_stride[2] != 1 || p.o_stride[2] != 1) return false;
+    if (p.kc_stride[4] != 1 || p.kc_stride[3] != p.x || p.kc_stride[2] != (int64_t)BS * p.x) return false;
+    if (p.vc_stride[3] != 1 || p.vc_stride[2] != BS) return false;
+    const int64_t al[] = {p.q_stride[0], p.q_stride[1], p.o_stride[0], p.o_stride[1], p.kc_stride[0], p.kc_stride[1],
+                          p.vc_stride[0], p.vc_stride[1], p.table_stride};
+    for (int64_t s : al)
+        if (s % 8) return false;                       // 16-byte rows
+    const void *ptrs[] = {p.q, p.o, p.k_cache, p.v_cache, p.cos_sin_cache};
+    for (const void *q : ptrs)
+        if (((uintptr_t)q) & 15) return false;
+    return true;
+}
+
+// slices of the page axis per (request, kv head): enough waves to fill the chip, at least four
+// pages per slice
+static int decode_splits(const lazyattn_prefill_params &p) {
+    if (p.num_splits > 0) return p.num_splits > 64 ? 64 : p.num_splits;
+    const int64_t natural = (int64_t)p.batch * p.num_kv_heads;
+    if (natural <= 0) return 1;
+    int64_t s = (256 * 8 + natural - 1) / natural;
+    const int64_t pages = p.max_seq_len > 0 ? (p.max_seq_len + BS - 1) / BS : 64;
+    if (s > pages / 4) s = pages / 4;
+    if (s > 64) s = 64;
+    return s < 1 ? 1 : (int)s;
+}
+
+size_t decode_workspace_bytes(const lazyattn_prefill_params &p) {
+    const int ns = decode_splits(p);
+    if (ns <= 1) return 0;
+    return (size_t)ns * (size_t)p.batch * p.num_q_heads * (D + 1) * sizeof(float);
+}
+
+int launch_decode_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
+    int nsplit = decode_splits(p);
+    if (nsplit > 1) {
+        // without room for the partials the call still runs, one slice per request and kv head
+        const size_t need = (size_t)nsplit * (size_t)p.batch * p.num_q_heads * (D + 1) * sizeof(float);
+        if (!p.workspace || (size_t)p.workspace_bytes < need || (((uintptr_t)p.workspace) & 15)) nsplit = 1;
+    }
+    const int phases = p.phases ? p.phases : LAZYATTN_PHASE_ALL;
+    const int64_t waves = (int64_t)p.batch * p.num_kv_heads * nsplit;
+    const unsigned nblocks = (unsigned)((waves + WAVES - 1) / WAVES);
+    if (phases & LAZYATTN_PHASE_MAIN) {
+        if (p.table_dtype == LAZYATTN_F32)
+            hipLaunchKernelGGL(paged_decode_kernel<float>, dim3(nblocks), dim3(WAVES * 64), 0, stream, p, nsplit);
+        else
+            hipLaunchKernelGGL(paged_decode_kernel<bf16_t>, dim3(nblocks), dim3(WAVES * 64), 0, stream, p, nsplit);
+        if (hipGetLastError() != hipSuccess) return LAZYATTN_E_LAUNCH;
+    }
+    if (nsplit > 1 && (phases & LAZYATTN_PHASE_COMBINE)) {
+        const int64_t rows = (int64_t)p.batch * p.num_q_heads;
+        hipLaunchKernelGGL(paged_decode_merge_kernel, dim3((unsigned)((rows + 7) / 8)), dim3(256), 0, stream, p, nsplit);
+        if (hipGetLastError() != hipSuccess) return LAZYATTN_E_LAUNCH;
+    }
+    return LAZYATTN_OK;
+}
+
+}  // namespace lazyattn

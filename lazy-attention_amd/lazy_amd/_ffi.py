@@ -20,7 +20,7 @@ KERNEL_AUTO, KERNEL_GENERIC, KERNEL_MFMA, KERNEL_MFMA4, KERNEL_MFMA8 = 0, 1, 2, 
 PHASE_MAIN, PHASE_COMBINE, PHASE_ALL = 1, 2, 3
 
 ERRORS = {-1: "NULL", -2: "SHAPE", -3: "DTYPE", -4: "UNSUPPORTED", -5: "WORKSPACE", -6: "LAUNCH"}
-EXPORTS = ("lazyattn_prefill_workspace_bytes", "lazyattn_prefix_prefill",
+EXPORTS = ("lazyattn_prefill_workspace_bytes", "lazyattn_prefix_prefill", "lazyattn_paged_decode_workspace_bytes",
            "lazyattn_paged_decode_rotary", "lazyattn_build_cos_sin_cache",
            "lazyattn_pack_cos_sin_cache",
            "lazyattn_error_string", "lazyattn_abi_version")
@@ -59,6 +59,8 @@ def lib() -> C.CDLL:
         L = C.CDLL(_LIB_PATH)
         L.lazyattn_prefill_workspace_bytes.restype = C.c_size_t
         L.lazyattn_prefill_workspace_bytes.argtypes = [C.POINTER(PrefillParams)]
+        L.lazyattn_paged_decode_workspace_bytes.restype = C.c_size_t
+        L.lazyattn_paged_decode_workspace_bytes.argtypes = [C.POINTER(PrefillParams)]
         for name in ("lazyattn_prefix_prefill", "lazyattn_paged_decode_rotary"):
             fn = getattr(L, name)
             fn.restype = C.c_int

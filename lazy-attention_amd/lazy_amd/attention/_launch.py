@@ -114,12 +114,12 @@ class PrefillPlan:
         self.params, self.device, self.decode, self._keep = params, device, decode, keep
         self._lib = _ffi.lib()
         self._ws = None
-        if not decode:
-            nbytes = self._lib.lazyattn_prefill_workspace_bytes(params)
-            self._ws = _ffi.workspace(device, nbytes)
-            if self._ws is not None:
-                params.workspace = self._ws.data_ptr()
-                params.workspace_bytes = self._ws.numel()
+        nbytes = (self._lib.lazyattn_paged_decode_workspace_bytes(params) if decode
+                  else self._lib.lazyattn_prefill_workspace_bytes(params))
+        self._ws = _ffi.workspace(device, nbytes)
+        if self._ws is not None:
+            params.workspace = self._ws.data_ptr()
+            params.workspace_bytes = self._ws.numel()
 
     def run(self) -> None:
         stream = torch.cuda.current_stream(self.device).cuda_stream

@@ -36,7 +36,7 @@ def chunked_prefill_paged_decode(query, key, value, output, kv_cache_dtype, key_
     _launch.launch_prefill(
         q=query, k=key, v=value, o=output, kv_cache_dtype=kv_cache_dtype, k_cache=key_cache,
         v_cache=value_cache, b_loc=block_table, b_start_loc=query_start_loc, b_seq_len=seq_lens,
-        max_input_len=1, k_scale=k_scale, v_scale=v_scale, alibi_slopes=alibi_slopes,
+        max_input_len=1, max_seq_len=max_seq_len, k_scale=k_scale, v_scale=v_scale, alibi_slopes=alibi_slopes,
         sliding_window=sliding_window, sm_scale=sm_scale, skip_decode=False,
         cos_sin_cache=cos_sin_cache, rotary_dim=rotary_dim, is_neox_style=is_neox_style,
         is_lazy=None, q_offset=None, q_mask=q_mask, pos_mode=_ffi.POS_NATURAL, rotate_new_k=True,

@@ -282,3 +282,28 @@ def config(index: int, *, variant: str = "natural", keep_aux: bool = False,
                              q_lens=[128] * nreq, variant=variant, kv_cache_dtype="fp8",
                              seed=seed, keep_aux=keep_aux)
     raise ValueError(f"no such config: {index}")
+
+
+def decode_config(*, variant: str = "natural", nreq: int = 32, ndoc: int = 20, doc_len: int = 256) -> Workload:
+    """q_len == 1 batch for the fused-rotary decode kernel: ``nreq`` requests, each over its own
+    ``ndoc`` documents of ``doc_len`` tokens in shuffled slot order (no sharing between requests, so
+    every K/V byte comes from HBM once), Llama-3-8B geometry, bf16.  The new token of every request is
+    already in the paged cache, as the attention backend leaves it (backends/triton_attn.py:100-109)."""
+    seed = 2000 + nreq
+    g = torch.Generator().manual_seed(seed)
+    reqs = [[b * ndoc + i for i in torch.randperm(ndoc, generator=g).tolist()] for b in range(nreq)]
+    w = make_workload(f"d1_8b_bf16_decode_{nreq}req_{ndoc}x{doc_len}", dtype=torch.bfloat16, **LLAMA_8B,
+                      block_size=16, doc_lens=[doc_len] * (nreq * ndoc), requests=reqs, q_lens=[1] * nreq,
+                      variant=variant, seed=seed)
+    hkv, d = LLAMA_8B["hkv"], LLAMA_8B["d"]
+    x = w.k_cache.shape[4]
+    bs = w.v_cache.shape[3]
+    for b in range(nreq):
+        qs = int(w.b_start_loc[b]); n = int(w.b_seq_len[b]) - 1
+        pb = int(w.block_table[b, n // bs])
+        w.k_cache[pb, :, :, n % bs, :] = w.k[qs].view(hkv, d // x, x)
+        w.v_cache[pb, :, :, n % bs] = w.v[qs]
+    keys = int(w.b_seq_len.sum())
+    w.bytes = float(keys * hkv * d * 2 * 2 + 2 * w.q.numel() * 2)      # K + V once, Q in, O out
+    w.flops = float(4 * LLAMA_8B["hq"] * d * keys)
+    return w

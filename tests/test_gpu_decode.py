@@ -1,0 +1,156 @@
+"""GPU parity of the q_len==1 kernel with the rotation fused in (``lazyattn_paged_decode_rotary``,
+reached through ``chunked_prefill_paged_decode`` of both variants) against the CPU oracle.
+
+Shapes follow the reference's own decode callers: every key, the new token included, is in the
+paged cache when the call is made (``backends/triton_attn.py:100-109``)."""
+import pytest
+import torch
+
+from oracle import deferred_rope as orc
+from lazy_amd import _ffi, workloads as wl
+from lazy_amd.attention import _launch
+from lazy_amd.attention.old_ops.chunked_prefill_paged_decode import chunked_prefill_paged_decode as entry_unrotated
+from lazy_amd.attention.ops.chunked_prefill_paged_decode import chunked_prefill_paged_decode as entry_block_uniform
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _decode_batch(variant, *, hq=8, hkv=2, q_lens=(1, 1, 1, 1, 1), table_f32=False, seed=77):
+    """Ragged documents (pads at document ends), requests of 1 to 9 documents, one new token each
+    (or more: such requests must be skipped)."""
+    d = 128
+    w = wl.make_workload("decode", dtype=torch.bfloat16, hq=hq, hkv=hkv, d=d, theta=500000.0, block_size=16,
+                         doc_lens=[40, 16, 33, 70, 5, 128, 97],
+                         requests=[[3, 1, 0], [2], [0, 2, 3, 1, 5, 6, 4, 5, 6], [4, 0], [6, 5, 3]],
+                         q_lens=list(q_lens), variant=variant, seed=seed)
+    if table_f32:
+        w.cos_sin_cache = w.cos_sin_cache.float()
+    x = w.k_cache.shape[4]
+    for b in range(len(q_lens)):
+        qs, qe = int(w.b_start_loc[b]), int(w.b_start_loc[b + 1])
+        ctx = int(w.b_seq_len[b]) - (qe - qs)
+        for t in range(qe - qs):
+            n = ctx + t
+            pb = int(w.block_table[b, n // 16]); o_ = n % 16
+            w.k_cache[pb, :, :, o_, :] = w.k[qs + t].view(hkv, d // x, x)
+            w.v_cache[pb, :, :, o_] = w.v[qs + t]
+    return w
+
+
+def _oracle(w, lazy=None):
+    ref = torch.full_like(w.q, 5.0)
+    orc.paged_decode(w.q, w.k_cache, w.v_cache, w.block_table, w.b_start_loc, w.b_seq_len,
+                     w.cos_sin_cache, w.q_mask, q_offset=w.q_offset, is_lazy=lazy,
+                     pos_mode=orc.POS_NATURAL if w.pos_mode != orc.POS_BLOCK_UNIFORM else w.pos_mode, out=ref)
+    return ref
+
+
+def _run(w, *, lazy=None, num_splits=0, kernel=_ffi.KERNEL_AUTO):
+    """The q_len==1 launch the entry points make, with the slicing and kernel choice exposed."""
+    g = w.to(DEV)
+    out = torch.full_like(g.q, 5.0)
+    bu = w.pos_mode == orc.POS_BLOCK_UNIFORM
+    _launch.launch_prefill(
+        q=g.q, k=g.k, v=g.v, o=out, kv_cache_dtype="auto", k_cache=g.k_cache, v_cache=g.v_cache,
+        b_loc=g.block_table, b_start_loc=g.b_start_loc, b_seq_len=g.b_seq_len, max_input_len=1,
+        max_seq_len=g.max_seq_len, k_scale=g.k_scale, v_scale=g.v_scale, alibi_slopes=None, sliding_window=0,
+        sm_scale=128 ** -0.5, skip_decode=False, cos_sin_cache=g.cos_sin_cache, rotary_dim=128,
+        is_neox_style=True, is_lazy=None if lazy is None else lazy.to(DEV),
+        q_offset=g.q_offset if bu else None, q_mask=g.q_mask,
+        pos_mode=_ffi.POS_BLOCK_UNIFORM if bu else _ffi.POS_NATURAL, rotate_new_k=not bu, decode=True,
+        kernel=kernel, num_splits=num_splits)
+    return out.cpu()
+
+
+def _err(a, b):
+    return (a.float() - b.float()).abs().max().item()
+
+
+@pytest.mark.parametrize("variant", ["natural", "block_uniform"])
+@pytest.mark.parametrize("nsplit", [0, 1, 3, 7])
+def test_decode_ragged(variant, nsplit):
+    print(f"case: decode ragged {variant} nsplit={nsplit}", flush=True)
+    w = _decode_batch(variant)
+    ref = _oracle(w)
+    got = _run(w, num_splits=nsplit)
+    assert _err(got, ref) < 2e-2, _err(got, ref)
+
+
+def test_decode_matches_generic_kernel():
+    print("case: decode fast vs generic kernel", flush=True)
+    w = _decode_batch("natural")
+    a = _run(w, num_splits=2)
+    b = _run(w, kernel=_ffi.KERNEL_GENERIC)
+    assert _err(a, b) < 2e-2, _err(a, b)
+
+
+def test_decode_skips_longer_requests_and_leaves_their_rows():
+    print("case: decode skips q_len>1", flush=True)
+    w = _decode_batch("natural", q_lens=(1, 4, 1, 2, 1))
+    ref = _oracle(w)
+    got = _run(w, num_splits=3)
+    assert _err(got, ref) < 2e-2, _err(got, ref)
+    qs = int(w.b_start_loc[1])
+    assert torch.all(got[qs:qs + 4] == 5.0)                      # old_ops/chunked_prefill_paged_decode.py:72-79
+
+
+def test_decode_vanilla_requests_and_fp32_table():
+    print("case: decode is_lazy mix, fp32 table", flush=True)
+    w = _decode_batch("block_uniform", table_f32=True)
+    lazy = torch.tensor([True, False, True, False, True])
+    ref = _oracle(w, lazy)
+    got = _run(w, lazy=lazy, num_splits=2)
+    assert _err(got, ref) < 2e-2, _err(got, ref)
+
+
+@pytest.mark.parametrize("hq,hkv", [(4, 4), (16, 2), (32, 2)])
+def test_decode_group_sizes(hq, hkv):
+    print(f"case: decode group {hq // hkv}", flush=True)
+    w = _decode_batch("natural", hq=hq, hkv=hkv)
+    ref = _oracle(w)
+    got = _run(w)
+    assert _err(got, ref) < 2e-2, _err(got, ref)
+
+
+def test_decode_pad_slots_may_hold_nan():
+    print("case: decode NaN pad", flush=True)
+    w = _decode_batch("natural")
+    ref = _oracle(w)
+    for b in range(5):
+        for j in range(w.block_table.shape[1]):
+            m = int(w.q_mask[b, j])
+            if m:
+                pb = int(w.block_table[b, j])
+                w.k_cache[pb, :, :, 16 - m:, :] = float("nan")
+                w.v_cache[pb, :, :, 16 - m:] = float("nan")
+    got = _run(w, num_splits=2)
+    assert _err(got, ref) < 2e-2, _err(got, ref)
+
+
+def test_decode_entry_points_long_context():
+    """Both entry points at a serving-like size: 8 requests x 2 K keys, Llama-3-8B geometry."""
+    print("case: decode entry points 8 x 2K", flush=True)
+    g0 = torch.Generator().manual_seed(3)
+    for variant, entry in (("natural", entry_unrotated), ("block_uniform", entry_block_uniform)):
+        reqs = [torch.randperm(16, generator=g0)[:8].tolist() for _ in range(8)]
+        w = wl.make_workload("dec8", dtype=torch.bfloat16, **wl.LLAMA_8B, block_size=16, doc_lens=[250] * 16,
+                             requests=reqs, q_lens=[1] * 8, variant=variant, seed=9)
+        x = w.k_cache.shape[4]
+        for b in range(8):
+            qs = int(w.b_start_loc[b]); n = int(w.b_seq_len[b]) - 1
+            pb = int(w.block_table[b, n // 16])
+            w.k_cache[pb, :, :, n % 16, :] = w.k[qs].view(8, 128 // x, x)
+            w.v_cache[pb, :, :, n % 16] = w.v[qs]
+        ref = _oracle(w)
+        g = w.to(DEV)
+        out = torch.full_like(g.q, 5.0)
+        if variant == "natural":
+            entry(g.q, g.k, g.v, out, "auto", g.k_cache, g.v_cache, g.block_table, g.b_start_loc, g.b_seq_len,
+                  g.max_seq_len, 1, g.k_scale, g.v_scale, sm_scale=128 ** -0.5, rotary_dim=128,
+                  cos_sin_cache=g.cos_sin_cache, q_mask=g.q_mask)
+        else:
+            entry(g.q, g.k, g.v, out, "auto", g.k_cache, g.v_cache, g.block_table, g.b_start_loc, g.b_seq_len,
+                  g.max_seq_len, 1, g.k_scale, g.v_scale, sm_scale=128 ** -0.5, rotary_dim=128,
+                  cos_sin_cache=g.cos_sin_cache, is_lazy=g.is_lazy, q_offset=g.q_offset, q_mask=g.q_mask)
+        assert _err(out.cpu(), ref) < 2e-2, (variant, _err(out.cpu(), ref))
