@@ -1,4 +1,4 @@
-// q_len == 1 rows with the rotation fused in: bf16, head_dim 128, 16-token pages, gfx950.
+// q_len == 1 rows with the rotation fused in: bf16 (cache bf16 or fp8 e4m3), head_dim 128, 16-token pages, gfx950.
 //
 // Follows old_ops/chunked_prefill_paged_decode.py:23-280 (un-rotated cache, key n rotated
 // at position n) and ops/models/llama_v1.py:18-637 (block-uniform rotation by q_offset-1,
@@ -19,6 +19,8 @@
 //   * P^T (two pages = 32 tokens) is the B operand of O^T += V^T . P^T as it stands if the
 //     contraction index is ordered (page X tokens 4g..4g+3 | page Y tokens 4g..4g+3) per lane
 //     group g, which is how the V rows [D][16] are read: 8 bytes per page, row and lane.
+// fp8 e4m3 pages ([D/16][16][16] and [D][16] bytes) are read with 8- and 4-byte loads at the same lane mapping,
+// converted, scaled and rounded to bf16 (old_ops/prefix_prefill.py:239-241 arithmetic), then treated alike.
 // Slices of one request are merged by paged_decode_merge_kernel.
 #include "common.hpp"
 
@@ -47,6 +49,15 @@ __device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirs
 __device__ __forceinline__ void unpack8(const uint4 &w, float *f) {
     f[0] = bf16_lo(w.x); f[1] = bf16_hi(w.x); f[2] = bf16_lo(w.y); f[3] = bf16_hi(w.y);
     f[4] = bf16_lo(w.z); f[5] = bf16_hi(w.z); f[6] = bf16_lo(w.w); f[7] = bf16_hi(w.w);
+}
+
+// 8 fp8 e4m3 bytes -> (float * scale) rounded to bf16, as floats
+__device__ __forceinline__ void unpack8_fp8(uint32_t lo, uint32_t hi, float scale, float *f) {
+    const f32x2_t a = __builtin_amdgcn_cvt_pk_f32_fp8(lo, false), b = __builtin_amdgcn_cvt_pk_f32_fp8(lo >> 16, false);
+    const f32x2_t c = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false), d = __builtin_amdgcn_cvt_pk_f32_fp8(hi >> 16, false);
+    const float t[8] = {a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = round_to<bf16_t>(t[i] * scale);
 }
 
 // 8 consecutive cos (or sin) entries of one table row
@@ -79,7 +90,7 @@ struct ValRegs {
 
 }  // namespace
 
-template <typename TT>
+template <typename TT, bool FP8>
 __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2)))
 paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     constexpr int TSZ = sizeof(TT);
@@ -120,13 +131,20 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     const int64_t qm_s1 = use_qmask ? p.qm_stride[1] : p.bt_stride[1];
     const int qo_and = use_qo ? -1 : 0, qm_and = use_qmask ? -1 : 0;
 
-    const uint8_t *kc_base = (const uint8_t *)p.k_cache + (int64_t)g * p.kc_stride[1] * 2;
-    const uint8_t *vc_base = (const uint8_t *)p.v_cache + (int64_t)g * p.vc_stride[1] * 2;
-    const int64_t kc_page_bytes = p.kc_stride[0] * 2, vc_page_bytes = p.vc_stride[0] * 2;
+    constexpr int CSZ = FP8 ? 1 : 2;                             // bytes per cache element
+    const uint8_t *kc_base = (const uint8_t *)p.k_cache + (int64_t)g * p.kc_stride[1] * CSZ;
+    const uint8_t *vc_base = (const uint8_t *)p.v_cache + (int64_t)g * p.vc_stride[1] * CSZ;
+    const int64_t kc_page_bytes = p.kc_stride[0] * CSZ, vc_page_bytes = p.vc_stride[0] * CSZ;
+    const float k_scale = FP8 ? *p.k_scale : 1.f, v_scale = FP8 ? *p.v_scale : 1.f;
     const uint8_t *tab = (const uint8_t *)p.cos_sin_cache;
     const int64_t row_bytes = p.table_stride * TSZ;
-    const uint32_t k_off = (uint32_t)(grp * 256 + t * 16);       // + m * 1024 for chunk 4 m + grp
-    const uint32_t v_off = (uint32_t)(t * 32 + grp * 8);         // + blk * 512 for d = 16 blk + t
+    // bf16: chunk 4 m + grp of token t at (4 m + grp) * 256 + t * 16, 16 bytes
+    // fp8 : the same 8 d are half (grp & 1) of 16-d chunk 2 m + grp / 2: (2 m + grp / 2) * 256 + t * 16 + (grp & 1) * 8
+    const uint32_t k_off = FP8 ? (uint32_t)((grp >> 1) * 256 + t * 16 + (grp & 1) * 8) : (uint32_t)(grp * 256 + t * 16);
+    constexpr uint32_t K_STEP = FP8 ? 512 : 1024;                // per m
+    // V[d = 16 blk + t][tokens 4 grp ..]: 8 bytes (bf16) or 4 bytes (fp8) of the row
+    const uint32_t v_off = FP8 ? (uint32_t)(t * 16 + grp * 4) : (uint32_t)(t * 32 + grp * 8);
+    constexpr uint32_t V_STEP = FP8 ? 256 : 512;                 // per blk
 
     auto page_block = [&](int j) -> int {
         int jc = j < n_pages ? j : n_pages - 1;
@@ -145,7 +163,14 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
         r.lim = l < 0 ? 0 : l;
         const uint8_t *kb = kc_base + bt * kc_page_bytes;
 #pragma unroll
-        for (int m = 0; m < 4; ++m) r.k[m] = *reinterpret_cast<const uint4 *>(kb + k_off + m * 1024);
+        for (int m = 0; m < 4; ++m) {
+            if (FP8) {
+                const uint2 w = *reinterpret_cast<const uint2 *>(kb + k_off + m * K_STEP);
+                r.k[m] = make_uint4(w.x, w.y, 0, 0);
+            } else {
+                r.k[m] = *reinterpret_cast<const uint4 *>(kb + k_off + m * K_STEP);
+            }
+        }
         // position of this lane's token: its index in the sequence (un-rotated cache), or one
         // angle for the whole page (block-uniform), or row 0 = identity (un-rotated request)
         int pos = qo ? qo - 1 : 0;                                                   // ops/models/llama_v1.py:231-262
@@ -163,13 +188,21 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     auto load_values = [&](int j, ValRegs &r) {
         const uint8_t *vb = vc_base + page_block(j) * vc_page_bytes;
 #pragma unroll
-        for (int blk = 0; blk < 8; ++blk) r.v[blk] = *reinterpret_cast<const uint2 *>(vb + v_off + blk * 512);
+        for (int blk = 0; blk < 8; ++blk) {
+            if (FP8) r.v[blk] = make_uint2(*reinterpret_cast<const uint32_t *>(vb + v_off + blk * V_STEP), 0);
+            else r.v[blk] = *reinterpret_cast<const uint2 *>(vb + v_off + blk * V_STEP);
+        }
     };
     // rotate the pair (lo, hi) = (d, d + 64) in fp32, one rounding to bf16
     auto rotate = [&](const uint4 &lo, const uint4 &hi, const Tab8<TT> &c, const Tab8<TT> &s, bf16x8_t &xo, bf16x8_t &yo) {
         float a[8], bb[8], cs[8], sn[8], x[8], y[8];
-        unpack8(lo, a);
-        unpack8(hi, bb);
+        if (FP8) {
+            unpack8_fp8(lo.x, lo.y, k_scale, a);
+            unpack8_fp8(hi.x, hi.y, k_scale, bb);
+        } else {
+            unpack8(lo, a);
+            unpack8(hi, bb);
+        }
         c.get(cs);
         s.get(sn);
 #pragma unroll
@@ -220,6 +253,10 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     // V words of a page with the masked tokens zeroed (a masked slot may hold anything)
     auto masked_v = [&](const ValRegs &r, int lim, int blk) -> uint2 {
         uint2 w = r.v[blk];
+        if (FP8) {
+            const f32x2_t lo = __builtin_amdgcn_cvt_pk_f32_fp8(w.x, false), hi = __builtin_amdgcn_cvt_pk_f32_fp8(w.x >> 16, false);
+            w = make_uint2(pack_bf16(lo[0] * v_scale, lo[1] * v_scale), pack_bf16(hi[0] * v_scale, hi[1] * v_scale));
+        }
         if (lim < BS) {
             if (4 * grp + 0 >= lim) w.x &= 0xffff0000u;
             if (4 * grp + 1 >= lim) w.x &= 0x0000ffffu;
@@ -335,9 +372,10 @@ paged_decode_merge_kernel(const lazyattn_prefill_params p, const int nsplit) {
 
 // ------------------------------------------------------------------ host side
 bool decode_mfma_supports(const lazyattn_prefill_params &p) {
-    if (p.dtype != LAZYATTN_BF16 || p.cache_dtype != LAZYATTN_BF16) return false;
+    const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3;
+    if (p.dtype != LAZYATTN_BF16 || !(p.cache_dtype == LAZYATTN_BF16 || fp8)) return false;
     if (p.table_dtype != LAZYATTN_BF16 && p.table_dtype != LAZYATTN_F32) return false;
-    if (p.head_dim != D || p.block_size != BS || p.x != 8) return false;
+    if (p.head_dim != D || p.block_size != BS || p.x != (fp8 ? 16 : 8)) return false;
     if (p.sliding_window > 0) return false;
     if (p.pos_mode != LAZYATTN_POS_NATURAL && p.pos_mode != LAZYATTN_POS_BLOCK_UNIFORM) return false;
     if (p.num_q_heads / p.num_kv_heads > 16) return false;
@@ -347,7 +385,7 @@ bool decode_mfma_supports(const lazyattn_prefill_params &p) {
     const int64_t al[] = {p.q_stride[0], p.q_stride[1], p.o_stride[0], p.o_stride[1], p.kc_stride[0], p.kc_stride[1],
                           p.vc_stride[0], p.vc_stride[1], p.table_stride};
     for (int64_t s : al)
-        if (s % 8) return false;                       // 16-byte rows
+        if (s % 16) return false;                      // 16-byte rows whatever the element size
     const void *ptrs[] = {p.q, p.o, p.k_cache, p.v_cache, p.cos_sin_cache};
     for (const void *q : ptrs)
         if (((uintptr_t)q) & 15) return false;
@@ -384,10 +422,12 @@ int launch_decode_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
     const int64_t waves = (int64_t)p.batch * p.num_kv_heads * nsplit;
     const unsigned nblocks = (unsigned)((waves + WAVES - 1) / WAVES);
     if (phases & LAZYATTN_PHASE_MAIN) {
-        if (p.table_dtype == LAZYATTN_F32)
-            hipLaunchKernelGGL(paged_decode_kernel<float>, dim3(nblocks), dim3(WAVES * 64), 0, stream, p, nsplit);
-        else
-            hipLaunchKernelGGL(paged_decode_kernel<bf16_t>, dim3(nblocks), dim3(WAVES * 64), 0, stream, p, nsplit);
+        const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3, t32 = p.table_dtype == LAZYATTN_F32;
+        const dim3 grid(nblocks), block(WAVES * 64);
+        if (fp8 && t32) hipLaunchKernelGGL((paged_decode_kernel<float, true>), grid, block, 0, stream, p, nsplit);
+        else if (fp8) hipLaunchKernelGGL((paged_decode_kernel<bf16_t, true>), grid, block, 0, stream, p, nsplit);
+        else if (t32) hipLaunchKernelGGL((paged_decode_kernel<float, false>), grid, block, 0, stream, p, nsplit);
+        else hipLaunchKernelGGL((paged_decode_kernel<bf16_t, false>), grid, block, 0, stream, p, nsplit);
         if (hipGetLastError() != hipSuccess) return LAZYATTN_E_LAUNCH;
     }
     if (nsplit > 1 && (phases & LAZYATTN_PHASE_COMBINE)) {

@@ -16,25 +16,29 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda"
 
 
-def _decode_batch(variant, *, hq=8, hkv=2, q_lens=(1, 1, 1, 1, 1), table_f32=False, seed=77):
+def _decode_batch(variant, *, hq=8, hkv=2, q_lens=(1, 1, 1, 1, 1), table_f32=False, seed=77, kv="auto"):
     """Ragged documents (pads at document ends), requests of 1 to 9 documents, one new token each
     (or more: such requests must be skipped)."""
     d = 128
     w = wl.make_workload("decode", dtype=torch.bfloat16, hq=hq, hkv=hkv, d=d, theta=500000.0, block_size=16,
                          doc_lens=[40, 16, 33, 70, 5, 128, 97],
                          requests=[[3, 1, 0], [2], [0, 2, 3, 1, 5, 6, 4, 5, 6], [4, 0], [6, 5, 3]],
-                         q_lens=list(q_lens), variant=variant, seed=seed)
+                         q_lens=list(q_lens), variant=variant, seed=seed, kv_cache_dtype=kv)
     if table_f32:
         w.cos_sin_cache = w.cos_sin_cache.float()
     x = w.k_cache.shape[4]
+    fp8 = "fp8" in kv
+
+    def to_cache(t, scale):
+        return (t.float() / scale).to(torch.float8_e4m3fn).view(torch.uint8) if fp8 else t
     for b in range(len(q_lens)):
         qs, qe = int(w.b_start_loc[b]), int(w.b_start_loc[b + 1])
         ctx = int(w.b_seq_len[b]) - (qe - qs)
         for t in range(qe - qs):
             n = ctx + t
             pb = int(w.block_table[b, n // 16]); o_ = n % 16
-            w.k_cache[pb, :, :, o_, :] = w.k[qs + t].view(hkv, d // x, x)
-            w.v_cache[pb, :, :, o_] = w.v[qs + t]
+            w.k_cache[pb, :, :, o_, :] = to_cache(w.k[qs + t], w.k_scale).view(hkv, d // x, x)
+            w.v_cache[pb, :, :, o_] = to_cache(w.v[qs + t], w.v_scale)
     return w
 
 
@@ -42,6 +46,7 @@ def _oracle(w, lazy=None):
     ref = torch.full_like(w.q, 5.0)
     orc.paged_decode(w.q, w.k_cache, w.v_cache, w.block_table, w.b_start_loc, w.b_seq_len,
                      w.cos_sin_cache, w.q_mask, q_offset=w.q_offset, is_lazy=lazy,
+                     kv_cache_dtype=w.kv_cache_dtype, k_scale=w.k_scale, v_scale=w.v_scale,
                      pos_mode=orc.POS_NATURAL if w.pos_mode != orc.POS_BLOCK_UNIFORM else w.pos_mode, out=ref)
     return ref
 
@@ -52,7 +57,7 @@ def _run(w, *, lazy=None, num_splits=0, kernel=_ffi.KERNEL_AUTO):
     out = torch.full_like(g.q, 5.0)
     bu = w.pos_mode == orc.POS_BLOCK_UNIFORM
     _launch.launch_prefill(
-        q=g.q, k=g.k, v=g.v, o=out, kv_cache_dtype="auto", k_cache=g.k_cache, v_cache=g.v_cache,
+        q=g.q, k=g.k, v=g.v, o=out, kv_cache_dtype=w.kv_cache_dtype, k_cache=g.k_cache, v_cache=g.v_cache,
         b_loc=g.block_table, b_start_loc=g.b_start_loc, b_seq_len=g.b_seq_len, max_input_len=1,
         max_seq_len=g.max_seq_len, k_scale=g.k_scale, v_scale=g.v_scale, alibi_slopes=None, sliding_window=0,
         sm_scale=128 ** -0.5, skip_decode=False, cos_sin_cache=g.cos_sin_cache, rotary_dim=128,
@@ -111,6 +116,17 @@ def test_decode_group_sizes(hq, hkv):
     ref = _oracle(w)
     got = _run(w)
     assert _err(got, ref) < 2e-2, _err(got, ref)
+
+
+@pytest.mark.parametrize("variant,table_f32", [("natural", False), ("block_uniform", True)])
+def test_decode_fp8_cache(variant, table_f32):
+    print(f"case: decode fp8 {variant} table_f32={table_f32}", flush=True)
+    w = _decode_batch(variant, kv="fp8", table_f32=table_f32)
+    ref = _oracle(w)
+    got = _run(w, num_splits=3)
+    assert _err(got, ref) < 5e-2, _err(got, ref)
+    same = _run(w, kernel=_ffi.KERNEL_GENERIC)
+    assert _err(got, same) < 2e-2, _err(got, same)
 
 
 def test_decode_pad_slots_may_hold_nan():
