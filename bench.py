@@ -135,6 +135,65 @@ def bench_decode(a):
     print(json.dumps(out))
 
 
+def bench_rope_write(a):
+    """The step before the attention call for a prefill chunk of 8 192 new tokens, 8B geometry, bf16:
+    Q rotated in place, un-rotated K and V scattered into 16-token pages.  One launch."""
+    import torch
+    from oracle import deferred_rope as orc
+    from lazy_amd.model_executor.layers import rotary_embedding as rope
+    T, hq, hkv, d, bs = 8192, 32, 8, 128, 16
+    gen = torch.Generator().manual_seed(4)
+    table = orc.build_cos_sin_table(T + bs, d, 500000.0).to(torch.bfloat16).cuda()
+    q = torch.randn(T, hq, d, generator=gen).to(torch.bfloat16).cuda()
+    k = torch.randn(T, hkv, d, generator=gen).to(torch.bfloat16).cuda()
+    v = torch.randn(T, hkv, d, generator=gen).to(torch.bfloat16).cuda()
+    pos = torch.arange(T, device="cuda")
+    nb = T // bs + 4
+    blocks = torch.randperm(nb, generator=gen)[:T // bs]
+    slots = (blocks[:, None] * bs + torch.arange(bs)[None, :]).flatten().cuda()     # whole pages, shuffled blocks
+    kc = torch.zeros(nb, hkv, d // 8, bs, 8, device="cuda", dtype=torch.bfloat16)
+    vc = torch.zeros(nb, hkv, d, bs, device="cuda", dtype=torch.bfloat16)
+
+    class Plan:
+        def run(self):
+            rope.rotate_and_write(pos, q, k, v, d, table, rotate_query=True, rotate_key=False, key_cache=kc,
+                                  value_cache=vc, slot_mapping=slots)
+    plan = Plan()
+    for _ in range(a.warmup):
+        plan.run()
+    torch.cuda.synchronize()
+    ms = time_calls(plan, a.steps)
+    nbytes = T * (2 * hq + 4 * hkv) * d * 2            # Q read + written, K and V read, both caches written
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    out = {
+        "metric": "Q rotary + paged-cache write of new tokens: GB/s, 8B geometry, 8192 tokens",
+        "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "w1_8b_bf16_rope_write_8192tok", "hq": hq, "hkv": hkv, "head_dim": d, "page": bs,
+                   "tokens": T, "mb_per_call": round(nbytes / 1e6, 2)},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None, "kernel": "rope_cache_write_kernel",
+                     "kernel_ms": round(ms, 5)},
+    }
+    if not a.no_cpu:
+        torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))
+        Ts = 1024
+        qc, kcpu, vcpu = q[:Ts].cpu(), k[:Ts].cpu(), v[:Ts].cpu()
+        kcc, vcc, tc, sc = kc.cpu(), vc.cpu(), table.cpu(), slots[:Ts].cpu()
+        ts = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            orc.rotary_new_tokens(pos[:Ts].cpu(), qc, kcpu, tc, q_only=True)
+            orc.paged_cache_write(kcpu, vcpu, kcc, vcc, sc)
+            ts.append(time.perf_counter() - t0)
+        sec = statistics.median(ts)
+        out["cpu_baseline"] = {"value": round(nbytes * Ts / T / sec / 1e9, 3), "unit": "GB/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"first {Ts} of the {T} tokens, 3 calls, median {sec * 1e3:.1f} ms"}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -143,8 +202,9 @@ def main():
     ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5])
     ap.add_argument("--num-splits", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--path", choices=["prefill", "decode"], default="prefill",
-                    help="prefill: the headline prefix-prefill call (default); decode: the q_len==1 kernel, an HBM-bound path")
+    ap.add_argument("--path", choices=["prefill", "decode", "rope_write"], default="prefill",
+                    help="prefill: the headline prefix-prefill call (default); decode: the q_len==1 kernel; "
+                         "rope_write: Q rotary + paged-cache write of the new tokens (both HBM-bound)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a 256 MiB device-to-device copy (known traffic, for scaling profiler counters)")
     a = ap.parse_args()
@@ -162,6 +222,8 @@ def main():
     torch.cuda.set_device(0)
     if a.path == "decode":
         return bench_decode(a)
+    if a.path == "rope_write":
+        return bench_rope_write(a)
     w = wl.config(a.config)
     g = w.to("cuda:0")
     plan, o = make_plan(g, a.num_splits, _ffi.PHASE_ALL)

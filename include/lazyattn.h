@@ -137,6 +137,40 @@ int lazyattn_paged_decode_rotary(const lazyattn_prefill_params *p, void *stream)
  * counterpart (the Triton kernel is one program per (sequence, kv head)). */
 size_t lazyattn_paged_decode_workspace_bytes(const lazyattn_prefill_params *p);
 
+/* ---- the step before the attention call: rotary embedding of the new tokens + paged-cache write ----
+ * One launch does what the reference does with two third-party ops per layer:
+ *   rotary_embedding(positions, query, key_or_None, head_size, cos_sin_cache, is_neox)
+ *     (lazy_attn/lazy/model_executor/layers/rotary_embedding.py:67-94: query only under the
+ *      un-rotated-cache variant, query and key otherwise, :48-49), in place, NeoX pairing (d, d + R/2);
+ *   PagedAttention.write_to_paged_cache(key, value, key_cache, value_cache, slot_mapping,
+ *     kv_cache_dtype, k_scale, v_scale)  (lazy_attn/lazy/attention/backends/triton_attn.py:100-109):
+ *     token t -> slot_mapping[t] = block * block_size + offset (negative: not written);
+ *     fp8 caches store value / scale, saturated to +-448, rounded to e4m3.
+ * The key written to the cache is the key as it is left in `k` (rotated iff rotate_k). */
+typedef struct lazyattn_rope_write_params {
+    void *q;                    /* [T, Hq, D], rotated in place when rotate_q; may be NULL when !rotate_q */
+    void *k;                    /* [T, Hkv, D], rotated in place when rotate_k */
+    const void *v;              /* [T, Hkv, D] */
+    void *k_cache;              /* [NB, Hkv, D/x, BS, x]; NULL = no cache write */
+    void *v_cache;              /* [NB, Hkv, D, BS] */
+    const void *slot_mapping;   /* [T] int32 or int64 (slot_bits); NULL = no cache write */
+    const void *positions;      /* [T] int32 or int64 (pos_bits): rows of the cos/sin table */
+    const void *cos_sin_cache;  /* [max_pos, rotary_dim] */
+    const float *k_scale;       /* 1 element each, read only for fp8 caches */
+    const float *v_scale;
+    int64_t q_stride[3], k_stride[3], v_stride[3];   /* in elements */
+    int64_t kc_stride[5], vc_stride[4];
+    int64_t table_stride;
+    int32_t num_tokens, num_q_heads, num_kv_heads, head_dim, rotary_dim, block_size, x;
+    int32_t dtype;              /* q/k/v: LAZYATTN_F32 / BF16 / F16 */
+    int32_t cache_dtype;        /* = dtype, or LAZYATTN_FP8_E4M3 */
+    int32_t table_dtype;        /* = dtype, or LAZYATTN_F32 */
+    int32_t rotate_q, rotate_k;
+    int32_t pos_bits, slot_bits;
+} lazyattn_rope_write_params;
+
+int lazyattn_rope_and_cache_write(const lazyattn_rope_write_params *p, void *stream);
+
 /* cos/sin table builder on the device: out[p, i] = cos(p*inv[i]), out[p, R/2+i] = sin(..),
  * inv = base^(-2i/R), optionally Llama-3 smoothed.  Restates
  * lazy_attn/lazy/model_executor/rope/cos_sin.py:24-66 and the third-party table layout

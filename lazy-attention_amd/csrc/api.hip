@@ -9,6 +9,7 @@ size_t mfma_workspace_bytes(const lazyattn_prefill_params &p);
 int launch_decode_mfma(const lazyattn_prefill_params &p, hipStream_t stream);
 bool decode_mfma_supports(const lazyattn_prefill_params &p);
 size_t decode_workspace_bytes(const lazyattn_prefill_params &p);
+int launch_rope_cache_write(const lazyattn_rope_write_params &p, hipStream_t stream);
 int launch_cos_sin_table(void *out, int out_dtype, int64_t row_stride, int max_position,
                          int rotary_dim, double base, int rope_type, double factor, double low,
                          double high, int orig_max, hipStream_t stream);
@@ -92,6 +93,43 @@ extern "C" size_t lazyattn_paged_decode_workspace_bytes(const lazyattn_prefill_p
     if (!p || check_common(p, true) != LAZYATTN_OK) return 0;
     if (p->kernel == LAZYATTN_KERNEL_GENERIC || !decode_mfma_supports(*p)) return 0;
     return decode_workspace_bytes(*p);
+}
+
+extern "C" int lazyattn_rope_and_cache_write(const lazyattn_rope_write_params *p, void *stream) {
+    if (!p) return LAZYATTN_E_NULL;
+    const bool write = p->k_cache && p->slot_mapping;
+    if ((p->rotate_q && !p->q) || ((p->rotate_k || write) && !p->k) || (write && (!p->v || !p->v_cache))) return LAZYATTN_E_NULL;
+    if ((p->rotate_q || p->rotate_k) && (!p->positions || !p->cos_sin_cache)) return LAZYATTN_E_NULL;
+    if (p->num_tokens < 0 || p->num_q_heads < 0 || p->num_kv_heads <= 0 || p->head_dim <= 0) return LAZYATTN_E_SHAPE;
+    if (p->head_dim % 8 || p->rotary_dim % 16 || p->rotary_dim <= 0 || p->rotary_dim > p->head_dim) return LAZYATTN_E_SHAPE;
+    if (p->dtype != LAZYATTN_F32 && p->dtype != LAZYATTN_BF16 && p->dtype != LAZYATTN_F16) return LAZYATTN_E_DTYPE;
+    if (p->table_dtype != p->dtype && p->table_dtype != LAZYATTN_F32) return LAZYATTN_E_DTYPE;
+    if (p->pos_bits != 32 && p->pos_bits != 64) return LAZYATTN_E_DTYPE;
+    const int64_t vec = p->dtype == LAZYATTN_F32 ? 4 : 8;       // elements per 16 bytes
+    if (p->q_stride[2] != 1 && p->q) return LAZYATTN_E_UNSUPPORTED;
+    if (p->k_stride[2] != 1 || (write && p->v_stride[2] != 1)) return LAZYATTN_E_UNSUPPORTED;
+    if ((p->q && (p->q_stride[0] % vec || p->q_stride[1] % vec || ((uintptr_t)p->q & 15))) ||
+        p->k_stride[0] % vec || p->k_stride[1] % vec || ((uintptr_t)p->k & 15))
+        return LAZYATTN_E_UNSUPPORTED;
+    if ((p->rotate_q || p->rotate_k) &&
+        (p->table_stride % (p->table_dtype == LAZYATTN_F32 ? 4 : 8) || ((uintptr_t)p->cos_sin_cache & 15)))
+        return LAZYATTN_E_UNSUPPORTED;
+    if (write) {
+        const bool fp8 = p->cache_dtype == LAZYATTN_FP8_E4M3;
+        if (!fp8 && p->cache_dtype != p->dtype) return LAZYATTN_E_DTYPE;
+        if (fp8 && (!p->k_scale || !p->v_scale)) return LAZYATTN_E_NULL;
+        if (p->slot_bits != 32 && p->slot_bits != 64) return LAZYATTN_E_DTYPE;
+        if (p->block_size <= 0 || p->x <= 0 || p->head_dim % p->x) return LAZYATTN_E_SHAPE;
+        if (p->v_stride[0] % vec || p->v_stride[1] % vec || ((uintptr_t)p->v & 15)) return LAZYATTN_E_UNSUPPORTED;
+        if (p->kc_stride[4] != 1) return LAZYATTN_E_UNSUPPORTED;
+        // a K chunk of 8 elements is one store when x is a multiple of 8 (16-byte aligned for 2-byte types,
+        // 8-byte aligned for fp8); x = 4 (fp32 caches) is written element-wise
+        if (p->x % 8 == 0 &&
+            (((uintptr_t)p->k_cache & 15) || p->kc_stride[0] % 16 || p->kc_stride[1] % 16 || p->kc_stride[2] % 8 || p->kc_stride[3] % 8))
+            return LAZYATTN_E_UNSUPPORTED;
+    }
+    if (p->num_tokens == 0) return LAZYATTN_OK;
+    return launch_rope_cache_write(*p, (hipStream_t)stream);
 }
 
 extern "C" int lazyattn_build_cos_sin_cache(void *out, int32_t out_dtype, int64_t row_stride,

@@ -22,7 +22,7 @@ PHASE_MAIN, PHASE_COMBINE, PHASE_ALL = 1, 2, 3
 ERRORS = {-1: "NULL", -2: "SHAPE", -3: "DTYPE", -4: "UNSUPPORTED", -5: "WORKSPACE", -6: "LAUNCH"}
 EXPORTS = ("lazyattn_prefill_workspace_bytes", "lazyattn_prefix_prefill", "lazyattn_paged_decode_workspace_bytes",
            "lazyattn_paged_decode_rotary", "lazyattn_build_cos_sin_cache",
-           "lazyattn_pack_cos_sin_cache",
+           "lazyattn_pack_cos_sin_cache", "lazyattn_rope_and_cache_write",
            "lazyattn_error_string", "lazyattn_abi_version")
 
 _DTYPE = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
@@ -46,6 +46,17 @@ class PrefillParams(C.Structure):
                                     "num_splits", "phases")]
         + [("sm_scale", C.c_float), ("num_tokens", C.c_int32), ("max_seq_len", C.c_int32),
            ("packed_rows", C.c_int32)])
+
+
+class RopeWriteParams(C.Structure):
+    _fields_ = (
+        [(n, C.c_void_p) for n in ("q", "k", "v", "k_cache", "v_cache", "slot_mapping", "positions",
+                                   "cos_sin_cache", "k_scale", "v_scale")]
+        + [("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3), ("v_stride", C.c_int64 * 3),
+           ("kc_stride", C.c_int64 * 5), ("vc_stride", C.c_int64 * 4), ("table_stride", C.c_int64)]
+        + [(n, C.c_int32) for n in ("num_tokens", "num_q_heads", "num_kv_heads", "head_dim", "rotary_dim",
+                                    "block_size", "x", "dtype", "cache_dtype", "table_dtype", "rotate_q",
+                                    "rotate_k", "pos_bits", "slot_bits")])
 
 
 def lib() -> C.CDLL:
@@ -72,6 +83,8 @@ def lib() -> C.CDLL:
         L.lazyattn_pack_cos_sin_cache.restype = C.c_int
         L.lazyattn_pack_cos_sin_cache.argtypes = [C.c_void_p, C.c_void_p, C.c_int32, C.c_int64, C.c_int32,
                                                   C.c_int32, C.c_void_p]
+        L.lazyattn_rope_and_cache_write.restype = C.c_int
+        L.lazyattn_rope_and_cache_write.argtypes = [C.POINTER(RopeWriteParams), C.c_void_p]
         L.lazyattn_error_string.restype = C.c_char_p
         L.lazyattn_error_string.argtypes = [C.c_int]
         L.lazyattn_abi_version.restype = C.c_int

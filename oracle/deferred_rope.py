@@ -343,6 +343,42 @@ def paged_decode(q, k_cache, v_cache, block_table, query_start_loc, seq_lens,
 
 
 # --------------------------------------------------------------------------
+# The step before the attention call: rotary embedding of the new tokens and the
+# paged-cache write (rotary_embedding.py:40-94; backends/triton_attn.py:100-109).
+# The two third-party ops behind them (vLLM rotary_embedding / reshape_and_cache) are absent
+# from the reference tree: their published layouts are restated; the write is pinned by the
+# round trip through gather_pages (the inverse index map the attention oracle reads with).
+# --------------------------------------------------------------------------
+def rotary_new_tokens(positions, query, key, table, *, q_only: bool, compute_dtype=torch.float32):
+    """NeoX rotary of query [T,Hq,D] (and key [T,Hkv,D] unless q_only) at positions[t];
+    returns new tensors in the inputs' dtypes (rotary_embedding.py:40-65 arithmetic, one rounding)."""
+    tab = table.to(compute_dtype)
+    q = rotate_at(query.to(compute_dtype), positions, tab).to(query.dtype)
+    k = key if q_only else rotate_at(key.to(compute_dtype), positions, tab).to(key.dtype)
+    return q, k
+
+
+def paged_cache_write(key, value, k_cache, v_cache, slot_mapping, kv_cache_dtype="auto", k_scale=1.0, v_scale=1.0):
+    """In place: token t -> slot_mapping[t] = block*BS + offset (negative: skipped);
+    K[block, h, d // x, offset, d % x] = key[t, h, d]; V[block, h, d, offset] = value[t, h, d];
+    fp8 caches (uint8 storage) hold (value / scale) saturated to +-448 as e4m3."""
+    nb, hkv, dx, bs, x = k_cache.shape
+    fp8 = "fp8" in kv_cache_dtype
+
+    def enc(t, scale):
+        if not fp8:
+            return t.to(k_cache.dtype)
+        return (t.float() / float(scale)).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8)
+    for t in range(key.shape[0]):
+        slot = int(slot_mapping[t])
+        if slot < 0:
+            continue
+        blk, off = slot // bs, slot % bs
+        k_cache[blk, :, :, off, :] = enc(key[t], k_scale).view(hkv, dx, x)
+        v_cache[blk, :, :, off] = enc(value[t], v_scale)
+
+
+# --------------------------------------------------------------------------
 # Brute force (independent of everything above except the table rows):
 # scalar loops in Python floats.  Tiny shapes only.
 # --------------------------------------------------------------------------

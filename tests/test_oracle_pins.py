@@ -364,3 +364,43 @@ def test_lazy_decode_rotating_keys_equals_derotating_query():
     p = torch.softmax(scores, dim=-1)
     ref = torch.stack([(p[h][:, None] * vals[:, h // 2]).sum(0) for h in range(4)])
     assert (got[0].double() - ref).abs().max() < 1e-6
+
+
+def test_paged_cache_write_is_inverse_of_gather_and_matches_layout_formula():
+    """K[block, h, d // x, off, d % x], V[block, h, d, off] (the third-party reshape_and_cache layout the
+    reference's kernels index at old_ops/prefix_prefill.py:172-181,196-199): element-wise formula on a
+    small case, and the round trip through gather_pages."""
+    g = torch.Generator().manual_seed(1)
+    t, hkv, d, bs, x, nb = 20, 2, 16, 4, 8, 7
+    k = torch.randn(t, hkv, d, generator=g); v = torch.randn(t, hkv, d, generator=g)
+    kc = torch.zeros(nb, hkv, d // x, bs, x); vc = torch.zeros(nb, hkv, d, bs)
+    slots = torch.randperm(nb * bs, generator=g)[:t]
+    slots[5] = -1
+    orc.paged_cache_write(k, v, kc, vc, slots)
+    for tok in range(t):
+        s_ = int(slots[tok])
+        if s_ < 0:
+            continue
+        for h in range(hkv):
+            for dd in range(d):
+                assert kc[s_ // bs, h, dd // x, s_ % bs, dd % x] == k[tok, h, dd]
+                assert vc[s_ // bs, h, dd, s_ % bs] == v[tok, h, dd]
+    assert kc.count_nonzero() == (t - 1) * hkv * d                 # the skipped token wrote nothing
+    slots = torch.arange(bs, bs + t)
+    kc.zero_(); vc.zero_()
+    orc.paged_cache_write(k, v, kc, vc, slots)
+    kb, vb = orc.gather_pages(kc, vc, torch.arange(1, 1 + t // bs))
+    assert torch.equal(kb, k) and torch.equal(vb, v)
+
+
+def test_rotary_new_tokens_q_only_leaves_key_and_preserves_norm():
+    g = torch.Generator().manual_seed(2)
+    table = orc.build_cos_sin_table(512, 32, 10000.0)
+    q = torch.randn(9, 4, 32, generator=g, dtype=torch.float64); k = torch.randn(9, 2, 32, generator=g, dtype=torch.float64)
+    pos = torch.randint(0, 512, (9,), generator=g)
+    q1, k1 = orc.rotary_new_tokens(pos, q, k, table, q_only=True, compute_dtype=torch.float64)
+    assert k1 is k
+    assert torch.allclose(q1.norm(dim=-1), q.norm(dim=-1), atol=1e-12)
+    q2, k2 = orc.rotary_new_tokens(pos, q, k, table, q_only=False, compute_dtype=torch.float64)
+    # relative-position property: <R(p)q, R(p)k> = <q, k>
+    assert torch.allclose((q2[:, :2] * k2).sum(-1), (q[:, :2] * k).sum(-1), atol=1e-10)
