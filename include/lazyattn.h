@@ -171,6 +171,20 @@ typedef struct lazyattn_rope_write_params {
 
 int lazyattn_rope_and_cache_write(const lazyattn_rope_write_params *p, void *stream);
 
+/* Per-page rotation metadata of a batch, written on the device into the [batch, row_len] int32
+ * buffers the attention kernels read.  Same integers as metadata_for_lazy_attention /
+ * metadata_for_mepic (lazy_attn/lazy/core/sched/scheduler.py:758-787); replaces the per-request host
+ * loop and the two host-to-device copies of lazy_attn/lazy/worker/gpu_model_runner.py:193-239.
+ * Documents in CSR form: request b owns doc_lens[doc_start[b] .. doc_start[b+1]) (true lengths) and
+ * the matching doc_lens_padded (multiples of block_size).  zero_offsets = the un-rotated-cache
+ * variant (all q_offset 0).  Rows are written completely (zeros beyond the query page).
+ * max_offset (optional, [batch]) receives each request's largest offset value, for the
+ * 16-bit admission check of the packed block table (worker/gpu_model_runner.py:212-226). */
+int lazyattn_build_rotation_metadata(const int32_t *doc_lens, const int32_t *doc_lens_padded,
+                                     const int32_t *doc_start, int32_t batch, int32_t block_size,
+                                     int32_t zero_offsets, int32_t *q_offset, int32_t *q_mask,
+                                     int64_t row_stride, int32_t row_len, int32_t *max_offset, void *stream);
+
 /* cos/sin table builder on the device: out[p, i] = cos(p*inv[i]), out[p, R/2+i] = sin(..),
  * inv = base^(-2i/R), optionally Llama-3 smoothed.  Restates
  * lazy_attn/lazy/model_executor/rope/cos_sin.py:24-66 and the third-party table layout

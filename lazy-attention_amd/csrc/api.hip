@@ -10,6 +10,9 @@ int launch_decode_mfma(const lazyattn_prefill_params &p, hipStream_t stream);
 bool decode_mfma_supports(const lazyattn_prefill_params &p);
 size_t decode_workspace_bytes(const lazyattn_prefill_params &p);
 int launch_rope_cache_write(const lazyattn_rope_write_params &p, hipStream_t stream);
+int launch_rotation_metadata(const int32_t *doc_lens, const int32_t *doc_lens_padded, const int32_t *doc_start, int batch,
+                             int block_size, int zero_offsets, int32_t *q_offset, int32_t *q_mask, int64_t row_stride,
+                             int row_len, int32_t *max_offset, hipStream_t stream);
 int launch_cos_sin_table(void *out, int out_dtype, int64_t row_stride, int max_position,
                          int rotary_dim, double base, int rope_type, double factor, double low,
                          double high, int orig_max, hipStream_t stream);
@@ -130,6 +133,16 @@ extern "C" int lazyattn_rope_and_cache_write(const lazyattn_rope_write_params *p
     }
     if (p->num_tokens == 0) return LAZYATTN_OK;
     return launch_rope_cache_write(*p, (hipStream_t)stream);
+}
+
+extern "C" int lazyattn_build_rotation_metadata(const int32_t *doc_lens, const int32_t *doc_lens_padded,
+                                                const int32_t *doc_start, int32_t batch, int32_t block_size,
+                                                int32_t zero_offsets, int32_t *q_offset, int32_t *q_mask,
+                                                int64_t row_stride, int32_t row_len, int32_t *max_offset, void *stream) {
+    if (!doc_lens || !doc_lens_padded || !doc_start || !q_offset || !q_mask) return LAZYATTN_E_NULL;
+    if (batch < 0 || block_size <= 0 || row_len <= 0 || row_stride < row_len) return LAZYATTN_E_SHAPE;
+    return launch_rotation_metadata(doc_lens, doc_lens_padded, doc_start, batch, block_size, zero_offsets, q_offset, q_mask,
+                                    row_stride, row_len, max_offset, (hipStream_t)stream);
 }
 
 extern "C" int lazyattn_build_cos_sin_cache(void *out, int32_t out_dtype, int64_t row_stride,
