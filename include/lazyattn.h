@@ -185,6 +185,27 @@ int lazyattn_build_rotation_metadata(const int32_t *doc_lens, const int32_t *doc
                                      int32_t zero_offsets, int32_t *q_offset, int32_t *q_mask,
                                      int64_t row_stride, int32_t row_len, int32_t *max_offset, void *stream);
 
+/* Copy-and-re-rotate of cached document blocks, all blocks of one layer in one launch.
+ * Replaces the per-layer, per-block eager loop of block_attn_vllm/gpu_model_runner.py:94-106 over
+ * copy_paged_block + place_paged_block_keys (block_attn_vllm/utils.py:48-95).
+ * items: [num_items][4] int32 on the device = (new_id, old_id, from_start, to_start): block old_id
+ * (K and V) is copied to new_id, and slot o of the K copy goes from rotation position from_start + o to
+ * to_start + o (un-rotate, then rotate, NeoX pairing, rows of cos_sin_cache).  new_id == old_id re-rotates
+ * in place.  The new blocks must be distinct from each other and from every old block of the call. */
+typedef struct lazyattn_reposition_params {
+    void *k_cache;              /* [NB, Hkv, D/x, BS, x] */
+    void *v_cache;              /* [NB, Hkv, D, BS] */
+    const int32_t *items;
+    const void *cos_sin_cache;  /* [max_pos, D] */
+    int64_t kc_stride[5], vc_stride[4];
+    int64_t table_stride;
+    int32_t num_items, num_kv_heads, head_dim, block_size, x;
+    int32_t dtype;              /* cache element type: LAZYATTN_F32 / BF16 / F16 */
+    int32_t table_dtype;        /* = dtype, or LAZYATTN_F32 */
+} lazyattn_reposition_params;
+
+int lazyattn_reposition_blocks(const lazyattn_reposition_params *p, void *stream);
+
 /* cos/sin table builder on the device: out[p, i] = cos(p*inv[i]), out[p, R/2+i] = sin(..),
  * inv = base^(-2i/R), optionally Llama-3 smoothed.  Restates
  * lazy_attn/lazy/model_executor/rope/cos_sin.py:24-66 and the third-party table layout

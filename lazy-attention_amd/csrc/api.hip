@@ -13,6 +13,7 @@ int launch_rope_cache_write(const lazyattn_rope_write_params &p, hipStream_t str
 int launch_rotation_metadata(const int32_t *doc_lens, const int32_t *doc_lens_padded, const int32_t *doc_start, int batch,
                              int block_size, int zero_offsets, int32_t *q_offset, int32_t *q_mask, int64_t row_stride,
                              int row_len, int32_t *max_offset, hipStream_t stream);
+int launch_block_reposition(const lazyattn_reposition_params &p, hipStream_t stream);
 int launch_cos_sin_table(void *out, int out_dtype, int64_t row_stride, int max_position,
                          int rotary_dim, double base, int rope_type, double factor, double low,
                          double high, int orig_max, hipStream_t stream);
@@ -143,6 +144,29 @@ extern "C" int lazyattn_build_rotation_metadata(const int32_t *doc_lens, const i
     if (batch < 0 || block_size <= 0 || row_len <= 0 || row_stride < row_len) return LAZYATTN_E_SHAPE;
     return launch_rotation_metadata(doc_lens, doc_lens_padded, doc_start, batch, block_size, zero_offsets, q_offset, q_mask,
                                     row_stride, row_len, max_offset, (hipStream_t)stream);
+}
+
+extern "C" int lazyattn_reposition_blocks(const lazyattn_reposition_params *p, void *stream) {
+    if (!p || !p->k_cache || !p->v_cache || !p->items || !p->cos_sin_cache) return LAZYATTN_E_NULL;
+    if (p->num_items < 0 || p->num_kv_heads <= 0 || p->head_dim <= 0 || p->head_dim % 16 || p->block_size <= 0 || p->x <= 0 ||
+        p->head_dim % p->x)
+        return LAZYATTN_E_SHAPE;
+    if (p->dtype != LAZYATTN_F32 && p->dtype != LAZYATTN_BF16 && p->dtype != LAZYATTN_F16) return LAZYATTN_E_DTYPE;
+    if (p->table_dtype != p->dtype && p->table_dtype != LAZYATTN_F32) return LAZYATTN_E_DTYPE;
+    const int esz = p->dtype == LAZYATTN_F32 ? 4 : 2;
+    // the V block is copied as one contiguous run of 16-byte pieces; K chunks of 8 are single accesses when x allows
+    if (p->kc_stride[4] != 1 || p->vc_stride[3] != 1 || p->vc_stride[2] != p->block_size ||
+        p->vc_stride[1] != (int64_t)p->head_dim * p->block_size)
+        return LAZYATTN_E_UNSUPPORTED;
+    if (((uintptr_t)p->k_cache & 15) || ((uintptr_t)p->v_cache & 15) || ((uintptr_t)p->cos_sin_cache & 15) ||
+        (p->vc_stride[0] * esz) % 16 || ((int64_t)p->num_kv_heads * p->head_dim * p->block_size * esz) % 16 ||
+        (p->table_stride * (p->table_dtype == LAZYATTN_F32 ? 4 : 2)) % 16)
+        return LAZYATTN_E_UNSUPPORTED;
+    if (p->x % 8 == 0 && ((p->kc_stride[0] * esz) % 16 || (p->kc_stride[1] * esz) % 16 || (p->kc_stride[2] * esz) % 16 ||
+                          (p->kc_stride[3] * esz) % 16))
+        return LAZYATTN_E_UNSUPPORTED;
+    if (p->num_items == 0) return LAZYATTN_OK;
+    return launch_block_reposition(*p, (hipStream_t)stream);
 }
 
 extern "C" int lazyattn_build_cos_sin_cache(void *out, int32_t out_dtype, int64_t row_stride,

@@ -379,6 +379,28 @@ def paged_cache_write(key, value, k_cache, v_cache, slot_mapping, kv_cache_dtype
 
 
 # --------------------------------------------------------------------------
+# Block re-positioning (block_attn_vllm/utils.py:48-95): copy a paged block, un-rotate its keys
+# from from_start+slot to position 0, rotate them to to_start+slot.  Two explicit steps.
+# --------------------------------------------------------------------------
+def reposition_blocks(k_cache, v_cache, items, table, compute_dtype=torch.float32):
+    """In place on the caches; items = [(new_id, old_id, from_start, to_start)]."""
+    nb, hkv, dx, bs, x = k_cache.shape
+    d = dx * x
+    half = d // 2
+    tab = table.to(compute_dtype)
+    src_k = {old: k_cache[old].clone() for _, old, _, _ in items}
+    src_v = {old: v_cache[old].clone() for _, old, _, _ in items}
+    for new_id, old_id, from_start, to_start in items:
+        k = src_k[old_id].permute(0, 2, 1, 3).reshape(hkv, bs, d).to(compute_dtype)      # [Hkv, BS, D]
+        o = torch.arange(bs)
+        rf, rt = tab[from_start + o], tab[to_start + o]
+        k = neox_rotate(k, rf[None, :, :half], -rf[None, :, half:])                  # R(-from)  utils.py:84
+        k = neox_rotate(k, rt[None, :, :half], rt[None, :, half:])                   # R(+to)    utils.py:86
+        k_cache[new_id] = k.to(k_cache.dtype).reshape(hkv, bs, dx, x).permute(0, 2, 1, 3)
+        v_cache[new_id] = src_v[old_id]
+
+
+# --------------------------------------------------------------------------
 # Brute force (independent of everything above except the table rows):
 # scalar loops in Python floats.  Tiny shapes only.
 # --------------------------------------------------------------------------

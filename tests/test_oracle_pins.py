@@ -404,3 +404,22 @@ def test_rotary_new_tokens_q_only_leaves_key_and_preserves_norm():
     q2, k2 = orc.rotary_new_tokens(pos, q, k, table, q_only=False, compute_dtype=torch.float64)
     # relative-position property: <R(p)q, R(p)k> = <q, k>
     assert torch.allclose((q2[:, :2] * k2).sum(-1), (q[:, :2] * k).sum(-1), atol=1e-10)
+
+
+def test_reposition_blocks_equals_rotation_of_the_unrotated_keys():
+    """With an exact (float64) table, un-rotating from `from` and rotating to `to` must give the keys
+    one gets by rotating the never-rotated keys at `to` directly -- and must leave norms alone."""
+    g = torch.Generator().manual_seed(4)
+    hkv, d, bs, x, nb = 2, 32, 8, 8, 5
+    table = orc.build_cos_sin_table(256, d, 10000.0, dtype=torch.float64, math_dtype=torch.float64)
+    raw = torch.randn(bs, hkv, d, generator=g, dtype=torch.float64)                     # un-rotated keys of one block
+    stored = orc.rotate_at(raw, 40 + torch.arange(bs), table)                            # as cached: local positions 40..
+    kc = torch.zeros(nb, hkv, d // x, bs, x, dtype=torch.float64); vc = torch.randn(nb, hkv, d, bs, generator=g, dtype=torch.float64)
+    kc[1] = stored.reshape(bs, hkv, d // x, x).permute(1, 2, 0, 3)
+    v_old = vc[1].clone()
+    orc.reposition_blocks(kc, vc, [(3, 1, 40, 113)], table, compute_dtype=torch.float64)
+    got = kc[3].permute(2, 0, 1, 3).reshape(bs, hkv, d)
+    want = orc.rotate_at(raw, 113 + torch.arange(bs), table)
+    assert torch.allclose(got, want, atol=1e-9)
+    assert torch.allclose(got.norm(dim=-1), raw.norm(dim=-1), atol=1e-9)
+    assert torch.equal(vc[3], v_old) and torch.equal(kc[1].permute(2, 0, 1, 3).reshape(bs, hkv, d), stored)
