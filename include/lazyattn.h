@@ -185,6 +185,14 @@ int lazyattn_build_rotation_metadata(const int32_t *doc_lens, const int32_t *doc
                                      int32_t zero_offsets, int32_t *q_offset, int32_t *q_mask,
                                      int64_t row_stride, int32_t row_len, int32_t *max_offset, void *stream);
 
+/* Packed block table of the block-uniform decode path, [block:32 | q_offset:16 | q_mask:16] per int64
+ * entry (layout of lazy_attn/lazy/attention/ops/models/llama_v1.py:157-160), for the listed rows
+ * (rows == NULL: rows 0 .. n_rows-1), in one launch.  Replaces the tensor-op sequence of
+ * _rebuild_packed_block_table (lazy_attn/lazy/worker/gpu_model_runner.py:296-340), full or delta. */
+int lazyattn_pack_block_table(const int32_t *block_table, int64_t bt_stride, const int32_t *q_offset,
+                              const int32_t *q_mask, int64_t row_stride, const int32_t *rows, int32_t n_rows,
+                              int32_t row_len, int64_t *packed, int64_t packed_stride, void *stream);
+
 /* Copy-and-re-rotate of cached document blocks, all blocks of one layer in one launch.
  * Replaces the per-layer, per-block eager loop of block_attn_vllm/gpu_model_runner.py:94-106 over
  * copy_paged_block + place_paged_block_keys (block_attn_vllm/utils.py:48-95).

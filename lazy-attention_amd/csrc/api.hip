@@ -14,6 +14,9 @@ int launch_rotation_metadata(const int32_t *doc_lens, const int32_t *doc_lens_pa
                              int block_size, int zero_offsets, int32_t *q_offset, int32_t *q_mask, int64_t row_stride,
                              int row_len, int32_t *max_offset, hipStream_t stream);
 int launch_block_reposition(const lazyattn_reposition_params &p, hipStream_t stream);
+int launch_pack_block_table(const int32_t *block_table, int64_t bt_stride, const int32_t *q_offset, const int32_t *q_mask,
+                            int64_t row_stride, const int32_t *rows, int n_rows, int row_len, int64_t *packed,
+                            int64_t packed_stride, hipStream_t stream);
 int launch_cos_sin_table(void *out, int out_dtype, int64_t row_stride, int max_position,
                          int rotary_dim, double base, int rope_type, double factor, double low,
                          double high, int orig_max, hipStream_t stream);
@@ -144,6 +147,15 @@ extern "C" int lazyattn_build_rotation_metadata(const int32_t *doc_lens, const i
     if (batch < 0 || block_size <= 0 || row_len <= 0 || row_stride < row_len) return LAZYATTN_E_SHAPE;
     return launch_rotation_metadata(doc_lens, doc_lens_padded, doc_start, batch, block_size, zero_offsets, q_offset, q_mask,
                                     row_stride, row_len, max_offset, (hipStream_t)stream);
+}
+
+extern "C" int lazyattn_pack_block_table(const int32_t *block_table, int64_t bt_stride, const int32_t *q_offset,
+                                         const int32_t *q_mask, int64_t row_stride, const int32_t *rows, int32_t n_rows,
+                                         int32_t row_len, int64_t *packed, int64_t packed_stride, void *stream) {
+    if (!block_table || !q_offset || !q_mask || !packed) return LAZYATTN_E_NULL;
+    if (n_rows < 0 || row_len < 0 || bt_stride < row_len || row_stride < row_len || packed_stride < row_len) return LAZYATTN_E_SHAPE;
+    return launch_pack_block_table(block_table, bt_stride, q_offset, q_mask, row_stride, rows, n_rows, row_len, packed,
+                                   packed_stride, (hipStream_t)stream);
 }
 
 extern "C" int lazyattn_reposition_blocks(const lazyattn_reposition_params *p, void *stream) {

@@ -47,6 +47,30 @@ rotation_metadata_kernel(const int32_t *doc_lens, const int32_t *doc_lens_padded
     }
 }
 
+// packed[r, j] = block_table[r, j] << 32 | q_offset[r, j] << 16 | q_mask[r, j] for the listed rows
+// (rows == nullptr: rows 0 .. n_rows-1): the table the block-uniform decode kernels of the
+// reference read (worker/gpu_model_runner.py:296-340, five tensor ops per row there).
+__global__ void __launch_bounds__(256)
+pack_block_table_kernel(const int32_t *block_table, int64_t bt_stride, const int32_t *q_offset, const int32_t *q_mask,
+                        int64_t row_stride, const int32_t *rows, int row_len, int64_t *packed, int64_t packed_stride) {
+    const int r = rows ? rows[blockIdx.y] : (int)blockIdx.y;
+    const int j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= row_len) return;
+    const uint64_t blk = (uint32_t)block_table[r * bt_stride + j];
+    const uint64_t off = (uint32_t)q_offset[r * row_stride + j] & 0xffffu;
+    const uint64_t msk = (uint32_t)q_mask[r * row_stride + j] & 0xffffu;
+    packed[r * packed_stride + j] = (int64_t)((blk << 32) | (off << 16) | msk);
+}
+
+int launch_pack_block_table(const int32_t *block_table, int64_t bt_stride, const int32_t *q_offset, const int32_t *q_mask,
+                            int64_t row_stride, const int32_t *rows, int n_rows, int row_len, int64_t *packed,
+                            int64_t packed_stride, hipStream_t stream) {
+    if (n_rows <= 0 || row_len <= 0) return LAZYATTN_OK;
+    hipLaunchKernelGGL(pack_block_table_kernel, dim3((row_len + 255) / 256, n_rows), dim3(256), 0, stream, block_table, bt_stride,
+                       q_offset, q_mask, row_stride, rows, row_len, packed, packed_stride);
+    return hipGetLastError() == hipSuccess ? LAZYATTN_OK : LAZYATTN_E_LAUNCH;
+}
+
 int launch_rotation_metadata(const int32_t *doc_lens, const int32_t *doc_lens_padded, const int32_t *doc_start, int batch,
                              int block_size, int zero_offsets, int32_t *q_offset, int32_t *q_mask, int64_t row_stride,
                              int row_len, int32_t *max_offset, hipStream_t stream) {

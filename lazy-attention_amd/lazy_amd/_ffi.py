@@ -22,7 +22,7 @@ PHASE_MAIN, PHASE_COMBINE, PHASE_ALL = 1, 2, 3
 ERRORS = {-1: "NULL", -2: "SHAPE", -3: "DTYPE", -4: "UNSUPPORTED", -5: "WORKSPACE", -6: "LAUNCH"}
 EXPORTS = ("lazyattn_prefill_workspace_bytes", "lazyattn_prefix_prefill", "lazyattn_paged_decode_workspace_bytes",
            "lazyattn_paged_decode_rotary", "lazyattn_build_cos_sin_cache",
-           "lazyattn_pack_cos_sin_cache", "lazyattn_rope_and_cache_write", "lazyattn_build_rotation_metadata", "lazyattn_reposition_blocks",
+           "lazyattn_pack_cos_sin_cache", "lazyattn_rope_and_cache_write", "lazyattn_build_rotation_metadata", "lazyattn_reposition_blocks", "lazyattn_pack_block_table",
            "lazyattn_error_string", "lazyattn_abi_version")
 
 _DTYPE = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
@@ -97,6 +97,9 @@ def lib() -> C.CDLL:
                                                        C.c_void_p, C.c_void_p, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p]
         L.lazyattn_reposition_blocks.restype = C.c_int
         L.lazyattn_reposition_blocks.argtypes = [C.POINTER(RepositionParams), C.c_void_p]
+        L.lazyattn_pack_block_table.restype = C.c_int
+        L.lazyattn_pack_block_table.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_int32,
+                                                C.c_int32, C.c_void_p, C.c_int64, C.c_void_p]
         L.lazyattn_error_string.restype = C.c_char_p
         L.lazyattn_error_string.argtypes = [C.c_int]
         L.lazyattn_abi_version.restype = C.c_int

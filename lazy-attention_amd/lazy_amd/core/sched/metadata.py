@@ -75,3 +75,26 @@ def build_rotation_metadata_device(document_lens, document_lens_padded, block_si
         q_mask.data_ptr(), q_offset.stride(0), q_offset.shape[1], None if max_offset is None else max_offset.data_ptr(),
         torch.cuda.current_stream(dev).cuda_stream)
     _ffi.check(rc, "lazyattn_build_rotation_metadata")
+
+
+def pack_block_table_device(block_table, q_offset, q_mask, packed, rows=None) -> None:
+    """``packed[r, j] = block << 32 | q_offset << 16 | q_mask`` on the GPU for ``rows`` (an int32 device tensor or a
+    list; ``None`` = every row of ``packed``): ``_rebuild_packed_block_table``
+    (``lazy_attn/lazy/worker/gpu_model_runner.py:296-340``), full or delta, in one launch."""
+    import torch
+    from ... import _ffi
+    dev = packed.device
+    if dev.type != "cuda":
+        raise RuntimeError("pack_block_table_device writes a GPU buffer; there is no CPU path")
+    assert block_table.dtype == torch.int32 and q_offset.dtype == torch.int32 and q_mask.dtype == torch.int32
+    assert packed.dtype == torch.int64 and q_offset.stride() == q_mask.stride()
+    assert block_table.stride(1) == 1 and q_offset.stride(1) == 1 and packed.stride(1) == 1
+    row_len = min(packed.shape[1], block_table.shape[1], q_offset.shape[1])
+    if rows is not None and not torch.is_tensor(rows):
+        rows = torch.tensor(list(rows), dtype=torch.int32, device=dev)
+    n_rows = packed.shape[0] if rows is None else rows.numel()
+    rc = _ffi.lib().lazyattn_pack_block_table(
+        block_table.data_ptr(), block_table.stride(0), q_offset.data_ptr(), q_mask.data_ptr(), q_offset.stride(0),
+        None if rows is None else rows.data_ptr(), n_rows, row_len, packed.data_ptr(), packed.stride(0),
+        torch.cuda.current_stream(dev).cuda_stream)
+    _ffi.check(rc, "lazyattn_pack_block_table")

@@ -51,3 +51,22 @@ def test_buffers_too_small_is_refused_on_the_host():
     qo = torch.zeros(1, 4, dtype=torch.int32, device=DEV); qm = torch.zeros_like(qo)
     with pytest.raises(ValueError):
         md.build_rotation_metadata_device([[100]], [[112]], 16, qo, qm)
+
+
+def test_packed_block_table_full_and_delta():
+    print("case: packed block table", flush=True)
+    from lazy_amd.attention.ops.chunked_prefill_paged_decode import unpack_block_table
+    g = torch.Generator().manual_seed(2)
+    bt = torch.randint(0, 2 ** 31 - 1, (9, 40), generator=g, dtype=torch.int32)
+    qo = torch.randint(0, 0x10000, (9, 40), generator=g, dtype=torch.int32)
+    qm = torch.randint(0, 17, (9, 40), generator=g, dtype=torch.int32)
+    want = (bt.long() << 32) | (qo.long() << 16) | qm.long()          # gpu_model_runner.py:325-331
+    packed = torch.zeros(9, 40, dtype=torch.int64, device=DEV)
+    md.pack_block_table_device(bt.to(DEV), qo.to(DEV), qm.to(DEV), packed)
+    assert torch.equal(packed.cpu(), want)
+    blk, off, msk = unpack_block_table(packed)
+    assert torch.equal(blk.cpu(), bt) and torch.equal(off.cpu(), qo) and torch.equal(msk.cpu(), qm)
+    packed.zero_()
+    md.pack_block_table_device(bt.to(DEV), qo.to(DEV), qm.to(DEV), packed, rows=[7, 2])
+    got = packed.cpu()
+    assert torch.equal(got[[7, 2]], want[[7, 2]]) and int(got[[0, 1, 3, 4, 5, 6, 8]].abs().sum()) == 0
