@@ -392,15 +392,16 @@ bool decode_mfma_supports(const lazyattn_prefill_params &p) {
     return true;
 }
 
-// slices of the page axis per (request, kv head): enough waves to fill the chip, at least four
-// pages per slice
+// slices of the page axis per (request, kv head): enough waves to fill the chip, at least twelve
+// pages (six loop iterations) per slice -- shorter slices cost more in prologue, partials and merge
+// than they gain in parallelism (5 K keys, one request: 16-32 slices 32 us, 64 slices 43 us)
 static int decode_splits(const lazyattn_prefill_params &p) {
     if (p.num_splits > 0) return p.num_splits > 64 ? 64 : p.num_splits;
     const int64_t natural = (int64_t)p.batch * p.num_kv_heads;
     if (natural <= 0) return 1;
     int64_t s = (256 * 8 + natural - 1) / natural;
     const int64_t pages = p.max_seq_len > 0 ? (p.max_seq_len + BS - 1) / BS : 64;
-    if (s > pages / 4) s = pages / 4;
+    if (s > pages / 12) s = pages / 12;
     if (s > 64) s = 64;
     return s < 1 ? 1 : (int)s;
 }
