@@ -202,9 +202,16 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     }
     const int n_ctx_tiles = (n_pages + PAGES - 1) / PAGES;
     const int n_new_tiles = (t_end + NT - 1) / NT;
-    const int n_tiles = n_ctx_tiles + n_new_tiles;
-    const int tile_begin = (int)((int64_t)n_tiles * split / nsplit);
-    const int tile_end = (int)((int64_t)n_tiles * (split + 1) / nsplit);
+    // The key axis is cut into nsplit ranges of equal estimated cost.  A new-token tile costs about
+    // three context tiles (element-wise V scatter, per-row causal masks, branchy loads), and all of them
+    // sit at the end: with equal tile counts the last split was the tail of every launch.
+    constexpr int NEW_COST = 3;
+    const int64_t cost = n_ctx_tiles + (int64_t)NEW_COST * n_new_tiles;
+    auto tile_at = [&](int64_t c) -> int {         // first tile whose cost interval ends after c
+        return c <= n_ctx_tiles ? (int)c : n_ctx_tiles + (int)((c - n_ctx_tiles) / NEW_COST);
+    };
+    const int tile_begin = tile_at(cost * split / nsplit);
+    const int tile_end = split + 1 == nsplit ? n_ctx_tiles + n_new_tiles : tile_at(cost * (split + 1) / nsplit);
 
     // ---- page metadata, fetched ahead of its use ----
     // Gathering wave w owns page w of every tile, so it needs one block-table entry, one
@@ -732,17 +739,35 @@ prefill_combine_kernel(const lazyattn_prefill_params p, const int nsplit) {
     const int64_t T = p.num_tokens;
     const float *wo = (const float *)p.workspace;
     const float *wl = wo + (int64_t)nsplit * T * p.num_q_heads * D;
+    // splits are taken eight at a time with all loads of a batch issued before the first use: a loop
+    // of one dependent load per split would pay one memory round trip per split
+    const int64_t row0 = tok * p.num_q_heads + h, split_rows = T * p.num_q_heads;
     float mx = -INFINITY;
-    for (int s = 0; s < nsplit; ++s) mx = fmaxf(mx, wl[((int64_t)s * T + tok) * p.num_q_heads + h]);
+    for (int s0 = 0; s0 < nsplit; s0 += 8) {
+        float e[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) e[j] = wl[(int64_t)(s0 + j < nsplit ? s0 + j : nsplit - 1) * split_rows + row0];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) mx = fmaxf(mx, e[j]);
+    }
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
     float wsum = 0.f;
     if (mx != -INFINITY) {
-        for (int s = 0; s < nsplit; ++s) {
-            const int64_t ri = ((int64_t)s * T + tok) * p.num_q_heads + h;
-            const float w = __builtin_amdgcn_exp2f(wl[ri] - mx);
-            const float4 v = *reinterpret_cast<const float4 *>(wo + ri * D + d);
-            o.x = fmaf(w, v.x, o.x); o.y = fmaf(w, v.y, o.y); o.z = fmaf(w, v.z, o.z); o.w = fmaf(w, v.w, o.w);
-            wsum += w;
+        for (int s0 = 0; s0 < nsplit; s0 += 8) {
+            float e[8];
+            float4 v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int64_t ri = (int64_t)(s0 + j < nsplit ? s0 + j : nsplit - 1) * split_rows + row0;
+                e[j] = wl[ri];
+                v[j] = *reinterpret_cast<const float4 *>(wo + ri * D + d);
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float w = s0 + j < nsplit ? __builtin_amdgcn_exp2f(e[j] - mx) : 0.f;
+                o.x = fmaf(w, v[j].x, o.x); o.y = fmaf(w, v[j].y, o.y); o.z = fmaf(w, v[j].z, o.z); o.w = fmaf(w, v[j].w, o.w);
+                wsum += w;
+            }
         }
     }
     const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
