@@ -725,8 +725,16 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
 }
 
 // ---- merge split-KV partials: one 32-lane group per (token, q-head) row ----
+// The few fields the merge needs, not the whole parameter block: a launch with ~450 bytes of kernel
+// arguments costs about a microsecond more than one with 64 on this part.
+struct MergeArgs {
+    const void *workspace, *b_start_loc;
+    void *o;
+    int64_t o_stride[2];
+    int32_t num_tokens, num_q_heads, index_bits, skip_decode;
+};
 __global__ void __launch_bounds__(256)
-prefill_combine_kernel(const lazyattn_prefill_params p, const int nsplit) {
+prefill_combine_kernel(const MergeArgs p, const int nsplit) {
     const int b = blockIdx.y;
     const int64_t qs = load_index(p.b_start_loc, b, p.index_bits);
     const int64_t q_len = load_index(p.b_start_loc, b + 1, p.index_bits) - qs;
@@ -874,7 +882,9 @@ int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
     }
     if (nsplit > 1 && (phases & LAZYATTN_PHASE_COMBINE)) {
         const int64_t rows = (int64_t)p.max_q_len * p.num_q_heads;
-        hipLaunchKernelGGL(prefill_combine_kernel, dim3((unsigned)((rows + 7) / 8), p.batch), dim3(256), 0, stream, p,
+        const MergeArgs m{p.workspace, p.b_start_loc, p.o, {p.o_stride[0], p.o_stride[1]}, p.num_tokens, p.num_q_heads,
+                          p.index_bits, p.skip_decode};
+        hipLaunchKernelGGL(prefill_combine_kernel, dim3((unsigned)((rows + 7) / 8), p.batch), dim3(256), 0, stream, m,
                            nsplit);
         if (hipGetLastError() != hipSuccess) return LAZYATTN_E_LAUNCH;
     }
