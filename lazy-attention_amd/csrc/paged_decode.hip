@@ -360,33 +360,33 @@ paged_decode_merge_kernel(const DecodeMergeArgs p, const int nsplit) {
     const float *wo = (const float *)p.workspace;
     const float *wl = wo + (int64_t)nsplit * p.batch * p.num_q_heads * D;
     const int64_t rows = (int64_t)p.batch * p.num_q_heads;
-    // eight slices per batch of loads (one dependent load per slice would pay a round trip each)
-    float mx = -INFINITY;
+    // eight slices per batch, log-sum-exps and partial rows requested together: one memory round trip
+    // per batch; batches are chained by a running maximum
+    float mx = -INFINITY, wsum = 0.f;
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int s0 = 0; s0 < nsplit; s0 += 8) {
         float e[8];
+        float4 v[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) e[j] = wl[(int64_t)(s0 + j < nsplit ? s0 + j : nsplit - 1) * rows + r];
+        for (int j = 0; j < 8; ++j) {
+            const int64_t ri = (int64_t)(s0 + j < nsplit ? s0 + j : nsplit - 1) * rows + r;
+            e[j] = wl[ri];
+            v[j] = *reinterpret_cast<const float4 *>(wo + ri * D + d);
+        }
+        float bm = e[0];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) mx = fmaxf(mx, e[j]);
-    }
-    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-    float wsum = 0.f;
-    if (mx != -INFINITY) {
-        for (int s0 = 0; s0 < nsplit; s0 += 8) {
-            float e[8];
-            float4 v[8];
+        for (int j = 1; j < 8; ++j) bm = fmaxf(bm, e[j]);
+        const float m_new = fmaxf(mx, bm);
+        if (m_new == -INFINITY) continue;
+        const float keep = __builtin_amdgcn_exp2f(mx - m_new);
+        o.x *= keep; o.y *= keep; o.z *= keep; o.w *= keep;
+        wsum *= keep;
+        mx = m_new;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int64_t ri = (int64_t)(s0 + j < nsplit ? s0 + j : nsplit - 1) * rows + r;
-                e[j] = wl[ri];
-                v[j] = *reinterpret_cast<const float4 *>(wo + ri * D + d);
-            }
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const float w = s0 + j < nsplit ? __builtin_amdgcn_exp2f(e[j] - mx) : 0.f;
-                o.x = fmaf(w, v[j].x, o.x); o.y = fmaf(w, v[j].y, o.y); o.z = fmaf(w, v[j].z, o.z); o.w = fmaf(w, v[j].w, o.w);
-                wsum += w;
-            }
+        for (int j = 0; j < 8; ++j) {
+            const float w = s0 + j < nsplit ? __builtin_amdgcn_exp2f(e[j] - mx) : 0.f;
+            o.x = fmaf(w, v[j].x, o.x); o.y = fmaf(w, v[j].y, o.y); o.z = fmaf(w, v[j].z, o.z); o.w = fmaf(w, v[j].w, o.w);
+            wsum += w;
         }
     }
     const float inv = wsum > 0.f ? 1.f / wsum : 0.f;

@@ -166,7 +166,13 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     int mt, kvgrp;
     {
         const int L = blockIdx.x;
-        if ((n_groups & 7) == 0) {
+        if (((p.batch * p.num_kv_heads) & 7) == 0) {
+            // every split and m-tile of one (request, kv-head) on one XCD: they share K/V through its L2
+            const int xcd = L & 7, q = L >> 3;
+            mt = q % n_mt;
+            const int r = q / n_mt;
+            kvgrp = ((r / nsplit) * 8 + xcd) * nsplit + r % nsplit;
+        } else if ((n_groups & 7) == 0) {
             const int xcd = L & 7, q = L >> 3;
             mt = q % n_mt;
             kvgrp = (q / n_mt) * 8 + xcd;
@@ -747,35 +753,35 @@ prefill_combine_kernel(const MergeArgs p, const int nsplit) {
     const int64_t T = p.num_tokens;
     const float *wo = (const float *)p.workspace;
     const float *wl = wo + (int64_t)nsplit * T * p.num_q_heads * D;
-    // splits are taken eight at a time with all loads of a batch issued before the first use: a loop
-    // of one dependent load per split would pay one memory round trip per split
+    // Splits are taken eight at a time, log-sum-exps and partial rows of a batch requested together and
+    // before the first use: one memory round trip per eight splits.  Batches are chained like the
+    // tiles of the main kernel, by a running maximum.
     const int64_t row0 = tok * p.num_q_heads + h, split_rows = T * p.num_q_heads;
-    float mx = -INFINITY;
+    float mx = -INFINITY, wsum = 0.f;
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int s0 = 0; s0 < nsplit; s0 += 8) {
         float e[8];
+        float4 v[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) e[j] = wl[(int64_t)(s0 + j < nsplit ? s0 + j : nsplit - 1) * split_rows + row0];
+        for (int j = 0; j < 8; ++j) {
+            const int64_t ri = (int64_t)(s0 + j < nsplit ? s0 + j : nsplit - 1) * split_rows + row0;
+            e[j] = wl[ri];
+            v[j] = *reinterpret_cast<const float4 *>(wo + ri * D + d);
+        }
+        float bm = e[0];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) mx = fmaxf(mx, e[j]);
-    }
-    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-    float wsum = 0.f;
-    if (mx != -INFINITY) {
-        for (int s0 = 0; s0 < nsplit; s0 += 8) {
-            float e[8];
-            float4 v[8];
+        for (int j = 1; j < 8; ++j) bm = fmaxf(bm, e[j]);
+        const float m_new = fmaxf(mx, bm);
+        if (m_new == -INFINITY) continue;                    // nothing visible so far
+        const float keep = __builtin_amdgcn_exp2f(mx - m_new);   // mx = -inf -> 0
+        o.x *= keep; o.y *= keep; o.z *= keep; o.w *= keep;
+        wsum *= keep;
+        mx = m_new;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int64_t ri = (int64_t)(s0 + j < nsplit ? s0 + j : nsplit - 1) * split_rows + row0;
-                e[j] = wl[ri];
-                v[j] = *reinterpret_cast<const float4 *>(wo + ri * D + d);
-            }
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const float w = s0 + j < nsplit ? __builtin_amdgcn_exp2f(e[j] - mx) : 0.f;
-                o.x = fmaf(w, v[j].x, o.x); o.y = fmaf(w, v[j].y, o.y); o.z = fmaf(w, v[j].z, o.z); o.w = fmaf(w, v[j].w, o.w);
-                wsum += w;
-            }
+        for (int j = 0; j < 8; ++j) {
+            const float w = s0 + j < nsplit ? __builtin_amdgcn_exp2f(e[j] - mx) : 0.f;
+            o.x = fmaf(w, v[j].x, o.x); o.y = fmaf(w, v[j].y, o.y); o.z = fmaf(w, v[j].z, o.z); o.w = fmaf(w, v[j].w, o.w);
+            wsum += w;
         }
     }
     const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
