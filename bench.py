@@ -27,7 +27,7 @@ PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
 # WRITE_SIZE, each scaled by what the same counter reads for a 256 MiB copy; summary under profiles/).
 # Counters cannot be read from inside this script, so the figure is the committed measurement of the
 # named workload; workloads without one report null.
-MEASURED_TRAFFIC_BYTES = {"c2_8b_bf16_10x512_q128": 49_600_000, "d1_8b_bf16_decode_32req_20x256": 683_700_000}
+MEASURED_TRAFFIC_BYTES = {"c2_8b_bf16_10x512_q128": 51_700_000, "d1_8b_bf16_decode_32req_20x256": 683_700_000}
 PEAK_HBM_GBS = 8000.0
 
 
@@ -194,6 +194,61 @@ def bench_rope_write(a):
     print(json.dumps(out))
 
 
+def bench_reposition(a):
+    """Copy-on-write re-positioning of shared blocks (the per-block loop of the reference's block-attention
+    model runner): 2 048 blocks of one layer copied to new blocks, their keys moved from one rotation
+    position to another.  One launch."""
+    import torch
+    from oracle import deferred_rope as orc
+    from lazy_amd.block_attn import utils as ba
+    n, hkv, d, bs = 2048, 8, 128, 16
+    gen = torch.Generator().manual_seed(6)
+    nb = 2 * n
+    kc = torch.randn(nb, hkv, d // 8, bs, 8, generator=gen).to(torch.bfloat16).cuda()
+    vc = torch.randn(nb, hkv, d, bs, generator=gen).to(torch.bfloat16).cuda()
+    table = orc.build_cos_sin_table(n * bs + 4096 + bs, d, 500000.0).to(torch.bfloat16).cuda()
+    perm = torch.randperm(n, generator=gen)
+    items = torch.stack([n + torch.arange(n), perm, perm * bs % 4096, torch.arange(n) * bs], 1).int()
+    items_dev = items.cuda()
+
+    class Plan:
+        def run(self):
+            ba.reposition_blocks(kc, vc, items_dev, table)
+    plan = Plan()
+    for _ in range(a.warmup):
+        plan.run()
+    torch.cuda.synchronize()
+    ms = time_calls(plan, a.steps)
+    nbytes = n * hkv * d * bs * 2 * 2 * 2              # K and V of every block, read and written
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    out = {
+        "metric": "block re-positioning (copy + un-rotate + rotate): GB/s read+written, 8B geometry, 2048 blocks",
+        "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "r1_8b_bf16_reposition_2048blocks", "hkv": hkv, "head_dim": d, "page": bs,
+                   "blocks": n, "mb_per_call": round(nbytes / 1e6, 2)},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None, "kernel": "block_reposition_kernel",
+                     "kernel_ms": round(ms, 5)},
+    }
+    if not a.no_cpu:
+        torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))
+        ns = 256
+        kcc, vcc, tc = kc.cpu(), vc.cpu(), table.cpu()
+        sample = [tuple(int(x) for x in row) for row in items[:ns]]
+        ts = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            orc.reposition_blocks(kcc, vcc, sample, tc)
+            ts.append(time.perf_counter() - t0)
+        sec = statistics.median(ts)
+        out["cpu_baseline"] = {"value": round(nbytes * ns / n / sec / 1e9, 3), "unit": "GB/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"first {ns} of the {n} blocks, 3 calls, median {sec * 1e3:.1f} ms"}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -202,9 +257,10 @@ def main():
     ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5])
     ap.add_argument("--num-splits", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--path", choices=["prefill", "decode", "rope_write"], default="prefill",
+    ap.add_argument("--path", choices=["prefill", "decode", "rope_write", "reposition"], default="prefill",
                     help="prefill: the headline prefix-prefill call (default); decode: the q_len==1 kernel; "
-                         "rope_write: Q rotary + paged-cache write of the new tokens (both HBM-bound)")
+                         "rope_write: Q rotary + paged-cache write of the new tokens; reposition: copy-on-write block "
+                         "re-positioning (all three HBM-bound)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a 256 MiB device-to-device copy (known traffic, for scaling profiler counters)")
     a = ap.parse_args()
@@ -224,6 +280,8 @@ def main():
         return bench_decode(a)
     if a.path == "rope_write":
         return bench_rope_write(a)
+    if a.path == "reposition":
+        return bench_reposition(a)
     w = wl.config(a.config)
     g = w.to("cuda:0")
     plan, o = make_plan(g, a.num_splits, _ffi.PHASE_ALL)
