@@ -35,6 +35,7 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
 
 constexpr int D = 128;          // head_dim
 constexpr int HALF = 64;
@@ -713,20 +714,37 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                                pack_bf16(acc[dt][4 * i4 + 2] * inv, acc[dt][4 * i4 + 3] * inv));
             }
     } else {
+        // Partial row = 128 halves sharing one power-of-two scale (the row's largest |O/l| lands in
+        // [0.5, 1)) + (log2-sum-exp, scale) as two floats: half the bytes of an fp32 row, written by every
+        // workgroup at the same moment and read back by the merge, for an error of at most 2^-12 of the
+        // row's largest element -- an eighth of the rounding of the bf16 output.
+        float am = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; i += 2) am = max3(am, fabsf(acc[dt][i]), fabsf(acc[dt][i + 1]));
+        am = fmaxf(am, partner32(am, gh != 0)) * inv;
+        uint32_t eb = (__float_as_uint(am) >> 23) & 0xffu;           // biased exponent: am in [2^(eb-127), 2^(eb-126))
+        eb = eb > 252u ? 252u : eb;
+        const float down = __uint_as_float((253u - eb) << 23) * inv;   // 2^-(eb-126) / l
+        const float up = __uint_as_float((eb + 1u) << 23);            // 2^(eb-126)
         const int64_t T = p.num_tokens;
-        float *wo = (float *)p.workspace;
-        float *wl = wo + (int64_t)nsplit * T * p.num_q_heads * D;
+        _Float16 *wo = (_Float16 *)p.workspace;
+        float2 *wl = reinterpret_cast<float2 *>(wo + (int64_t)nsplit * T * p.num_q_heads * D);
         const int64_t r_idx = ((int64_t)split * T + (qs + row)) * p.num_q_heads + h;
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) {
                 const int d = dt * 32 + 8 * i4 + 4 * gh;
-                *reinterpret_cast<float4 *>(wo + r_idx * D + d) =
-                    make_float4(acc[dt][4 * i4] * inv, acc[dt][4 * i4 + 1] * inv, acc[dt][4 * i4 + 2] * inv,
-                                acc[dt][4 * i4 + 3] * inv);
+                const f32x2_t lo = {acc[dt][4 * i4] * down, acc[dt][4 * i4 + 1] * down};
+                const f32x2_t hi = {acc[dt][4 * i4 + 2] * down, acc[dt][4 * i4 + 3] * down};
+                const f16x2_t hl = __builtin_convertvector(lo, f16x2_t), hh = __builtin_convertvector(hi, f16x2_t);   // RNE
+                *reinterpret_cast<uint2 *>(wo + r_idx * D + d) =
+                    make_uint2(*reinterpret_cast<const uint32_t *>(&hl), *reinterpret_cast<const uint32_t *>(&hh));
             }
-        if (gh == 0) wl[r_idx] = l_run > 0.f ? m_run * cs2 + __builtin_amdgcn_logf(l_run) : -INFINITY;
+        if (gh == 0)
+            wl[r_idx] = make_float2(l_run > 0.f ? m_run * cs2 + __builtin_amdgcn_logf(l_run) : -INFINITY, up);
     }
 }
 
@@ -751,8 +769,8 @@ prefill_combine_kernel(const MergeArgs p, const int nsplit) {
     const int h = (int)(r % p.num_q_heads);
     const int d = (threadIdx.x & 31) * 4;
     const int64_t T = p.num_tokens;
-    const float *wo = (const float *)p.workspace;
-    const float *wl = wo + (int64_t)nsplit * T * p.num_q_heads * D;
+    const _Float16 *wo = (const _Float16 *)p.workspace;
+    const float2 *wl = reinterpret_cast<const float2 *>(wo + (int64_t)nsplit * T * p.num_q_heads * D);
     // Splits are taken eight at a time, log-sum-exps and partial rows of a batch requested together and
     // before the first use: one memory round trip per eight splits.  Batches are chained like the
     // tiles of the main kernel, by a running maximum.
@@ -760,17 +778,17 @@ prefill_combine_kernel(const MergeArgs p, const int nsplit) {
     float mx = -INFINITY, wsum = 0.f;
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int s0 = 0; s0 < nsplit; s0 += 8) {
-        float e[8];
-        float4 v[8];
+        float2 e[8];                                         // (log2-sum-exp, scale of the row's halves)
+        uint2 v[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int64_t ri = (int64_t)(s0 + j < nsplit ? s0 + j : nsplit - 1) * split_rows + row0;
             e[j] = wl[ri];
-            v[j] = *reinterpret_cast<const float4 *>(wo + ri * D + d);
+            v[j] = *reinterpret_cast<const uint2 *>(wo + ri * D + d);
         }
-        float bm = e[0];
+        float bm = e[0].x;
 #pragma unroll
-        for (int j = 1; j < 8; ++j) bm = fmaxf(bm, e[j]);
+        for (int j = 1; j < 8; ++j) bm = fmaxf(bm, e[j].x);
         const float m_new = fmaxf(mx, bm);
         if (m_new == -INFINITY) continue;                    // nothing visible so far
         const float keep = __builtin_amdgcn_exp2f(mx - m_new);   // mx = -inf -> 0
@@ -779,8 +797,11 @@ prefill_combine_kernel(const MergeArgs p, const int nsplit) {
         mx = m_new;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            const float w = s0 + j < nsplit ? __builtin_amdgcn_exp2f(e[j] - mx) : 0.f;
-            o.x = fmaf(w, v[j].x, o.x); o.y = fmaf(w, v[j].y, o.y); o.z = fmaf(w, v[j].z, o.z); o.w = fmaf(w, v[j].w, o.w);
+            const float w = s0 + j < nsplit ? __builtin_amdgcn_exp2f(e[j].x - mx) : 0.f;
+            const float ws = w * e[j].y;
+            const f16x2_t lo = *reinterpret_cast<const f16x2_t *>(&v[j].x), hi = *reinterpret_cast<const f16x2_t *>(&v[j].y);
+            o.x = fmaf(ws, (float)lo[0], o.x); o.y = fmaf(ws, (float)lo[1], o.y);
+            o.z = fmaf(ws, (float)hi[0], o.z); o.w = fmaf(ws, (float)hi[1], o.w);
             wsum += w;
         }
     }
@@ -790,6 +811,8 @@ prefill_combine_kernel(const MergeArgs p, const int nsplit) {
 }
 
 // ------------------------------------------------------------------ host side
+// a split-KV partial row: 128 halves + (log2-sum-exp, scale)
+constexpr size_t PARTIAL_ROW_BYTES = D * sizeof(_Float16) + 2 * sizeof(float);
 static int mfma_units(const lazyattn_prefill_params &p) {
     const int group = p.num_q_heads / p.num_kv_heads;
     return ((p.max_q_len + UNIT - 1) / UNIT) * group;
@@ -844,7 +867,7 @@ size_t mfma_workspace_bytes(const lazyattn_prefill_params &p) {
     const int nw = mfma_waves(p);
     const int ns = mfma_splits(p, nw);
     if (ns <= 1) return 0;
-    return (size_t)ns * (size_t)p.num_tokens * p.num_q_heads * (D + 1) * sizeof(float);
+    return (size_t)ns * (size_t)p.num_tokens * p.num_q_heads * PARTIAL_ROW_BYTES;
 }
 
 template <int NC, bool FP8, typename TT>
@@ -878,7 +901,7 @@ int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
     const int n_mt = mfma_mtiles(p, nw);
     const int phases = p.phases ? p.phases : LAZYATTN_PHASE_ALL;
     if (nsplit > 1) {
-        const size_t need = (size_t)nsplit * (size_t)p.num_tokens * p.num_q_heads * (D + 1) * sizeof(float);
+        const size_t need = (size_t)nsplit * (size_t)p.num_tokens * p.num_q_heads * PARTIAL_ROW_BYTES;
         if (!p.workspace || (size_t)p.workspace_bytes < need) return LAZYATTN_E_WORKSPACE;
         if (((uintptr_t)p.workspace) & 15) return LAZYATTN_E_WORKSPACE;
     }
