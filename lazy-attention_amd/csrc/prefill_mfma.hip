@@ -513,6 +513,11 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     // Q^T fragments: B operand of S^T = K.Q^T, lane = (row l32, d = ks*16 + gh*8 .. +8).
     // They live in this wave's own LDS slice (not in registers: three waves share a SIMD's
     // register file) and are re-read for every tile.
+    // Q is multiplied by sm_scale * log2(e) here, once, and rounded to bf16 again: the MFMA then
+    // delivers the scores in log2 units and no per-score multiply is left in the tile loop (the
+    // reference scales the fp32 scores, old_ops:287; the extra rounding of Q is one more relative
+    // 2^-9 per element, like the one the rotated K already carries).
+    const float cs2 = p.sm_scale * 1.4426950408889634f;
     uint8_t *qlds = lds + KV_BYTES + wave * 8192 + lane * 16;
     {
         const bf16_t *qp = (const bf16_t *)p.q + (qs + row) * p.q_stride[0] + (int64_t)h * p.q_stride[1] + gh * 8;
@@ -520,11 +525,24 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         for (int ks = 0; ks < 8; ++ks) {
             uint4 v = make_uint4(0, 0, 0, 0);
             if (row_ok) v = *reinterpret_cast<const uint4 *>(qp + ks * 16);
-            *reinterpret_cast<uint4 *>(qlds + ks * 1024) = v;
+            float f[8];
+            unpack8(v, f);
+            *reinterpret_cast<uint4 *>(qlds + ks * 1024) =
+                make_uint4(pack_bf16(f[0] * cs2, f[1] * cs2), pack_bf16(f[2] * cs2, f[3] * cs2),
+                           pack_bf16(f[4] * cs2, f[5] * cs2), pack_bf16(f[6] * cs2, f[7] * cs2));
         }
     }
-    const float cs2 = p.sm_scale * 1.4426950408889634f;          // scores -> log2 units
-    float m_run = -INFINITY, l_run = 0.f, l_alt = 0.f;              // row sum kept as two chains
+    // Online softmax against a reference m_ref per row that moves rarely.  The MFMA accumulators of S^T
+    // start at -m_ref, so the scores arrive already relative to it and P = exp2(S) needs no subtraction.
+    // m_ref is moved (and O, l rescaled, old_ops:287-291) only when a row's tile maximum exceeds it by more
+    // than REBASE, or when the row sees its first valid key; in between P may exceed 1 (by at most
+    // 2^REBASE), which fp32 accumulation and bf16's exponent range carry without loss.
+    constexpr float REBASE = 16.f;
+    float m_ref = 0.f, l_run = 0.f, l_alt = 0.f;                    // row sum kept as two chains
+    bool seen = false;                                              // the row has had a valid key
+    f32x16_t cinit;                                                 // -m_ref in every element
+#pragma unroll
+    for (int i = 0; i < 16; ++i) cinit[i] = 0.f;
     f32x16_t acc[4];
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt)
@@ -533,16 +551,14 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
 
     // ---- S^T = K . Q^T for one 64-key tile: two independent 32-key accumulation chains ----
     auto qk_tile = [&](const uint8_t *ktile, f32x16_t &s0, f32x16_t &s1) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) { s0[i] = 0.f; s1[i] = 0.f; }
         const uint8_t *kp = ktile + (l32 >> 4) * K_PAGE + gh * 256 + (l32 & 15) * 16;
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
             const bf16x8_t a0 = *reinterpret_cast<const bf16x8_t *>(kp + ks * 512);
             const bf16x8_t a1 = *reinterpret_cast<const bf16x8_t *>(kp + 2 * K_PAGE + ks * 512);
             const bf16x8_t q = *reinterpret_cast<const bf16x8_t *>(qlds + ks * 1024);
-            s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, q, s0, 0, 0, 0);
-            s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, q, s1, 0, 0, 0);
+            s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, q, ks ? s0 : cinit, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, q, ks ? s1 : cinit, 0, 0, 0);
         }
     };
     // ---- masks: register i of half `sub` holds key sub*32 + 8*(i/4) + 4*gh + i%4 ----
@@ -557,32 +573,36 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             s[i] = ok ? s[i] : -INFINITY;
         }
     };
-    // ---- running max over the tile, rescale of the accumulators when it grew (old_ops:287-291) ----
-    auto update_max = [&](const f32x16_t &s0, const f32x16_t &s1) -> float {
+    // ---- tile maximum per row; move the reference if a row needs it (rare after its first tile) ----
+    auto rebase = [&](f32x16_t &s0, f32x16_t &s1) {
         // v_maximum3_f32: no quieting pre-pass over the MFMA results, NaN scores stay NaN
         float ma = max3(s0[0], s0[1], s0[2]), mb = max3(s1[0], s1[1], s1[2]);
 #pragma unroll
         for (int i = 3; i < 15; i += 2) { ma = max3(ma, s0[i], s0[i + 1]); mb = max3(mb, s1[i], s1[i + 1]); }
         float mx = max3(ma, mb, s0[15]);
         mx = max3(mx, s1[15], s1[15]);
-        mx = max3(mx, partner32(mx, gh != 0), mx);
-        const float m_new = fmaxf(m_run, mx);
-        const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f((m_run - m_safe) * cs2);          // m_run = -inf -> 0
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
+        mx = max3(mx, partner32(mx, gh != 0), mx);                  // relative to m_ref; -inf: no valid key in this tile
+        const bool valid = mx > -INFINITY;                          // false for NaN too: NaN rows stay NaN below
+        const float delta = (valid && (!seen || mx > REBASE)) ? mx : 0.f;
+        if (__builtin_amdgcn_ballot_w64(delta != 0.f)) {
+            const float alpha = seen ? __builtin_amdgcn_exp2f(-delta) : 1.f;   // nothing accumulated before the first key
 #pragma unroll
             for (int dt = 0; dt < 4; ++dt) acc[dt] *= alpha;
             l_run *= alpha;
             l_alt *= alpha;
+            s0 -= delta;
+            s1 -= delta;
+            m_ref += delta;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) cinit[i] = -m_ref;
         }
-        m_run = m_new;
-        return m_safe * cs2;
+        seen = seen || valid;
     };
-    // ---- P = exp2(S*cs2 - mc) for 32 keys, packed as the two B operands of the PV steps ----
-    auto exp_half = [&](const f32x16_t &s, float mc, bf16x8_t &p0, bf16x8_t &p1) {
+    // ---- P = exp2(S) for 32 keys (S is relative to m_ref), packed as the two B operands of the PV steps ----
+    auto exp_half = [&](const f32x16_t &s, bf16x8_t &p0, bf16x8_t &p1) {
         float pr[16];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) pr[i] = __builtin_amdgcn_exp2f(fmaf(s[i], cs2, -mc));
+        for (int i = 0; i < 16; ++i) pr[i] = __builtin_amdgcn_exp2f(s[i]);
         uint32_t w[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) w[i] = pack_bf16(pr[2 * i], pr[2 * i + 1]);
@@ -609,12 +629,12 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, p1, acc[dt], 0, 0, 0);
         }
     };
-    auto attend = [&](const uint8_t *vtile, const f32x16_t &s0, const f32x16_t &s1) {
-        const float mc = update_max(s0, s1);
+    auto attend = [&](const uint8_t *vtile, f32x16_t &s0, f32x16_t &s1) {
+        rebase(s0, s1);
         bf16x8_t p0, p1, p2, p3;
-        exp_half(s0, mc, p0, p1);
+        exp_half(s0, p0, p1);
         pv_half(vtile, 0, p0, p1);
-        exp_half(s1, mc, p2, p3);
+        exp_half(s1, p2, p3);
         pv_half(vtile, 1, p2, p3);
     };
 
@@ -744,7 +764,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                     make_uint2(*reinterpret_cast<const uint32_t *>(&hl), *reinterpret_cast<const uint32_t *>(&hh));
             }
         if (gh == 0)
-            wl[r_idx] = make_float2(l_run > 0.f ? m_run * cs2 + __builtin_amdgcn_logf(l_run) : -INFINITY, up);
+            wl[r_idx] = make_float2(l_run > 0.f ? m_ref + __builtin_amdgcn_logf(l_run) : -INFINITY, up);
     }
 }
 
