@@ -67,6 +67,31 @@ def test_mfma_vanilla_requests():
     assert e < 2e-2, e
 
 
+@pytest.mark.parametrize("nsplit", [1, 2])
+def test_mfma_softmax_reference_moves_down_then_far_up(nsplit):
+    """Un-rotated requests, so the scores are under control: every query row is 3u, the first 64 cached keys
+    of every request are -3u (scores of about -150 in log2 units, the first tile's maximum), a later page
+    is +u (about +50, far above everything before).  The kernel's softmax reference first settles on the
+    very negative first tile, then jumps by ~150 and again by ~50; the early keys end with weight ~0."""
+    print(f"case: mfma softmax reference jumps nsplit={nsplit}", flush=True)
+    w = _ragged("block_uniform")
+    lazy = torch.zeros(5, dtype=torch.bool)
+    u = torch.ones(128)
+    w.q[:] = (3.0 * u).to(w.q.dtype)
+    hkv, x = w.k_cache.shape[1], w.k_cache.shape[4]
+    for b in range(4):
+        n_ctx = int(w.b_seq_len[b]) - int(w.b_start_loc[b + 1] - w.b_start_loc[b])
+        for j in range(min(4, n_ctx // 16)):
+            w.k_cache[int(w.block_table[b, j])] = (-3.0 * u).view(128 // x, 1, x).expand(hkv, 128 // x, 16, x).to(w.k_cache.dtype)
+        if n_ctx // 16 > 9:
+            w.k_cache[int(w.block_table[b, 9])] = u.view(128 // x, 1, x).expand(hkv, 128 // x, 16, x).to(w.k_cache.dtype)
+    ref = run_oracle(w, is_lazy=lazy)
+    got = run_op(w.to(DEV), kernel=_ffi.KERNEL_MFMA, num_splits=nsplit, is_lazy=lazy.to(DEV)).cpu()
+    assert torch.isfinite(got.float()).all()
+    e = _err(got, ref)
+    assert e < 2e-2, e
+
+
 @pytest.mark.parametrize("table_f32", [False, True])
 def test_mfma_fp8_cache(table_f32):
     print(f"case: mfma fp8 table_f32={table_f32}", flush=True)
