@@ -16,9 +16,10 @@
 //            (old_ops/prefix_prefill.py:248-257 with FORCE_FP32_ROTARY), write to LDS in
 //            the cache's own [page][D/8][slot][8] order, which is exactly the A-operand
 //            order of v_mfma_f32_32x32x16_bf16;
-//   S^T      = K . Q^T (keys x rows) in two 32-key halves, Q fragments stay in registers;
-//   softmax  per lane one query row; row max via one v_permlane32_swap; exp2 with
-//            sm_scale*log2(e) folded into one fma (old_ops:287-291);
+//   S^T      = K . Q^T (keys x rows) in two 32-key halves, Q fragments re-read from LDS;
+//   softmax  per lane one query row; Q carries sm_scale*log2(e) and the accumulators start at
+//            minus a per-row reference, so P = exp2(S) directly; the row max (one
+//            v_permlane32_swap) only decides when that reference moves (old_ops:287-291);
 //   O^T     += V^T . P^T: the S^T accumulator registers ARE the B operand (the k index of
 //            the MFMA is permuted so that no shuffle is needed), V^T comes from LDS.
 // Tiles come in three kinds: full context tiles (no masking code at all), edge context
