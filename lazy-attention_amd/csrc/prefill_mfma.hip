@@ -258,6 +258,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     if (gatherer) {
         // ====================================================================== gather
         const int gw = wave - NC;                                // this wave's page of every tile
+        const int nat_step = (vanilla || pos_mode == LAZYATTN_POS_BLOCK_UNIFORM) ? 0 : BS;
         const bool rot_new = p.rotate_new_k && !vanilla;
         const float k_scale = FP8 ? *p.k_scale : 1.f;
         const float v_scale = FP8 ? *p.v_scale : 1.f;
@@ -294,12 +295,11 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         auto issue_loads_ctx = [&](int tile, const PageMeta &pm) {
             const int j = tile * PAGES + gw;
             const uint8_t *kb = kc_base + pm.bt * kc_page_bytes;
-            // un-rotated requests read row 0 of the table (cos 1, sin 0): exact identity
-            const int nat = j * BS;                                                  // old_ops:183-184
-            int pos0 = pos_mode == LAZYATTN_POS_NATURAL ? nat
-                     : pos_mode == LAZYATTN_POS_OFFSET ? (pm.qo ? pm.qo - 1 : nat)      // old_ops:186-191
-                                                       : (pm.qo ? pm.qo - 1 : 0);       // ops:180-186
-            pos0 = vanilla ? 0 : pos0;
+            // Position of the page's first slot.  Natural: j*16 (old_ops:183-184); offset: q_offset-1 if
+            // set, else natural (old_ops:186-191); block-uniform: q_offset-1 if set, else 0 (ops:180-186);
+            // un-rotated requests read row 0 of the table (cos 1, sin 0): exact identity.  pm.qo is 0
+            // wherever q_offset is not consulted, nat_step is 0 wherever the fallback is row 0.
+            const int pos0 = pm.qo ? pm.qo - 1 : j * nat_step;
             const uint8_t *tb = ctab_base + (int64_t)pos0 * pos_bytes;
 #pragma unroll
             for (int i = 0; i < KI; ++i) {
