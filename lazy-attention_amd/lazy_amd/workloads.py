@@ -120,7 +120,8 @@ def make_workload(name: str, *, dtype: torch.dtype, hq: int, hkv: int, d: int,
     new_pages = [(ql + bs - 1) // bs for ql in q_lens]
     nb = sum(doc_pages) + sum(new_pages) + spare_blocks
     perm = torch.randperm(nb, generator=gen)
-    max_pos = max(c + ql for c, ql in zip(ctx_lens, q_lens)) + bs
+    # rows for every request position and (rotated-cache variant) every document-local position
+    max_pos = max(max(c + ql for c, ql in zip(ctx_lens, q_lens)), max(padded)) + bs
     table = cos_sin_table(max_pos, d, theta, dtype, llama3)
     table_f32 = table.float()
 

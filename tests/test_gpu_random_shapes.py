@@ -1,0 +1,53 @@
+"""Randomised ragged batches through the operators against the CPU oracle: document lengths, request
+composition, new-token counts, GQA group, split count, position mode and cache type are drawn from a
+seeded generator (the reference's own tests sweep fixed grids, tests/kernels/test_prefix_prefill.py:27-60;
+the draws here reach the corners in between: documents shorter than a page, requests with no context,
+one-token requests next to long ones, tiles that end inside a page)."""
+import random
+
+import pytest
+import torch
+
+from lazy_amd import _ffi, workloads as wl
+from opcall import run_op, run_oracle
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _draw(seed):
+    r = random.Random(seed)
+    hkv = r.choice([1, 2, 4, 8])
+    group = r.choice([1, 2, 4, 8])
+    n_docs = r.randint(1, 7)
+    doc_lens = [r.choice([1, 5, 15, 16, 17, 31, 48, 63, 64, 65, 100, 129, 200, 333]) for _ in range(n_docs)]
+    n_req = r.randint(1, 5)
+    requests = []
+    for _ in range(n_req):
+        k = r.randint(0, min(4, n_docs))
+        requests.append(r.sample(range(n_docs), k))
+    q_lens = [r.choice([1, 2, 7, 31, 32, 33, 64, 70, 129]) for _ in range(n_req)]
+    variant = r.choice(["natural", "offset", "block_uniform"])
+    kv = r.choice(["auto", "auto", "fp8"])
+    nsplit = r.choice([0, 1, 2, 3, 5])
+    kernel = r.choice([_ffi.KERNEL_MFMA4, _ffi.KERNEL_MFMA8, _ffi.KERNEL_AUTO])
+    return dict(hq=hkv * group, hkv=hkv, doc_lens=doc_lens, requests=requests, q_lens=q_lens, variant=variant,
+                kv=kv, nsplit=nsplit, kernel=kernel)
+
+
+@pytest.mark.parametrize("seed", range(64))
+def test_random_ragged_batch(seed):
+    c = _draw(1000 + seed)
+    print(f"case: random batch seed={seed} {c}", flush=True)
+    w = wl.make_workload("rand", dtype=torch.bfloat16, hq=c["hq"], hkv=c["hkv"], d=128, theta=500000.0, block_size=16,
+                         doc_lens=c["doc_lens"], requests=c["requests"], q_lens=c["q_lens"], variant=c["variant"],
+                         kv_cache_dtype=c["kv"], seed=seed)
+    lazy = None
+    if c["variant"] == "block_uniform":
+        lazy = torch.tensor([(seed + b) % 3 != 0 for b in range(len(c["q_lens"]))])
+    ref = run_oracle(w, **({"is_lazy": lazy} if lazy is not None else {}))
+    got = run_op(w.to(DEV), kernel=c["kernel"], num_splits=c["nsplit"],
+                 is_lazy=None if lazy is None else lazy.to(DEV)).cpu()
+    assert torch.isfinite(got.float()).all()
+    err = (got.float() - ref.float()).abs().max().item()
+    assert err < (5e-2 if c["kv"] == "fp8" else 2e-2), err
