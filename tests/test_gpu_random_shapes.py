@@ -51,3 +51,27 @@ def test_random_ragged_batch(seed):
     assert torch.isfinite(got.float()).all()
     err = (got.float() - ref.float()).abs().max().item()
     assert err < (5e-2 if c["kv"] == "fp8" else 2e-2), err
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_decode_batch(seed):
+    """The q_len == 1 rows through the decode launch: every key, the new token included, sits in the paged
+    cache when the call is made; requests with more than one new token must be left alone."""
+    from oracle import deferred_rope as orc
+    import test_gpu_decode as dec
+    r = random.Random(5000 + seed)
+    hkv = r.choice([1, 2, 8])
+    group = r.choice([1, 2, 4, 8, 16])
+    variant = r.choice(["natural", "block_uniform"])
+    kv = r.choice(["auto", "auto", "fp8"])
+    q_lens = tuple(r.choice([1, 1, 1, 3]) for _ in range(5))
+    nsplit = r.choice([0, 1, 2, 5, 9])
+    print(f"case: random decode seed={seed} hkv={hkv} group={group} {variant} kv={kv} q_lens={q_lens} nsplit={nsplit}",
+          flush=True)
+    w = dec._decode_batch(variant, hq=hkv * group, hkv=hkv, q_lens=q_lens, seed=seed, kv=kv)
+    lazy = torch.tensor([(seed + b) % 4 != 0 for b in range(5)]) if variant == "block_uniform" else None
+    ref = dec._oracle(w, lazy)
+    got = dec._run(w, lazy=lazy, num_splits=nsplit)
+    assert torch.isfinite(got.float()).all()
+    err = (got.float() - ref.float()).abs().max().item()
+    assert err < (5e-2 if kv == "fp8" else 2e-2), err
