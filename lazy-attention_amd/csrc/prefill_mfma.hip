@@ -553,6 +553,10 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     // ---- S^T = K . Q^T for one 64-key tile: two independent 32-key accumulation chains ----
     auto qk_tile = [&](const uint8_t *ktile, f32x16_t &s0, f32x16_t &s1) {
         const uint8_t *kp = ktile + (l32 >> 4) * K_PAGE + gh * 256 + (l32 & 15) * 16;
+        // A wave in a matrix phase goes first on its SIMD: its MFMAs are issued the moment the pipe is
+        // free and the vector work of the other waves fills the cycles in between (measured: -3 % on
+        // long key ranges against equal priorities).
+        __builtin_amdgcn_s_setprio(2);
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
             const bf16x8_t a0 = *reinterpret_cast<const bf16x8_t *>(kp + ks * 512);
@@ -561,6 +565,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, q, ks ? s0 : cinit, 0, 0, 0);
             s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, q, ks ? s1 : cinit, 0, 0, 0);
         }
+        __builtin_amdgcn_s_setprio(0);
     };
     // ---- masks: register i of half `sub` holds key sub*32 + 8*(i/4) + 4*gh + i%4 ----
     auto mask_half = [&](f32x16_t &s, uint32_t vbits, int sub, int kind, int m0) {
@@ -634,9 +639,11 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         rebase(s0, s1);
         bf16x8_t p0, p1, p2, p3;
         exp_half(s0, p0, p1);
+        __builtin_amdgcn_s_setprio(2);
         pv_half(vtile, 0, p0, p1);
         exp_half(s1, p2, p3);
         pv_half(vtile, 1, p2, p3);
+        __builtin_amdgcn_s_setprio(0);
     };
 
     // The two computing waves that share a SIMD (w and w + NC/2) run half a tile apart: the early one
