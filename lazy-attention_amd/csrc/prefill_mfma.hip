@@ -52,8 +52,7 @@ constexpr int K_TILE = PAGES * K_PAGE;
 constexpr int V_G = 2048;
 constexpr int V_PAGE = 2 * V_G;
 constexpr int V_TILE = PAGES * V_PAGE;
-constexpr int NVB = 3;                              // V tiles in LDS: the late computing waves read a tile one step longer
-constexpr int KV_BYTES = 2 * K_TILE + NVB * V_TILE;   // 80 KB
+constexpr int KV_BYTES = 2 * K_TILE + 2 * V_TILE;     // K and V tiles, double-buffered: 64 KB
 
 enum { TILE_FULL = 0, TILE_EDGE = 1, TILE_NEW = 2 };
 
@@ -450,9 +449,9 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             }
         };
         // tile + its page limit -> LDS buffer `buf`
-        auto store_tile = [&](int buf, int vbuf, int kind, int lim) {
+        auto store_tile = [&](int buf, int kind, int lim) {
             store_k(lds + buf * K_TILE, kind);
-            store_v(lds + 2 * K_TILE + vbuf * V_TILE, kind, lim);
+            store_v(lds + 2 * K_TILE + buf * V_TILE, kind, lim);
             if (lane == 0) page_lims[buf * PAGES + gw] = lim;
         };
 
@@ -465,7 +464,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             const PageMeta pm0 = load_page(tile_begin * PAGES + gw);
             const PageMeta pm1 = load_page((tile_begin + 1) * PAGES + gw);
             const int k0 = issue_loads(tile_begin, pm0);
-            store_tile(0, 0, k0, pm0.lim);
+            store_tile(0, k0, pm0.lim);
             if (tile_begin + 1 < tile_end) {
                 nxt_kind = issue_loads(tile_begin + 1, pm1);
                 nxt_lim = pm1.lim;
@@ -473,23 +472,20 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         }
         __syncthreads();
         int tile = tile_begin;
-        int vnx = 1;                                            // V buffer of tile + 1
         while (tile < tile_end) {
             // steady state: this wave's pages of tile+1 (in registers) and tile+2 (to load) are full context pages
             while (tile + 2 < n_ctx_tiles && tile + 2 < tile_end && nxt_kind == TILE_FULL && pm_pend.lim == BS) {
                 const int cur = (tile - tile_begin) & 1;
                 const PageMeta pm_new = load_page((tile + 3) * PAGES + gw);      // scalar loads, land during the rotation
-                store_tile(cur ^ 1, vnx, TILE_FULL, BS);
+                store_tile(cur ^ 1, TILE_FULL, BS);
                 issue_loads_ctx(tile + 2, pm_pend);
                 pm_pend = pm_new;
-                vnx = vnx == NVB - 1 ? 0 : vnx + 1;
                 ++tile;
                 __syncthreads();
             }
             if (tile >= tile_end) break;
             const int cur = (tile - tile_begin) & 1;
-            if (tile + 1 < tile_end) store_tile(cur ^ 1, vnx, nxt_kind, nxt_lim);
-            vnx = vnx == NVB - 1 ? 0 : vnx + 1;
+            if (tile + 1 < tile_end) store_tile(cur ^ 1, nxt_kind, nxt_lim);
             int new_kind = TILE_FULL;
             if (tile + 2 < tile_end) new_kind = issue_loads(tile + 2, pm_pend);
             nxt_kind = new_kind;
@@ -646,12 +642,6 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         __builtin_amdgcn_s_setprio(0);
     };
 
-    // The two computing waves that share a SIMD (w and w + NC/2) run half a tile apart: the early one
-    // does S = K.Q^T, softmax and P.V of a tile within one barrier interval; the late one first does
-    // the softmax and P.V of the previous tile and then S of the current one, so that one wave's
-    // matrix phase falls on the other's vector phase.  The late waves read V of tile t-1 while V of
-    // tile t+1 is being written: three V buffers.
-    const bool late = NC == 8 && wave >= NC / 2;
     // which of the tile's 64 keys exist: new-token tiles from the token count, context tiles from the
     // page limits the gathering waves left beside the tile
     struct Desc { int kind; uint32_t vlo, vhi; int m0; };
@@ -675,54 +665,24 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         return td;
     };
     __syncthreads();
-    if (!late) {
-        int vb = 0;
-        for (int tile = tile_begin; tile < tile_end; ++tile) {
-            const int cur = (tile - tile_begin) & 1;
-            const uint8_t *ktile = lds + cur * K_TILE;
-            const uint8_t *vtile = lds + 2 * K_TILE + vb * V_TILE;
-            const Desc td = describe(tile, cur);
-            // One call site for the tile body: the accumulators keep their registers round the loop.
-            // Rows of an idle wave are all-zero queries (harmless, never stored); a new-token tile
-            // entirely in this wave's future contributes nothing (causal) and is skipped.
-            if (td.kind != TILE_NEW || td.m0 <= t0 + UNIT - 1) {
-                f32x16_t s0, s1;
-                qk_tile(ktile, s0, s1);
-                if (td.kind != TILE_FULL) {
-                    mask_half(s0, td.vlo, 0, td.kind, td.m0);
-                    mask_half(s1, td.vhi, 1, td.kind, td.m0);
-                }
-                attend(vtile, s0, s1);
+    for (int tile = tile_begin; tile < tile_end; ++tile) {
+        const int cur = (tile - tile_begin) & 1;
+        const uint8_t *ktile = lds + cur * K_TILE;
+        const uint8_t *vtile = lds + 2 * K_TILE + cur * V_TILE;
+        const Desc td = describe(tile, cur);
+        // One call site for the tile body: the accumulators keep their registers round the loop.
+        // Rows of an idle wave are all-zero queries (harmless, never stored); a new-token tile
+        // entirely in this wave's future contributes nothing (causal) and is skipped.
+        if (td.kind != TILE_NEW || td.m0 <= t0 + UNIT - 1) {
+            f32x16_t s0, s1;
+            qk_tile(ktile, s0, s1);
+            if (td.kind != TILE_FULL) {
+                mask_half(s0, td.vlo, 0, td.kind, td.m0);
+                mask_half(s1, td.vhi, 1, td.kind, td.m0);
             }
-            vb = vb == NVB - 1 ? 0 : vb + 1;
-            __syncthreads();
+            attend(vtile, s0, s1);
         }
-    } else {
-        int vb = 0;
-        bool pend = false;                                       // scores of the previous tile wait in s0, s1
-        const uint8_t *pend_v = lds;
-        f32x16_t s0, s1;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) { s0[i] = 0.f; s1[i] = 0.f; }
-        for (int tile = tile_begin; tile < tile_end; ++tile) {
-            if (pend) attend(pend_v, s0, s1);
-            pend = false;
-            const int cur = (tile - tile_begin) & 1;
-            const uint8_t *ktile = lds + cur * K_TILE;
-            const Desc td = describe(tile, cur);
-            if (td.kind != TILE_NEW || td.m0 <= t0 + UNIT - 1) {
-                qk_tile(ktile, s0, s1);
-                if (td.kind != TILE_FULL) {
-                    mask_half(s0, td.vlo, 0, td.kind, td.m0);
-                    mask_half(s1, td.vhi, 1, td.kind, td.m0);
-                }
-                pend = true;
-                pend_v = lds + 2 * K_TILE + vb * V_TILE;
-            }
-            vb = vb == NVB - 1 ? 0 : vb + 1;
-            __syncthreads();
-        }
-        if (pend) attend(pend_v, s0, s1);
+        __syncthreads();
     }
 
     // ---- epilogue ----
