@@ -553,13 +553,22 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         // free and the vector work of the other waves fills the cycles in between (measured: -3 % on
         // long key ranges against equal priorities).
         __builtin_amdgcn_s_setprio(2);
+        // operands are requested two k-steps ahead of their MFMAs (a ring of three sets): one step ahead
+        // leaves the LDS latency exposed in every step
+        bf16x8_t a0[3], a1[3], q[3];
+        auto fetch = [&](int ks) {
+            a0[ks % 3] = *reinterpret_cast<const bf16x8_t *>(kp + ks * 512);
+            a1[ks % 3] = *reinterpret_cast<const bf16x8_t *>(kp + 2 * K_PAGE + ks * 512);
+            q[ks % 3] = *reinterpret_cast<const bf16x8_t *>(qlds + ks * 1024);
+        };
+        fetch(0);
+        fetch(1);
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
-            const bf16x8_t a0 = *reinterpret_cast<const bf16x8_t *>(kp + ks * 512);
-            const bf16x8_t a1 = *reinterpret_cast<const bf16x8_t *>(kp + 2 * K_PAGE + ks * 512);
-            const bf16x8_t q = *reinterpret_cast<const bf16x8_t *>(qlds + ks * 1024);
-            s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, q, ks ? s0 : cinit, 0, 0, 0);
-            s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, q, ks ? s1 : cinit, 0, 0, 0);
+            if (ks + 2 < 8) fetch(ks + 2);
+            s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0[ks % 3], q[ks % 3], ks ? s0 : cinit, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1[ks % 3], q[ks % 3], ks ? s1 : cinit, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
         __builtin_amdgcn_s_setprio(0);
     };
@@ -620,15 +629,16 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     // k index j of a 16-key step <-> slot 4*gh + j (j < 4), 8 + 4*gh + j - 4 (j >= 4)
     auto pv_half = [&](const uint8_t *vtile, int sub, const bf16x8_t &p0, const bf16x8_t &p1) {
         const uint8_t *vp = vtile + (sub * 2) * V_PAGE + gh * V_G + l32 * 16;
+        // eight MFMAs: 32-row blocks of d 0..3 for the first page of the half, then for the second;
+        // their V^T operands are requested two MFMAs ahead
+        bf16x8_t a[3];
+        auto fetch = [&](int j) { a[j % 3] = *reinterpret_cast<const bf16x8_t *>(vp + (j >> 2) * V_PAGE + (j & 3) * 512); };
+        fetch(0);
+        fetch(1);
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt) {
-            const bf16x8_t a = *reinterpret_cast<const bf16x8_t *>(vp + dt * 512);
-            acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, p0, acc[dt], 0, 0, 0);
-        }
-#pragma unroll
-        for (int dt = 0; dt < 4; ++dt) {
-            const bf16x8_t a = *reinterpret_cast<const bf16x8_t *>(vp + V_PAGE + dt * 512);
-            acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, p1, acc[dt], 0, 0, 0);
+        for (int j = 0; j < 8; ++j) {
+            if (j + 2 < 8) fetch(j + 2);
+            acc[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[j % 3], j < 4 ? p0 : p1, acc[j & 3], 0, 0, 0);
         }
     };
     auto attend = [&](const uint8_t *vtile, f32x16_t &s0, f32x16_t &s1) {
