@@ -67,6 +67,22 @@ def test_mfma_vanilla_requests():
     assert e < 2e-2, e
 
 
+@pytest.mark.parametrize("scale", [1e-6, 3e4])
+def test_mfma_split_partials_keep_their_precision_at_any_magnitude(scale):
+    """Split-KV partial rows are stored as halves with one power-of-two scale per row: values far outside
+    the half range (here V of the order 1e-6 and 3e4) must come through with bf16-level relative error."""
+    print(f"case: mfma partial rows, value scale {scale}", flush=True)
+    w = wl.make_workload("vscale", dtype=torch.bfloat16, **GEOM, doc_lens=[100, 16, 333, 70, 5, 250],
+                         requests=[[3, 1, 0], [2], [0, 2, 3, 1, 5]], q_lens=[70, 9, 33], variant="natural",
+                         seed=5, value_scale=1.0)
+    w.v_cache.mul_(scale)
+    w.v.mul_(scale)
+    ref = run_oracle(w)
+    got = run_op(w.to(DEV), kernel=_ffi.KERNEL_MFMA, num_splits=4).cpu()
+    rel = ((got.float() - ref.float()).abs().max() / ref.float().abs().max()).item()
+    assert rel < 1e-2, rel
+
+
 @pytest.mark.parametrize("nsplit", [1, 2])
 def test_mfma_softmax_reference_moves_down_then_far_up(nsplit):
     """Un-rotated requests, so the scores are under control: every query row is 3u, the first 64 cached keys
