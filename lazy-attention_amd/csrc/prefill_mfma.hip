@@ -37,6 +37,7 @@ typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 typedef __attribute__((ext_vector_type(2))) float f32x2_t;
 typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
 
 constexpr int D = 128;          // head_dim
 constexpr int HALF = 64;
@@ -56,24 +57,54 @@ constexpr int KV_BYTES = 2 * K_TILE + 2 * V_TILE;     // K and V tiles, double-b
 
 enum { TILE_FULL = 0, TILE_EDGE = 1, TILE_NEW = 2 };
 
-__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
-__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
-__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
-    f32x2_t f = {a, b};
-    bf16x2_t h = __builtin_convertvector(f, bf16x2_t);   // v_cvt_pk_bf16_f32, RNE
-    return *reinterpret_cast<uint32_t *>(&h);
-}
+// The two 16-bit element types of the matrix path.  Values travel as 32-bit words holding two elements;
+// `mfma` is v_mfma_f32_32x32x16_{bf16,f16} on 8-element operands given as four such words.
+template <typename T> struct Elem;
+template <> struct Elem<bf16_t> {
+    // largest P = 2^REBASE between two moves of the softmax reference: anything bf16's exponent carries
+    static constexpr float REBASE = 16.f;
+    static __device__ __forceinline__ float lo(uint32_t w) { return __uint_as_float(w << 16); }
+    static __device__ __forceinline__ float hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+    static __device__ __forceinline__ uint32_t pack(float a, float b) {
+        f32x2_t f = {a, b};
+        bf16x2_t h = __builtin_convertvector(f, bf16x2_t);   // v_cvt_pk_bf16_f32, RNE
+        return *reinterpret_cast<uint32_t *>(&h);
+    }
+    static __device__ __forceinline__ uint32_t splat(float w) { const uint32_t u = __float_as_uint(w) >> 16; return u | (u << 16); }
+    // acc + lo(w) + hi(w) (v_dot2c_f32_bf16 against (1, 1))
+    static __device__ __forceinline__ float dot2_ones(uint32_t w, float acc) {
+        const uint32_t one = 0x3f803f80u;
+        return __builtin_amdgcn_fdot2_f32_bf16(*reinterpret_cast<const bf16x2_t *>(&w),
+                                               *reinterpret_cast<const bf16x2_t *>(&one), acc, false);
+    }
+    static __device__ __forceinline__ f32x16_t mfma(const uint4 &a, const uint4 &b, const f32x16_t &c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8_t *>(&a),
+                                                       *reinterpret_cast<const bf16x8_t *>(&b), c, 0, 0, 0);
+    }
+};
+template <> struct Elem<f16_t> {
+    static constexpr float REBASE = 8.f;                      // P <= 256: far inside the half range
+    static __device__ __forceinline__ float lo(uint32_t w) { return (float)(*reinterpret_cast<const f16x2_t *>(&w))[0]; }
+    static __device__ __forceinline__ float hi(uint32_t w) { return (float)(*reinterpret_cast<const f16x2_t *>(&w))[1]; }
+    static __device__ __forceinline__ uint32_t pack(float a, float b) {
+        f32x2_t f = {a, b};
+        f16x2_t h = __builtin_convertvector(f, f16x2_t);     // RNE
+        return *reinterpret_cast<uint32_t *>(&h);
+    }
+    static __device__ __forceinline__ uint32_t splat(float w) { return pack(w, w); }
+    static __device__ __forceinline__ float dot2_ones(uint32_t w, float acc) {
+        const uint32_t one = 0x3c003c00u;
+        return __builtin_amdgcn_fdot2(*reinterpret_cast<const f16x2_t *>(&w), *reinterpret_cast<const f16x2_t *>(&one), acc, false);
+    }
+    static __device__ __forceinline__ f32x16_t mfma(const uint4 &a, const uint4 &b, const f32x16_t &c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<const f16x8_t *>(&a),
+                                                      *reinterpret_cast<const f16x8_t *>(&b), c, 0, 0, 0);
+    }
+};
 // value of x in the partner lane (lane ^ 32) of the wave, via v_permlane32_swap
 // IEEE-754 maximum of three (v_maximum3_f32): NaN-propagating, so no canonicalising pre-pass
 __device__ __forceinline__ float max3(float a, float b, float c) {
     return __builtin_elementwise_maximum(__builtin_elementwise_maximum(a, b), c);
-}
-// acc + lo(w) + hi(w) for a packed bf16 pair (v_dot2c_f32_bf16 against (1, 1))
-__device__ __forceinline__ float dot2_ones(uint32_t w, float acc) {
-    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
-    const uint32_t one = 0x3f803f80u;
-    return __builtin_amdgcn_fdot2_f32_bf16(*reinterpret_cast<const bf16x2_t *>(&w),
-                                           *reinterpret_cast<const bf16x2_t *>(&one), acc, false);
 }
 __device__ __forceinline__ float partner32(float x, bool upper) {
     uint32_t a = __float_as_uint(x), b = a;
@@ -92,17 +123,13 @@ __device__ __forceinline__ uint2 ldg8(const uint8_t *base, uint32_t off) {
 }
 
 // 8 consecutive cos (or sin) table entries
-template <typename TT> struct TabVec;
-template <> struct TabVec<bf16_t> {
+template <typename TT> struct TabVec {                     // a 16-bit table
     uint4 v;
     __device__ __forceinline__ void load(const uint8_t *base, uint32_t off) { v = ldg16(base, off); }
-    __device__ __forceinline__ void fill(float w) {
-        const uint32_t u = __float_as_uint(w) >> 16;
-        v = make_uint4(u | (u << 16), u | (u << 16), u | (u << 16), u | (u << 16));
-    }
+    __device__ __forceinline__ void fill(float w) { const uint32_t u = Elem<TT>::splat(w); v = make_uint4(u, u, u, u); }
     __device__ __forceinline__ void get(float *f) const {
-        f[0] = bf16_lo(v.x); f[1] = bf16_hi(v.x); f[2] = bf16_lo(v.y); f[3] = bf16_hi(v.y);
-        f[4] = bf16_lo(v.z); f[5] = bf16_hi(v.z); f[6] = bf16_lo(v.w); f[7] = bf16_hi(v.w);
+        f[0] = Elem<TT>::lo(v.x); f[1] = Elem<TT>::hi(v.x); f[2] = Elem<TT>::lo(v.y); f[3] = Elem<TT>::hi(v.y);
+        f[4] = Elem<TT>::lo(v.z); f[5] = Elem<TT>::hi(v.z); f[6] = Elem<TT>::lo(v.w); f[7] = Elem<TT>::hi(v.w);
     }
 };
 template <> struct TabVec<float> {
@@ -117,17 +144,17 @@ template <> struct TabVec<float> {
     }
 };
 
-__device__ __forceinline__ void unpack8(const uint4 &w, float *f) {
-    f[0] = bf16_lo(w.x); f[1] = bf16_hi(w.x); f[2] = bf16_lo(w.y); f[3] = bf16_hi(w.y);
-    f[4] = bf16_lo(w.z); f[5] = bf16_hi(w.z); f[6] = bf16_lo(w.w); f[7] = bf16_hi(w.w);
+template <typename T> __device__ __forceinline__ void unpack8(const uint4 &w, float *f) {
+    f[0] = Elem<T>::lo(w.x); f[1] = Elem<T>::hi(w.x); f[2] = Elem<T>::lo(w.y); f[3] = Elem<T>::hi(w.y);
+    f[4] = Elem<T>::lo(w.z); f[5] = Elem<T>::hi(w.z); f[6] = Elem<T>::lo(w.w); f[7] = Elem<T>::hi(w.w);
 }
-// 8 fp8 e4m3 bytes -> (float * scale) rounded to bf16, as floats  (old_ops:239-241)
-__device__ __forceinline__ void unpack8_fp8(uint32_t lo, uint32_t hi, float scale, float *f) {
+// 8 fp8 e4m3 bytes -> (float * scale) rounded to the query type, as floats  (old_ops:239-241)
+template <typename T> __device__ __forceinline__ void unpack8_fp8(uint32_t lo, uint32_t hi, float scale, float *f) {
     const f32x2_t a = __builtin_amdgcn_cvt_pk_f32_fp8(lo, false), b = __builtin_amdgcn_cvt_pk_f32_fp8(lo >> 16, false);
     const f32x2_t c = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false), d = __builtin_amdgcn_cvt_pk_f32_fp8(hi >> 16, false);
     const float t[8] = {a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
 #pragma unroll
-    for (int i = 0; i < 8; ++i) f[i] = round_to<bf16_t>(t[i] * scale);
+    for (int i = 0; i < 8; ++i) f[i] = round_to<T>(t[i] * scale);
 }
 
 // one K item in flight: 8 (d, d+64) pairs of one key
@@ -151,11 +178,12 @@ constexpr int lds_bytes(int nc) { return KV_BYTES + nc * 8 * 1024 + 2 * PAGES * 
 constexpr int KI = 2;                    // K items per gathering lane and tile: a page has 128 (8 chunks x 16 slots)
 constexpr int VI = 4;                    // V items per gathering lane and tile: a page has 256 of 16 bytes
 
-template <int NC, bool FP8, typename TT>
+template <int NC, bool FP8, typename T, typename TT>
 __global__ void __launch_bounds__((NC + 4) * 64)
 prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int n_mt) {
     constexpr int VI_CTX = FP8 ? VI / 2 : VI;        // an fp8 page row of 16 slots is one 16-byte item
     constexpr uint32_t TSZ = sizeof(TT);
+    using E = Elem<T>;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -329,7 +357,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                 kr[i].k1 = make_uint4(0, 0, 0, 0); kr[i].k2 = kr[i].k1;
                 kr[i].c.fill(1.f); kr[i].s.fill(0.f);
                 if (m < t_end) {
-                    const bf16_t *kn = (const bf16_t *)p.k + (qs + m) * p.k_stride[0] + (int64_t)g * p.k_stride[1] + cp * 8;
+                    const T *kn = (const T *)p.k + (qs + m) * p.k_stride[0] + (int64_t)g * p.k_stride[1] + cp * 8;
                     kr[i].k1 = *reinterpret_cast<const uint4 *>(kn);
                     kr[i].k2 = *reinterpret_cast<const uint4 *>(kn + HALF);
                     if (rot_new) {                                               // old_ops:342-343
@@ -345,7 +373,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                 const int dc = idx & 15, m = m0 + (idx >> 4);
                 vr[i] = make_uint4(0, 0, 0, 0);
                 if (m < t_end)
-                    vr[i] = *reinterpret_cast<const uint4 *>((const bf16_t *)p.v + (qs + m) * p.v_stride[0] +
+                    vr[i] = *reinterpret_cast<const uint4 *>((const T *)p.v + (qs + m) * p.v_stride[0] +
                                                              (int64_t)g * p.v_stride[1] + dc * 8);
             }
         };
@@ -366,11 +394,11 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             for (int i = 0; i < KI; ++i) {
                 float a[8], bb[8], cs[8], sn[8];
                 if (FP8 && kind != TILE_NEW) {
-                    unpack8_fp8(kr[i].k1.x, kr[i].k1.y, k_scale, a);
-                    unpack8_fp8(kr[i].k2.x, kr[i].k2.y, k_scale, bb);
+                    unpack8_fp8<T>(kr[i].k1.x, kr[i].k1.y, k_scale, a);
+                    unpack8_fp8<T>(kr[i].k2.x, kr[i].k2.y, k_scale, bb);
                 } else {
-                    unpack8(kr[i].k1, a);
-                    unpack8(kr[i].k2, bb);
+                    unpack8<T>(kr[i].k1, a);
+                    unpack8<T>(kr[i].k2, bb);
                 }
                 kr[i].c.get(cs);
                 kr[i].s.get(sn);
@@ -381,9 +409,9 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                     y[e] = a[e] * sn[e] + bb[e] * cs[e];                             // old_ops:254
                 }
                 *reinterpret_cast<uint4 *>(ktile + kr[i].lds_off) = make_uint4(
-                    pack_bf16(x[0], x[1]), pack_bf16(x[2], x[3]), pack_bf16(x[4], x[5]), pack_bf16(x[6], x[7]));
+                    E::pack(x[0], x[1]), E::pack(x[2], x[3]), E::pack(x[4], x[5]), E::pack(x[6], x[7]));
                 *reinterpret_cast<uint4 *>(ktile + kr[i].lds_off + 8 * 256) = make_uint4(
-                    pack_bf16(y[0], y[1]), pack_bf16(y[2], y[3]), pack_bf16(y[4], y[5]), pack_bf16(y[6], y[7]));
+                    E::pack(y[0], y[1]), E::pack(y[2], y[3]), E::pack(y[4], y[5]), E::pack(y[6], y[7]));
             }
         };
         // ---- write the V items to a V tile; lim = valid slots of the page ----
@@ -423,8 +451,8 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                             for (int s = 0; s < 4; ++s)
                                 if (q4 * 4 + s >= lim) f[s] = 0.f;   // masked slots contribute nothing, whatever they hold
                         }
-                        o2[q4][0] = pack_bf16(f[0], f[1]);
-                        o2[q4][1] = pack_bf16(f[2], f[3]);
+                        o2[q4][0] = E::pack(f[0], f[1]);
+                        o2[q4][1] = E::pack(f[2], f[3]);
                     }
                     uint8_t *dst = vtile + gw * V_PAGE + d * 16;
                     *reinterpret_cast<uint4 *>(dst) = make_uint4(o2[0][0], o2[0][1], o2[2][0], o2[2][1]);
@@ -517,16 +545,16 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     const float cs2 = p.sm_scale * 1.4426950408889634f;
     uint8_t *qlds = lds + KV_BYTES + wave * 8192 + lane * 16;
     {
-        const bf16_t *qp = (const bf16_t *)p.q + (qs + row) * p.q_stride[0] + (int64_t)h * p.q_stride[1] + gh * 8;
+        const T *qp = (const T *)p.q + (qs + row) * p.q_stride[0] + (int64_t)h * p.q_stride[1] + gh * 8;
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
             uint4 v = make_uint4(0, 0, 0, 0);
             if (row_ok) v = *reinterpret_cast<const uint4 *>(qp + ks * 16);
             float f[8];
-            unpack8(v, f);
+            unpack8<T>(v, f);
             *reinterpret_cast<uint4 *>(qlds + ks * 1024) =
-                make_uint4(pack_bf16(f[0] * cs2, f[1] * cs2), pack_bf16(f[2] * cs2, f[3] * cs2),
-                           pack_bf16(f[4] * cs2, f[5] * cs2), pack_bf16(f[6] * cs2, f[7] * cs2));
+                make_uint4(E::pack(f[0] * cs2, f[1] * cs2), E::pack(f[2] * cs2, f[3] * cs2),
+                           E::pack(f[4] * cs2, f[5] * cs2), E::pack(f[6] * cs2, f[7] * cs2));
         }
     }
     // Online softmax against a reference m_ref per row that moves rarely.  The MFMA accumulators of S^T
@@ -534,7 +562,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     // m_ref is moved (and O, l rescaled, old_ops:287-291) only when a row's tile maximum exceeds it by more
     // than REBASE, or when the row sees its first valid key; in between P may exceed 1 (by at most
     // 2^REBASE), which fp32 accumulation and bf16's exponent range carry without loss.
-    constexpr float REBASE = 16.f;
+    constexpr float REBASE = E::REBASE;
     float m_ref = 0.f, l_run = 0.f, l_alt = 0.f;                    // row sum kept as two chains
     bool seen = false;                                              // the row has had a valid key
     f32x16_t cinit;                                                 // -m_ref in every element
@@ -555,19 +583,19 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         __builtin_amdgcn_s_setprio(2);
         // operands are requested two k-steps ahead of their MFMAs (a ring of three sets): one step ahead
         // leaves the LDS latency exposed in every step
-        bf16x8_t a0[3], a1[3], q[3];
+        uint4 a0[3], a1[3], q[3];
         auto fetch = [&](int ks) {
-            a0[ks % 3] = *reinterpret_cast<const bf16x8_t *>(kp + ks * 512);
-            a1[ks % 3] = *reinterpret_cast<const bf16x8_t *>(kp + 2 * K_PAGE + ks * 512);
-            q[ks % 3] = *reinterpret_cast<const bf16x8_t *>(qlds + ks * 1024);
+            a0[ks % 3] = *reinterpret_cast<const uint4 *>(kp + ks * 512);
+            a1[ks % 3] = *reinterpret_cast<const uint4 *>(kp + 2 * K_PAGE + ks * 512);
+            q[ks % 3] = *reinterpret_cast<const uint4 *>(qlds + ks * 1024);
         };
         fetch(0);
         fetch(1);
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
             if (ks + 2 < 8) fetch(ks + 2);
-            s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0[ks % 3], q[ks % 3], ks ? s0 : cinit, 0, 0, 0);
-            s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1[ks % 3], q[ks % 3], ks ? s1 : cinit, 0, 0, 0);
+            s0 = E::mfma(a0[ks % 3], q[ks % 3], ks ? s0 : cinit);
+            s1 = E::mfma(a1[ks % 3], q[ks % 3], ks ? s1 : cinit);
             __builtin_amdgcn_sched_barrier(0);
         }
         __builtin_amdgcn_s_setprio(0);
@@ -610,40 +638,38 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         seen = seen || valid;
     };
     // ---- P = exp2(S) for 32 keys (S is relative to m_ref), packed as the two B operands of the PV steps ----
-    auto exp_half = [&](const f32x16_t &s, bf16x8_t &p0, bf16x8_t &p1) {
+    auto exp_half = [&](const f32x16_t &s, uint4 &p0, uint4 &p1) {
         float pr[16];
 #pragma unroll
         for (int i = 0; i < 16; ++i) pr[i] = __builtin_amdgcn_exp2f(s[i]);
         uint32_t w[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) w[i] = pack_bf16(pr[2 * i], pr[2 * i + 1]);
+        for (int i = 0; i < 8; ++i) w[i] = E::pack(pr[2 * i], pr[2 * i + 1]);
         // row sum of the rounded probabilities, two per instruction (old_ops:312 sums them unrounded)
 #pragma unroll
-        for (int i = 0; i < 8; i += 2) { l_run = dot2_ones(w[i], l_run); l_alt = dot2_ones(w[i + 1], l_alt); }
-        uint4 w0 = make_uint4(w[0], w[1], w[2], w[3]);
-        uint4 w1 = make_uint4(w[4], w[5], w[6], w[7]);
-        p0 = *reinterpret_cast<bf16x8_t *>(&w0);
-        p1 = *reinterpret_cast<bf16x8_t *>(&w1);
+        for (int i = 0; i < 8; i += 2) { l_run = E::dot2_ones(w[i], l_run); l_alt = E::dot2_ones(w[i + 1], l_alt); }
+        p0 = make_uint4(w[0], w[1], w[2], w[3]);
+        p1 = make_uint4(w[4], w[5], w[6], w[7]);
     };
     // ---- O^T += V^T . P^T for 32 keys (pages 2*sub, 2*sub+1 of the tile) ----
     // k index j of a 16-key step <-> slot 4*gh + j (j < 4), 8 + 4*gh + j - 4 (j >= 4)
-    auto pv_half = [&](const uint8_t *vtile, int sub, const bf16x8_t &p0, const bf16x8_t &p1) {
+    auto pv_half = [&](const uint8_t *vtile, int sub, const uint4 &p0, const uint4 &p1) {
         const uint8_t *vp = vtile + (sub * 2) * V_PAGE + gh * V_G + l32 * 16;
         // eight MFMAs: 32-row blocks of d 0..3 for the first page of the half, then for the second;
         // their V^T operands are requested two MFMAs ahead
-        bf16x8_t a[3];
-        auto fetch = [&](int j) { a[j % 3] = *reinterpret_cast<const bf16x8_t *>(vp + (j >> 2) * V_PAGE + (j & 3) * 512); };
+        uint4 a[3];
+        auto fetch = [&](int j) { a[j % 3] = *reinterpret_cast<const uint4 *>(vp + (j >> 2) * V_PAGE + (j & 3) * 512); };
         fetch(0);
         fetch(1);
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             if (j + 2 < 8) fetch(j + 2);
-            acc[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[j % 3], j < 4 ? p0 : p1, acc[j & 3], 0, 0, 0);
+            acc[j & 3] = E::mfma(a[j % 3], j < 4 ? p0 : p1, acc[j & 3]);
         }
     };
     auto attend = [&](const uint8_t *vtile, f32x16_t &s0, f32x16_t &s1) {
         rebase(s0, s1);
-        bf16x8_t p0, p1, p2, p3;
+        uint4 p0, p1, p2, p3;
         exp_half(s0, p0, p1);
         __builtin_amdgcn_s_setprio(2);
         pv_half(vtile, 0, p0, p1);
@@ -701,15 +727,15 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     if (!row_ok) return;
     const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
     if (nsplit == 1) {
-        bf16_t *op = (bf16_t *)p.o + (qs + row) * p.o_stride[0] + (int64_t)h * p.o_stride[1];
+        T *op = (T *)p.o + (qs + row) * p.o_stride[0] + (int64_t)h * p.o_stride[1];
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) {
                 const int d = dt * 32 + 8 * i4 + 4 * gh;
                 *reinterpret_cast<uint2 *>(op + d) =
-                    make_uint2(pack_bf16(acc[dt][4 * i4] * inv, acc[dt][4 * i4 + 1] * inv),
-                               pack_bf16(acc[dt][4 * i4 + 2] * inv, acc[dt][4 * i4 + 3] * inv));
+                    make_uint2(E::pack(acc[dt][4 * i4] * inv, acc[dt][4 * i4 + 1] * inv),
+                               E::pack(acc[dt][4 * i4 + 2] * inv, acc[dt][4 * i4 + 3] * inv));
             }
     } else {
         // Partial row = 128 halves sharing one power-of-two scale (the row's largest |O/l| lands in
@@ -726,10 +752,10 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         eb = eb > 252u ? 252u : eb;
         const float down = __uint_as_float((253u - eb) << 23) * inv;   // 2^-(eb-126) / l
         const float up = __uint_as_float((eb + 1u) << 23);            // 2^(eb-126)
-        const int64_t T = p.num_tokens;
+        const int64_t NTOK = p.num_tokens;
         _Float16 *wo = (_Float16 *)p.workspace;
-        float2 *wl = reinterpret_cast<float2 *>(wo + (int64_t)nsplit * T * p.num_q_heads * D);
-        const int64_t r_idx = ((int64_t)split * T + (qs + row)) * p.num_q_heads + h;
+        float2 *wl = reinterpret_cast<float2 *>(wo + (int64_t)nsplit * NTOK * p.num_q_heads * D);
+        const int64_t r_idx = ((int64_t)split * NTOK + (qs + row)) * p.num_q_heads + h;
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
@@ -755,8 +781,10 @@ struct MergeArgs {
     int64_t o_stride[2];
     int32_t num_tokens, num_q_heads, index_bits, skip_decode;
 };
+template <typename T>
 __global__ void __launch_bounds__(256)
 prefill_combine_kernel(const MergeArgs p, const int nsplit) {
+    using E = Elem<T>;
     const int b = blockIdx.y;
     const int64_t qs = load_index(p.b_start_loc, b, p.index_bits);
     const int64_t q_len = load_index(p.b_start_loc, b + 1, p.index_bits) - qs;
@@ -766,13 +794,13 @@ prefill_combine_kernel(const MergeArgs p, const int nsplit) {
     const int64_t tok = qs + r / p.num_q_heads;
     const int h = (int)(r % p.num_q_heads);
     const int d = (threadIdx.x & 31) * 4;
-    const int64_t T = p.num_tokens;
+    const int64_t NTOK = p.num_tokens;
     const _Float16 *wo = (const _Float16 *)p.workspace;
-    const float2 *wl = reinterpret_cast<const float2 *>(wo + (int64_t)nsplit * T * p.num_q_heads * D);
+    const float2 *wl = reinterpret_cast<const float2 *>(wo + (int64_t)nsplit * NTOK * p.num_q_heads * D);
     // Splits are taken eight at a time, log-sum-exps and partial rows of a batch requested together and
     // before the first use: one memory round trip per eight splits.  Batches are chained like the
     // tiles of the main kernel, by a running maximum.
-    const int64_t row0 = tok * p.num_q_heads + h, split_rows = T * p.num_q_heads;
+    const int64_t row0 = tok * p.num_q_heads + h, split_rows = NTOK * p.num_q_heads;
     float mx = -INFINITY, wsum = 0.f;
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int s0 = 0; s0 < nsplit; s0 += 8) {
@@ -804,8 +832,8 @@ prefill_combine_kernel(const MergeArgs p, const int nsplit) {
         }
     }
     const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
-    bf16_t *op = (bf16_t *)p.o + tok * p.o_stride[0] + (int64_t)h * p.o_stride[1] + d;
-    *reinterpret_cast<uint2 *>(op) = make_uint2(pack_bf16(o.x * inv, o.y * inv), pack_bf16(o.z * inv, o.w * inv));
+    T *op = (T *)p.o + tok * p.o_stride[0] + (int64_t)h * p.o_stride[1] + d;
+    *reinterpret_cast<uint2 *>(op) = make_uint2(E::pack(o.x * inv, o.y * inv), E::pack(o.z * inv, o.w * inv));
 }
 
 // ------------------------------------------------------------------ host side
@@ -841,9 +869,9 @@ static int mfma_splits(const lazyattn_prefill_params &p, int nw) {
 
 bool mfma_supports(const lazyattn_prefill_params &p) {
     const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3;
-    if (p.dtype != LAZYATTN_BF16) return false;
-    if (!(p.cache_dtype == LAZYATTN_BF16 || fp8)) return false;
-    if (p.table_dtype != LAZYATTN_BF16 && p.table_dtype != LAZYATTN_F32) return false;
+    if (p.dtype != LAZYATTN_BF16 && p.dtype != LAZYATTN_F16) return false;
+    if (!(p.cache_dtype == p.dtype || fp8)) return false;
+    if (p.table_dtype != p.dtype && p.table_dtype != LAZYATTN_F32) return false;
     if (p.head_dim != D || p.block_size != BS || p.x != (fp8 ? 16 : 8)) return false;
     if (p.sliding_window > 0) return false;
     if (p.q_stride[2] != 1 || p.k_stride[2] != 1 || p.v_stride[2] != 1 || p.o_stride[2] != 1) return false;
@@ -868,9 +896,9 @@ size_t mfma_workspace_bytes(const lazyattn_prefill_params &p) {
     return (size_t)ns * (size_t)p.num_tokens * p.num_q_heads * PARTIAL_ROW_BYTES;
 }
 
-template <int NC, bool FP8, typename TT>
+template <int NC, bool FP8, typename T, typename TT>
 static int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt, hipStream_t stream) {
-    auto kern = prefill_mfma_kernel<NC, FP8, TT>;
+    auto kern = prefill_mfma_kernel<NC, FP8, T, TT>;
     constexpr int LDS_BYTES = lds_bytes(NC);
     static bool attr_set = false;
     if (!attr_set) {
@@ -883,14 +911,14 @@ static int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt,
     return hipGetLastError() == hipSuccess ? LAZYATTN_OK : LAZYATTN_E_LAUNCH;
 }
 
-template <int NC>
+template <int NC, typename T>
 static int launch_mfma_nc(const lazyattn_prefill_params &p, int nsplit, int n_mt, hipStream_t stream) {
     const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3;
     const bool t32 = p.table_dtype == LAZYATTN_F32;
-    if (fp8) return t32 ? launch_mfma_t<NC, true, float>(p, nsplit, n_mt, stream)
-                        : launch_mfma_t<NC, true, bf16_t>(p, nsplit, n_mt, stream);
-    return t32 ? launch_mfma_t<NC, false, float>(p, nsplit, n_mt, stream)
-               : launch_mfma_t<NC, false, bf16_t>(p, nsplit, n_mt, stream);
+    if (fp8) return t32 ? launch_mfma_t<NC, true, T, float>(p, nsplit, n_mt, stream)
+                        : launch_mfma_t<NC, true, T, T>(p, nsplit, n_mt, stream);
+    return t32 ? launch_mfma_t<NC, false, T, float>(p, nsplit, n_mt, stream)
+               : launch_mfma_t<NC, false, T, T>(p, nsplit, n_mt, stream);
 }
 
 int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
@@ -904,15 +932,18 @@ int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
         if (((uintptr_t)p.workspace) & 15) return LAZYATTN_E_WORKSPACE;
     }
     if (phases & LAZYATTN_PHASE_MAIN) {
-        const int rc = nw == 8 ? launch_mfma_nc<8>(p, nsplit, n_mt, stream) : launch_mfma_nc<4>(p, nsplit, n_mt, stream);
+        const bool f16 = p.dtype == LAZYATTN_F16;
+        const int rc = nw == 8 ? (f16 ? launch_mfma_nc<8, f16_t>(p, nsplit, n_mt, stream) : launch_mfma_nc<8, bf16_t>(p, nsplit, n_mt, stream))
+                               : (f16 ? launch_mfma_nc<4, f16_t>(p, nsplit, n_mt, stream) : launch_mfma_nc<4, bf16_t>(p, nsplit, n_mt, stream));
         if (rc != LAZYATTN_OK) return rc;
     }
     if (nsplit > 1 && (phases & LAZYATTN_PHASE_COMBINE)) {
         const int64_t rows = (int64_t)p.max_q_len * p.num_q_heads;
         const MergeArgs m{p.workspace, p.b_start_loc, p.o, {p.o_stride[0], p.o_stride[1]}, p.num_tokens, p.num_q_heads,
                           p.index_bits, p.skip_decode};
-        hipLaunchKernelGGL(prefill_combine_kernel, dim3((unsigned)((rows + 7) / 8), p.batch), dim3(256), 0, stream, m,
-                           nsplit);
+        const dim3 grid((unsigned)((rows + 7) / 8), p.batch);
+        if (p.dtype == LAZYATTN_F16) hipLaunchKernelGGL(prefill_combine_kernel<f16_t>, grid, dim3(256), 0, stream, m, nsplit);
+        else hipLaunchKernelGGL(prefill_combine_kernel<bf16_t>, grid, dim3(256), 0, stream, m, nsplit);
         if (hipGetLastError() != hipSuccess) return LAZYATTN_E_LAUNCH;
     }
     return LAZYATTN_OK;

@@ -67,6 +67,23 @@ def test_mfma_vanilla_requests():
     assert e < 2e-2, e
 
 
+@pytest.mark.parametrize("variant", ["natural", "offset", "block_uniform"])
+@pytest.mark.parametrize("kv", ["auto", "fp8"])
+def test_mfma_float16_operands(variant, kv):
+    """float16 is the element type the reference's own kernel test runs (tests/kernels/test_prefix_prefill.py:45);
+    the matrix path takes it with v_mfma_f32_32x32x16_f16.  fp16 carries 11 bits: tolerance 5e-3 (fp8 cache: 5e-2)."""
+    print(f"case: mfma float16 {variant} kv={kv}", flush=True)
+    w = wl.make_workload("ragged16", dtype=torch.float16, **GEOM,
+                         doc_lens=[100, 16, 333, 70, 5, 250], requests=[[3, 1, 0], [2], [0, 2, 3, 1, 5], [4], []],
+                         q_lens=[70, 1, 9, 33, 130], variant=variant, kv_cache_dtype=kv, seed=77)
+    ref = run_oracle(w)
+    for nsplit in (1, 3):
+        got = run_op(w.to(DEV), kernel=_ffi.KERNEL_MFMA, num_splits=nsplit).cpu()
+        assert got.dtype == torch.float16
+        e = _err(got, ref)
+        assert e < (5e-2 if kv == "fp8" else 5e-3), (nsplit, e)
+
+
 @pytest.mark.parametrize("scale", [1e-6, 3e4])
 def test_mfma_split_partials_keep_their_precision_at_any_magnitude(scale):
     """Split-KV partial rows are stored as halves with one power-of-two scale per row: values far outside
