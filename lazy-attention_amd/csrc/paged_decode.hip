@@ -23,49 +23,38 @@
 // converted, scaled and rounded to bf16 (old_ops/prefix_prefill.py:239-241 arithmetic), then treated alike.
 // Slices of one request are merged by paged_decode_merge_kernel.
 #include "common.hpp"
+#include "elem16.hpp"
 
 namespace lazyattn {
 
 namespace {
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
-typedef __attribute__((ext_vector_type(4))) float f32x4_t;
-typedef __attribute__((ext_vector_type(2))) float f32x2_t;
 
 constexpr int D = 128;
 constexpr int HALF = 64;
 constexpr int BS = 16;
 constexpr int WAVES = 4;            // independent waves per workgroup
 
-__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
-__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
-__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
-    f32x2_t f = {a, b};
-    bf16x2_t h = __builtin_convertvector(f, bf16x2_t);   // v_cvt_pk_bf16_f32, RNE
-    return *reinterpret_cast<uint32_t *>(&h);
-}
 __device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
-__device__ __forceinline__ void unpack8(const uint4 &w, float *f) {
-    f[0] = bf16_lo(w.x); f[1] = bf16_hi(w.x); f[2] = bf16_lo(w.y); f[3] = bf16_hi(w.y);
-    f[4] = bf16_lo(w.z); f[5] = bf16_hi(w.z); f[6] = bf16_lo(w.w); f[7] = bf16_hi(w.w);
+template <typename T> __device__ __forceinline__ void unpack8(const uint4 &w, float *f) {
+    f[0] = Elem<T>::lo(w.x); f[1] = Elem<T>::hi(w.x); f[2] = Elem<T>::lo(w.y); f[3] = Elem<T>::hi(w.y);
+    f[4] = Elem<T>::lo(w.z); f[5] = Elem<T>::hi(w.z); f[6] = Elem<T>::lo(w.w); f[7] = Elem<T>::hi(w.w);
 }
 
-// 8 fp8 e4m3 bytes -> (float * scale) rounded to bf16, as floats
-__device__ __forceinline__ void unpack8_fp8(uint32_t lo, uint32_t hi, float scale, float *f) {
+// 8 fp8 e4m3 bytes -> (float * scale) rounded to the query type, as floats
+template <typename T> __device__ __forceinline__ void unpack8_fp8(uint32_t lo, uint32_t hi, float scale, float *f) {
     const f32x2_t a = __builtin_amdgcn_cvt_pk_f32_fp8(lo, false), b = __builtin_amdgcn_cvt_pk_f32_fp8(lo >> 16, false);
     const f32x2_t c = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false), d = __builtin_amdgcn_cvt_pk_f32_fp8(hi >> 16, false);
     const float t[8] = {a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
 #pragma unroll
-    for (int i = 0; i < 8; ++i) f[i] = round_to<bf16_t>(t[i] * scale);
+    for (int i = 0; i < 8; ++i) f[i] = round_to<T>(t[i] * scale);
 }
 
 // 8 consecutive cos (or sin) entries of one table row
-template <typename TT> struct Tab8;
-template <> struct Tab8<bf16_t> {
+template <typename TT> struct Tab8 {                        // a 16-bit table
     uint4 v;
     __device__ __forceinline__ void load(const uint8_t *row, int elem) { v = *reinterpret_cast<const uint4 *>(row + elem * 2); }
-    __device__ __forceinline__ void get(float *f) const { unpack8(v, f); }
+    __device__ __forceinline__ void get(float *f) const { unpack8<TT>(v, f); }
 };
 template <> struct Tab8<float> {
     float4 a, b;
@@ -90,9 +79,10 @@ struct ValRegs {
 
 }  // namespace
 
-template <typename TT, bool FP8>
+template <typename T, typename TT, bool FP8>
 __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2)))
 paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
+    using E = Elem<T>;
     constexpr int TSZ = sizeof(TT);
     const int lane = threadIdx.x & 63;
     const int wave = uniform(threadIdx.x >> 6);
@@ -194,14 +184,14 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
         }
     };
     // rotate the pair (lo, hi) = (d, d + 64) in fp32, one rounding to bf16
-    auto rotate = [&](const uint4 &lo, const uint4 &hi, const Tab8<TT> &c, const Tab8<TT> &s, bf16x8_t &xo, bf16x8_t &yo) {
+    auto rotate = [&](const uint4 &lo, const uint4 &hi, const Tab8<TT> &c, const Tab8<TT> &s, uint4 &xo, uint4 &yo) {
         float a[8], bb[8], cs[8], sn[8], x[8], y[8];
         if (FP8) {
-            unpack8_fp8(lo.x, lo.y, k_scale, a);
-            unpack8_fp8(hi.x, hi.y, k_scale, bb);
+            unpack8_fp8<T>(lo.x, lo.y, k_scale, a);
+            unpack8_fp8<T>(hi.x, hi.y, k_scale, bb);
         } else {
-            unpack8(lo, a);
-            unpack8(hi, bb);
+            unpack8<T>(lo, a);
+            unpack8<T>(hi, bb);
         }
         c.get(cs);
         s.get(sn);
@@ -210,22 +200,20 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
             x[e] = a[e] * cs[e] - bb[e] * sn[e];
             y[e] = a[e] * sn[e] + bb[e] * cs[e];
         }
-        uint4 xw = make_uint4(pack_bf16(x[0], x[1]), pack_bf16(x[2], x[3]), pack_bf16(x[4], x[5]), pack_bf16(x[6], x[7]));
-        uint4 yw = make_uint4(pack_bf16(y[0], y[1]), pack_bf16(y[2], y[3]), pack_bf16(y[4], y[5]), pack_bf16(y[6], y[7]));
-        xo = *reinterpret_cast<bf16x8_t *>(&xw);
-        yo = *reinterpret_cast<bf16x8_t *>(&yw);
+        xo = make_uint4(E::pack(x[0], x[1]), E::pack(x[2], x[3]), E::pack(x[4], x[5]), E::pack(x[6], x[7]));
+        yo = make_uint4(E::pack(y[0], y[1]), E::pack(y[2], y[3]), E::pack(y[4], y[5]), E::pack(y[6], y[7]));
     };
 
     // Q^T: column = head = t, contraction d = 32 m + 8 grp ..
-    bf16x8_t qf[4];
+    uint4 qf[4];
     {
         const bool head_ok = t < group;
-        const bf16_t *qp = (const bf16_t *)p.q + qs * p.q_stride[0] + (int64_t)(g * group + (head_ok ? t : 0)) * p.q_stride[1] + 8 * grp;
+        const T *qp = (const T *)p.q + qs * p.q_stride[0] + (int64_t)(g * group + (head_ok ? t : 0)) * p.q_stride[1] + 8 * grp;
 #pragma unroll
         for (int m = 0; m < 4; ++m) {
             uint4 w = make_uint4(0, 0, 0, 0);
             if (head_ok) w = *reinterpret_cast<const uint4 *>(qp + 32 * m);
-            qf[m] = *reinterpret_cast<bf16x8_t *>(&w);
+            qf[m] = w;
         }
     }
     const float cs2 = p.sm_scale * 1.4426950408889634f;
@@ -236,14 +224,14 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
 
     // scores of one page: S^T[token 4 grp + i][head t], masked
     auto scores = [&](const KeyRegs<TT> &r) -> f32x4_t {
-        bf16x8_t k0, k1, k2, k3;
+        uint4 k0, k1, k2, k3;
         rotate(r.k[0], r.k[2], r.c0, r.s0, k0, k2);
         rotate(r.k[1], r.k[3], r.c1, r.s1, k1, k3);
         f32x4_t s = {0.f, 0.f, 0.f, 0.f};
-        s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0, qf[0], s, 0, 0, 0);
-        s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1, qf[1], s, 0, 0, 0);
-        s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k2, qf[2], s, 0, 0, 0);
-        s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k3, qf[3], s, 0, 0, 0);
+        s = E::mfma16(k0, qf[0], s);
+        s = E::mfma16(k1, qf[1], s);
+        s = E::mfma16(k2, qf[2], s);
+        s = E::mfma16(k3, qf[3], s);
         if (r.lim < BS) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) s[i] = 4 * grp + i < r.lim ? s[i] : -INFINITY;
@@ -255,7 +243,7 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
         uint2 w = r.v[blk];
         if (FP8) {
             const f32x2_t lo = __builtin_amdgcn_cvt_pk_f32_fp8(w.x, false), hi = __builtin_amdgcn_cvt_pk_f32_fp8(w.x >> 16, false);
-            w = make_uint2(pack_bf16(lo[0] * v_scale, lo[1] * v_scale), pack_bf16(hi[0] * v_scale, hi[1] * v_scale));
+            w = make_uint2(E::pack(lo[0] * v_scale, lo[1] * v_scale), E::pack(hi[0] * v_scale, hi[1] * v_scale));
         }
         if (lim < BS) {
             if (4 * grp + 0 >= lim) w.x &= 0xffff0000u;
@@ -305,13 +293,11 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
             py[i] = __builtin_amdgcn_exp2f(fmaf(sy[i], cs2, -mc));
         }
         l_run += (px[0] + px[1]) + (px[2] + px[3]) + (py[0] + py[1]) + (py[2] + py[3]);
-        uint4 pw = make_uint4(pack_bf16(px[0], px[1]), pack_bf16(px[2], px[3]), pack_bf16(py[0], py[1]), pack_bf16(py[2], py[3]));
-        const bf16x8_t pf = *reinterpret_cast<bf16x8_t *>(&pw);
+        const uint4 pf = make_uint4(E::pack(px[0], px[1]), E::pack(px[2], px[3]), E::pack(py[0], py[1]), E::pack(py[2], py[3]));
 #pragma unroll
         for (int blk = 0; blk < 8; ++blk) {
             const uint2 vx = masked_v(X, lim_x, blk), vy = masked_v(Y, lim_y, blk);
-            uint4 vw = make_uint4(vx.x, vx.y, vy.x, vy.y);
-            acc[blk] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<bf16x8_t *>(&vw), pf, acc[blk], 0, 0, 0);
+            acc[blk] = E::mfma16(make_uint4(vx.x, vx.y, vy.x, vy.y), pf, acc[blk]);
         }
     }
 
@@ -322,11 +308,11 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     const int h = g * group + t;
     const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
     if (nsplit == 1) {
-        bf16_t *op = (bf16_t *)p.o + qs * p.o_stride[0] + (int64_t)h * p.o_stride[1] + 4 * grp;
+        T *op = (T *)p.o + qs * p.o_stride[0] + (int64_t)h * p.o_stride[1] + 4 * grp;
 #pragma unroll
         for (int blk = 0; blk < 8; ++blk)
             *reinterpret_cast<uint2 *>(op + 16 * blk) =
-                make_uint2(pack_bf16(acc[blk][0] * inv, acc[blk][1] * inv), pack_bf16(acc[blk][2] * inv, acc[blk][3] * inv));
+                make_uint2(E::pack(acc[blk][0] * inv, acc[blk][1] * inv), E::pack(acc[blk][2] * inv, acc[blk][3] * inv));
         return;
     }
     // partial of this slice: normalised O and log2-sum-exp, indexed by (slice, request, head)
@@ -349,8 +335,10 @@ struct DecodeMergeArgs {
     int64_t o_stride[2];
     int32_t batch, num_q_heads, index_bits;
 };
+template <typename T>
 __global__ void __launch_bounds__(256)
 paged_decode_merge_kernel(const DecodeMergeArgs p, const int nsplit) {
+    using E = Elem<T>;
     const int64_t r = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);
     if (r >= (int64_t)p.batch * p.num_q_heads) return;
     const int b = (int)(r / p.num_q_heads), h = (int)(r % p.num_q_heads);
@@ -390,15 +378,15 @@ paged_decode_merge_kernel(const DecodeMergeArgs p, const int nsplit) {
         }
     }
     const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
-    bf16_t *op = (bf16_t *)p.o + qs * p.o_stride[0] + (int64_t)h * p.o_stride[1] + d;
-    *reinterpret_cast<uint2 *>(op) = make_uint2(pack_bf16(o.x * inv, o.y * inv), pack_bf16(o.z * inv, o.w * inv));
+    T *op = (T *)p.o + qs * p.o_stride[0] + (int64_t)h * p.o_stride[1] + d;
+    *reinterpret_cast<uint2 *>(op) = make_uint2(E::pack(o.x * inv, o.y * inv), E::pack(o.z * inv, o.w * inv));
 }
 
 // ------------------------------------------------------------------ host side
 bool decode_mfma_supports(const lazyattn_prefill_params &p) {
     const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3;
-    if (p.dtype != LAZYATTN_BF16 || !(p.cache_dtype == LAZYATTN_BF16 || fp8)) return false;
-    if (p.table_dtype != LAZYATTN_BF16 && p.table_dtype != LAZYATTN_F32) return false;
+    if ((p.dtype != LAZYATTN_BF16 && p.dtype != LAZYATTN_F16) || !(p.cache_dtype == p.dtype || fp8)) return false;
+    if (p.table_dtype != p.dtype && p.table_dtype != LAZYATTN_F32) return false;
     if (p.head_dim != D || p.block_size != BS || p.x != (fp8 ? 16 : 8)) return false;
     if (p.sliding_window > 0) return false;
     if (p.pos_mode != LAZYATTN_POS_NATURAL && p.pos_mode != LAZYATTN_POS_BLOCK_UNIFORM) return false;
@@ -449,16 +437,22 @@ int launch_decode_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
     if (phases & LAZYATTN_PHASE_MAIN) {
         const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3, t32 = p.table_dtype == LAZYATTN_F32;
         const dim3 grid(nblocks), block(WAVES * 64);
-        if (fp8 && t32) hipLaunchKernelGGL((paged_decode_kernel<float, true>), grid, block, 0, stream, p, nsplit);
-        else if (fp8) hipLaunchKernelGGL((paged_decode_kernel<bf16_t, true>), grid, block, 0, stream, p, nsplit);
-        else if (t32) hipLaunchKernelGGL((paged_decode_kernel<float, false>), grid, block, 0, stream, p, nsplit);
-        else hipLaunchKernelGGL((paged_decode_kernel<bf16_t, false>), grid, block, 0, stream, p, nsplit);
+        auto launch = [&](auto elem) {
+            using T = decltype(elem);
+            if (fp8 && t32) hipLaunchKernelGGL((paged_decode_kernel<T, float, true>), grid, block, 0, stream, p, nsplit);
+            else if (fp8) hipLaunchKernelGGL((paged_decode_kernel<T, T, true>), grid, block, 0, stream, p, nsplit);
+            else if (t32) hipLaunchKernelGGL((paged_decode_kernel<T, float, false>), grid, block, 0, stream, p, nsplit);
+            else hipLaunchKernelGGL((paged_decode_kernel<T, T, false>), grid, block, 0, stream, p, nsplit);
+        };
+        if (p.dtype == LAZYATTN_F16) launch(f16_t{}); else launch(bf16_t{});
         if (hipGetLastError() != hipSuccess) return LAZYATTN_E_LAUNCH;
     }
     if (nsplit > 1 && (phases & LAZYATTN_PHASE_COMBINE)) {
         const int64_t rows = (int64_t)p.batch * p.num_q_heads;
         const DecodeMergeArgs m{p.workspace, p.b_start_loc, p.o, {p.o_stride[0], p.o_stride[1]}, p.batch, p.num_q_heads, p.index_bits};
-        hipLaunchKernelGGL(paged_decode_merge_kernel, dim3((unsigned)((rows + 7) / 8)), dim3(256), 0, stream, m, nsplit);
+        const dim3 mgrid((unsigned)((rows + 7) / 8));
+        if (p.dtype == LAZYATTN_F16) hipLaunchKernelGGL(paged_decode_merge_kernel<f16_t>, mgrid, dim3(256), 0, stream, m, nsplit);
+        else hipLaunchKernelGGL(paged_decode_merge_kernel<bf16_t>, mgrid, dim3(256), 0, stream, m, nsplit);
         if (hipGetLastError() != hipSuccess) return LAZYATTN_E_LAUNCH;
     }
     return LAZYATTN_OK;

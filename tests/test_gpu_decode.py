@@ -16,11 +16,12 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda"
 
 
-def _decode_batch(variant, *, hq=8, hkv=2, q_lens=(1, 1, 1, 1, 1), table_f32=False, seed=77, kv="auto"):
+def _decode_batch(variant, *, hq=8, hkv=2, q_lens=(1, 1, 1, 1, 1), table_f32=False, seed=77, kv="auto",
+                  dtype=torch.bfloat16):
     """Ragged documents (pads at document ends), requests of 1 to 9 documents, one new token each
     (or more: such requests must be skipped)."""
     d = 128
-    w = wl.make_workload("decode", dtype=torch.bfloat16, hq=hq, hkv=hkv, d=d, theta=500000.0, block_size=16,
+    w = wl.make_workload("decode", dtype=dtype, hq=hq, hkv=hkv, d=d, theta=500000.0, block_size=16,
                          doc_lens=[40, 16, 33, 70, 5, 128, 97],
                          requests=[[3, 1, 0], [2], [0, 2, 3, 1, 5, 6, 4, 5, 6], [4, 0], [6, 5, 3]],
                          q_lens=list(q_lens), variant=variant, seed=seed, kv_cache_dtype=kv)
@@ -127,6 +128,20 @@ def test_decode_fp8_cache(variant, table_f32):
     assert _err(got, ref) < 5e-2, _err(got, ref)
     same = _run(w, kernel=_ffi.KERNEL_GENERIC)
     assert _err(got, same) < 2e-2, _err(got, same)
+
+
+@pytest.mark.parametrize("variant", ["natural", "block_uniform"])
+@pytest.mark.parametrize("kv", ["auto", "fp8"])
+def test_decode_float16_operands(variant, kv):
+    print(f"case: decode float16 {variant} kv={kv}", flush=True)
+    w = _decode_batch(variant, kv=kv, dtype=torch.float16)
+    ref = _oracle(w)
+    for nsplit in (1, 3):
+        got = _run(w, num_splits=nsplit)
+        assert got.dtype == torch.float16
+        assert _err(got, ref) < (5e-2 if kv == "fp8" else 5e-3), (nsplit, _err(got, ref))
+    same = _run(w, kernel=_ffi.KERNEL_GENERIC)
+    assert _err(got, same) < (2e-2 if kv == "fp8" else 5e-3), _err(got, same)
 
 
 def test_decode_pad_slots_may_hold_nan():
