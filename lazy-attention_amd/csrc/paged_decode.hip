@@ -72,6 +72,7 @@ template <typename TT> struct KeyRegs {
     uint4 k[4];                 // chunks grp, 4 + grp, 8 + grp, 12 + grp of token t
     Tab8<TT> c0, s0, c1, s1;    // cos / sin for d = 8 grp .. (pair k[0], k[2]) and d = 32 + 8 grp .. (pair k[1], k[3])
     int lim;                    // valid slots
+    int first;                  // first slot inside the sliding window (<= 0: all)
 };
 struct ValRegs {
     uint2 v[8];                 // V[d = 16 blk + t][tokens 4 grp .. 4 grp + 3]
@@ -106,8 +107,12 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     const bool use_qo = !vanilla && p.pos_mode == LAZYATTN_POS_BLOCK_UNIFORM;
     const int n_pages = seq_len > 0 ? (seq_len + BS - 1) / BS : 0;
     const int n_pairs = (n_pages + 1) / 2;
-    const int pair_begin = (int)((int64_t)n_pairs * split / nsplit);
-    const int pair_end = (int)((int64_t)n_pairs * (split + 1) / nsplit);
+    // sliding window (old_ops/chunked_prefill_paged_decode.py:237-241): the row sits at position seq_len - 1 and
+    // sees the keys at seq_len - window .. seq_len - 1; the page pairs before that are not visited
+    const int first_key = p.sliding_window > 0 && seq_len > p.sliding_window ? seq_len - p.sliding_window : 0;
+    const int first_pair = first_key / (2 * BS);
+    const int pair_begin = first_pair + (int)((int64_t)(n_pairs - first_pair) * split / nsplit);
+    const int pair_end = first_pair + (int)((int64_t)(n_pairs - first_pair) * (split + 1) / nsplit);
 
     const int t = lane & 15, grp = lane >> 4;
 
@@ -151,6 +156,7 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
         l = l < BS - qm ? l : BS - qm;
         l = l > BS ? BS : l;
         r.lim = l < 0 ? 0 : l;
+        r.first = first_key - j * BS;                                                // slots below it lie before the window
         const uint8_t *kb = kc_base + bt * kc_page_bytes;
 #pragma unroll
         for (int m = 0; m < 4; ++m) {
@@ -232,9 +238,9 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
         s = E::mfma16(k1, qf[1], s);
         s = E::mfma16(k2, qf[2], s);
         s = E::mfma16(k3, qf[3], s);
-        if (r.lim < BS) {
+        if (r.lim < BS || r.first > 0) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) s[i] = 4 * grp + i < r.lim ? s[i] : -INFINITY;
+            for (int i = 0; i < 4; ++i) s[i] = (4 * grp + i < r.lim && 4 * grp + i >= r.first) ? s[i] : -INFINITY;
         }
         return s;
     };
@@ -388,7 +394,6 @@ bool decode_mfma_supports(const lazyattn_prefill_params &p) {
     if ((p.dtype != LAZYATTN_BF16 && p.dtype != LAZYATTN_F16) || !(p.cache_dtype == p.dtype || fp8)) return false;
     if (p.table_dtype != p.dtype && p.table_dtype != LAZYATTN_F32) return false;
     if (p.head_dim != D || p.block_size != BS || p.x != (fp8 ? 16 : 8)) return false;
-    if (p.sliding_window > 0) return false;
     if (p.pos_mode != LAZYATTN_POS_NATURAL && p.pos_mode != LAZYATTN_POS_BLOCK_UNIFORM) return false;
     if (p.num_q_heads / p.num_kv_heads > 16) return false;
     if (p.q_stride[2] != 1 || p.o_stride[2] != 1) return false;

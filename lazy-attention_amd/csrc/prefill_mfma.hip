@@ -129,7 +129,8 @@ constexpr int lds_bytes(int nc) { return KV_BYTES + nc * 8 * 1024 + 2 * PAGES * 
 constexpr int KI = 2;                    // K items per gathering lane and tile: a page has 128 (8 chunks x 16 slots)
 constexpr int VI = 4;                    // V items per gathering lane and tile: a page has 256 of 16 bytes
 
-template <int NC, bool FP8, typename T, typename TT>
+// WIN: built with the sliding-window code (calls without a window run the instantiation without it)
+template <int NC, bool FP8, bool WIN, typename T, typename TT>
 __global__ void __launch_bounds__((NC + 4) * 64)
 prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int n_mt) {
     constexpr int VI_CTX = FP8 ? VI / 2 : VI;        // an fp8 page row of 16 slots is one 16-byte item
@@ -192,9 +193,24 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     // three context tiles (element-wise V scatter, per-row causal masks, branchy loads), and all of them
     // sit at the end: with equal tile counts the last split was the tail of every launch.
     constexpr int NEW_COST = 3;
-    const int64_t cost = n_ctx_tiles + (int64_t)NEW_COST * n_new_tiles;
+    // Sliding window (old_ops:270-284, 373-376): the row at sequence position P sees the keys at positions
+    // P - window + 1 .. P only.  Positions: context slot n -> n, new token m -> ctx_len + m.  The tiles that
+    // lie entirely before the window of the workgroup's first row are not visited at all.
+    const int window = WIN ? p.sliding_window : 0;
+    int skip_ctx = 0, skip_new = 0;                 // whole context / new-token tiles before every window
+    if (window) {
+        const int first_row = ((mt * NC) / group) * UNIT;
+        const int lo_min = ctx_len + first_row - window + 1;
+        if (lo_min > 0) {
+            skip_ctx = lo_min < ctx_len ? lo_min / NT : n_ctx_tiles;
+            if (lo_min >= ctx_len) skip_new = (lo_min - ctx_len) / NT;
+            if (skip_new > n_new_tiles) skip_new = n_new_tiles;
+        }
+    }
+    const int live_ctx = n_ctx_tiles - skip_ctx, live_new = n_new_tiles - skip_new;
+    const int64_t cost = live_ctx + (int64_t)NEW_COST * live_new;
     auto tile_at = [&](int64_t c) -> int {         // first tile whose cost interval ends after c
-        return c <= n_ctx_tiles ? (int)c : n_ctx_tiles + (int)((c - n_ctx_tiles) / NEW_COST);
+        return skip_ctx + skip_new + (c <= live_ctx ? (int)c : live_ctx + (int)((c - live_ctx) / NEW_COST));
     };
     const int tile_begin = tile_at(cost * split / nsplit);
     const int tile_end = split + 1 == nsplit ? n_ctx_tiles + n_new_tiles : tile_at(cost * (split + 1) / nsplit);
@@ -552,14 +568,17 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         __builtin_amdgcn_s_setprio(0);
     };
     // ---- masks: register i of half `sub` holds key sub*32 + 8*(i/4) + 4*gh + i%4 ----
-    auto mask_half = [&](f32x16_t &s, uint32_t vbits, int sub, int kind, int m0) {
+    // key0 = sequence position of the tile's first key (only used under a sliding window)
+    auto mask_half = [&](f32x16_t &s, uint32_t vbits, int sub, int kind, int m0, int key0) {
         const uint32_t w = vbits >> (4 * gh);
         // causal: key m0 + kk <= row  <=>  8*(i/4) + i%4 <= row - m0 - sub*32 - 4*gh   (old_ops:371-372)
         const int lim = kind == TILE_NEW ? row - m0 - sub * 32 - 4 * gh : 64;
+        // window: key0 + sub*32 + 4*gh + kb >= ctx_len + row - window + 1
+        const int lb = window ? ctx_len + row - window + 1 - key0 - sub * 32 - 4 * gh : -64;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const int kb = 8 * (i >> 2) + (i & 3);
-            const bool ok = ((w >> kb) & 1u) && kb <= lim;
+            const bool ok = ((w >> kb) & 1u) && kb <= lim && (!WIN || kb >= lb);
             s[i] = ok ? s[i] : -INFINITY;
         }
     };
@@ -631,12 +650,13 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
 
     // which of the tile's 64 keys exist: new-token tiles from the token count, context tiles from the
     // page limits the gathering waves left beside the tile
-    struct Desc { int kind; uint32_t vlo, vhi; int m0; };
+    struct Desc { int kind; uint32_t vlo, vhi; int m0, key0; };
     auto describe = [&](int tile, int cur) -> Desc {
-        Desc td{TILE_FULL, ~0u, ~0u, 0};
+        Desc td{TILE_FULL, ~0u, ~0u, 0, tile * NT};
         if (tile >= n_ctx_tiles) {
             td.kind = TILE_NEW;
             td.m0 = (tile - n_ctx_tiles) * NT;
+            td.key0 = ctx_len + td.m0;
             const int n = t_end - td.m0;
             const uint64_t valid = n >= 64 ? ~0ull : (n <= 0 ? 0ull : ((1ull << n) - 1ull));
             td.vlo = (uint32_t)valid; td.vhi = (uint32_t)(valid >> 32);
@@ -649,6 +669,8 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                 td.vhi = ((1u << l2) - 1u) | (((1u << l3) - 1u) << BS);
             }
         }
+        // a tile that starts before the window of this wave's last row needs the per-row lower bound
+        if (window && td.kind == TILE_FULL && td.key0 < ctx_len + t0 + UNIT - window) td.kind = TILE_EDGE;
         return td;
     };
     __syncthreads();
@@ -664,8 +686,8 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             f32x16_t s0, s1;
             qk_tile(ktile, s0, s1);
             if (td.kind != TILE_FULL) {
-                mask_half(s0, td.vlo, 0, td.kind, td.m0);
-                mask_half(s1, td.vhi, 1, td.kind, td.m0);
+                mask_half(s0, td.vlo, 0, td.kind, td.m0, td.key0);
+                mask_half(s1, td.vhi, 1, td.kind, td.m0, td.key0);
             }
             attend(vtile, s0, s1);
         }
@@ -824,7 +846,6 @@ bool mfma_supports(const lazyattn_prefill_params &p) {
     if (!(p.cache_dtype == p.dtype || fp8)) return false;
     if (p.table_dtype != p.dtype && p.table_dtype != LAZYATTN_F32) return false;
     if (p.head_dim != D || p.block_size != BS || p.x != (fp8 ? 16 : 8)) return false;
-    if (p.sliding_window > 0) return false;
     if (p.q_stride[2] != 1 || p.k_stride[2] != 1 || p.v_stride[2] != 1 || p.o_stride[2] != 1) return false;
     if (p.kc_stride[4] != 1 || p.kc_stride[3] != p.x || p.kc_stride[2] != (int64_t)BS * p.x) return false;
     if (p.vc_stride[3] != 1 || p.vc_stride[2] != BS) return false;
@@ -847,9 +868,9 @@ size_t mfma_workspace_bytes(const lazyattn_prefill_params &p) {
     return (size_t)ns * (size_t)p.num_tokens * p.num_q_heads * PARTIAL_ROW_BYTES;
 }
 
-template <int NC, bool FP8, typename T, typename TT>
+template <int NC, bool FP8, bool WIN, typename T, typename TT>
 static int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt, hipStream_t stream) {
-    auto kern = prefill_mfma_kernel<NC, FP8, T, TT>;
+    auto kern = prefill_mfma_kernel<NC, FP8, WIN, T, TT>;
     constexpr int LDS_BYTES = lds_bytes(NC);
     static bool attr_set = false;
     if (!attr_set) {
@@ -866,10 +887,16 @@ template <int NC, typename T>
 static int launch_mfma_nc(const lazyattn_prefill_params &p, int nsplit, int n_mt, hipStream_t stream) {
     const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3;
     const bool t32 = p.table_dtype == LAZYATTN_F32;
-    if (fp8) return t32 ? launch_mfma_t<NC, true, T, float>(p, nsplit, n_mt, stream)
-                        : launch_mfma_t<NC, true, T, T>(p, nsplit, n_mt, stream);
-    return t32 ? launch_mfma_t<NC, false, T, float>(p, nsplit, n_mt, stream)
-               : launch_mfma_t<NC, false, T, T>(p, nsplit, n_mt, stream);
+    if (p.sliding_window > 0) {
+        if (fp8) return t32 ? launch_mfma_t<NC, true, true, T, float>(p, nsplit, n_mt, stream)
+                            : launch_mfma_t<NC, true, true, T, T>(p, nsplit, n_mt, stream);
+        return t32 ? launch_mfma_t<NC, false, true, T, float>(p, nsplit, n_mt, stream)
+                   : launch_mfma_t<NC, false, true, T, T>(p, nsplit, n_mt, stream);
+    }
+    if (fp8) return t32 ? launch_mfma_t<NC, true, false, T, float>(p, nsplit, n_mt, stream)
+                        : launch_mfma_t<NC, true, false, T, T>(p, nsplit, n_mt, stream);
+    return t32 ? launch_mfma_t<NC, false, false, T, float>(p, nsplit, n_mt, stream)
+               : launch_mfma_t<NC, false, false, T, T>(p, nsplit, n_mt, stream);
 }
 
 int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {

@@ -43,16 +43,16 @@ def _decode_batch(variant, *, hq=8, hkv=2, q_lens=(1, 1, 1, 1, 1), table_f32=Fal
     return w
 
 
-def _oracle(w, lazy=None):
+def _oracle(w, lazy=None, sliding_window=0):
     ref = torch.full_like(w.q, 5.0)
     orc.paged_decode(w.q, w.k_cache, w.v_cache, w.block_table, w.b_start_loc, w.b_seq_len,
                      w.cos_sin_cache, w.q_mask, q_offset=w.q_offset, is_lazy=lazy,
-                     kv_cache_dtype=w.kv_cache_dtype, k_scale=w.k_scale, v_scale=w.v_scale,
+                     kv_cache_dtype=w.kv_cache_dtype, k_scale=w.k_scale, v_scale=w.v_scale, sliding_window=sliding_window,
                      pos_mode=orc.POS_NATURAL if w.pos_mode != orc.POS_BLOCK_UNIFORM else w.pos_mode, out=ref)
     return ref
 
 
-def _run(w, *, lazy=None, num_splits=0, kernel=_ffi.KERNEL_AUTO):
+def _run(w, *, lazy=None, num_splits=0, kernel=_ffi.KERNEL_AUTO, sliding_window=0):
     """The q_len==1 launch the entry points make, with the slicing and kernel choice exposed."""
     g = w.to(DEV)
     out = torch.full_like(g.q, 5.0)
@@ -60,7 +60,7 @@ def _run(w, *, lazy=None, num_splits=0, kernel=_ffi.KERNEL_AUTO):
     _launch.launch_prefill(
         q=g.q, k=g.k, v=g.v, o=out, kv_cache_dtype=w.kv_cache_dtype, k_cache=g.k_cache, v_cache=g.v_cache,
         b_loc=g.block_table, b_start_loc=g.b_start_loc, b_seq_len=g.b_seq_len, max_input_len=1,
-        max_seq_len=g.max_seq_len, k_scale=g.k_scale, v_scale=g.v_scale, alibi_slopes=None, sliding_window=0,
+        max_seq_len=g.max_seq_len, k_scale=g.k_scale, v_scale=g.v_scale, alibi_slopes=None, sliding_window=sliding_window,
         sm_scale=128 ** -0.5, skip_decode=False, cos_sin_cache=g.cos_sin_cache, rotary_dim=128,
         is_neox_style=True, is_lazy=None if lazy is None else lazy.to(DEV),
         q_offset=g.q_offset if bu else None, q_mask=g.q_mask,
@@ -142,6 +142,19 @@ def test_decode_float16_operands(variant, kv):
         assert _err(got, ref) < (5e-2 if kv == "fp8" else 5e-3), (nsplit, _err(got, ref))
     same = _run(w, kernel=_ffi.KERNEL_GENERIC)
     assert _err(got, same) < (2e-2 if kv == "fp8" else 5e-3), _err(got, same)
+
+
+@pytest.mark.parametrize("variant", ["natural", "block_uniform"])
+@pytest.mark.parametrize("window", [3, 20, 100, 4096])
+def test_decode_sliding_window(variant, window):
+    print(f"case: decode sliding window {window} {variant}", flush=True)
+    w = _decode_batch(variant)
+    ref = _oracle(w, sliding_window=window)
+    for nsplit in (1, 3):
+        got = _run(w, num_splits=nsplit, sliding_window=window)
+        assert _err(got, ref) < 2e-2, (nsplit, _err(got, ref))
+    same = _run(w, kernel=_ffi.KERNEL_GENERIC, sliding_window=window)
+    assert _err(got, same) < 2e-2, _err(got, same)
 
 
 def test_decode_pad_slots_may_hold_nan():

@@ -84,6 +84,20 @@ def test_mfma_float16_operands(variant, kv):
         assert e < (5e-2 if kv == "fp8" else 5e-3), (nsplit, e)
 
 
+@pytest.mark.parametrize("variant", ["natural", "block_uniform"])
+@pytest.mark.parametrize("window", [5, 37, 200, 4096])
+def test_mfma_sliding_window(variant, window):
+    """Sliding windows shorter than a page, than a tile, of several tiles, and longer than every context
+    (old_ops/prefix_prefill.py:270-284, 373-376); the tiles before a workgroup's first window are skipped."""
+    print(f"case: mfma sliding window {window} {variant}", flush=True)
+    w = _ragged(variant)
+    ref = run_oracle(w, sliding_window=window)
+    for nsplit, kernel in ((1, _ffi.KERNEL_MFMA4), (3, _ffi.KERNEL_MFMA8)):
+        got = run_op(w.to(DEV), kernel=kernel, num_splits=nsplit, sliding_window=window).cpu()
+        e = _err(got, ref)
+        assert e < 2e-2, (nsplit, e)
+
+
 @pytest.mark.parametrize("scale", [1e-6, 3e4])
 def test_mfma_split_partials_keep_their_precision_at_any_magnitude(scale):
     """Split-KV partial rows are stored as halves with one power-of-two scale per row: values far outside
