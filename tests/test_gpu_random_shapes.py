@@ -32,7 +32,8 @@ def _draw(seed):
     nsplit = r.choice([0, 1, 2, 3, 5])
     kernel = r.choice([_ffi.KERNEL_MFMA4, _ffi.KERNEL_MFMA8, _ffi.KERNEL_AUTO])
     dtype = r.choice([torch.bfloat16, torch.bfloat16, torch.float16])
-    return dict(dtype=dtype, hq=hkv * group, hkv=hkv, doc_lens=doc_lens, requests=requests, q_lens=q_lens, variant=variant,
+    window = r.choice([0, 0, 7, 50, 300])
+    return dict(dtype=dtype, window=window, hq=hkv * group, hkv=hkv, doc_lens=doc_lens, requests=requests, q_lens=q_lens, variant=variant,
                 kv=kv, nsplit=nsplit, kernel=kernel)
 
 
@@ -46,8 +47,8 @@ def test_random_ragged_batch(seed):
     lazy = None
     if c["variant"] == "block_uniform":
         lazy = torch.tensor([(seed + b) % 3 != 0 for b in range(len(c["q_lens"]))])
-    ref = run_oracle(w, **({"is_lazy": lazy} if lazy is not None else {}))
-    got = run_op(w.to(DEV), kernel=c["kernel"], num_splits=c["nsplit"],
+    ref = run_oracle(w, sliding_window=c["window"], **({"is_lazy": lazy} if lazy is not None else {}))
+    got = run_op(w.to(DEV), kernel=c["kernel"], num_splits=c["nsplit"], sliding_window=c["window"] or None,
                  is_lazy=None if lazy is None else lazy.to(DEV)).cpu()
     assert torch.isfinite(got.float()).all()
     err = (got.float() - ref.float()).abs().max().item()
