@@ -98,6 +98,30 @@ def test_mfma_sliding_window(variant, window):
         assert e < 2e-2, (nsplit, e)
 
 
+def test_mfma_takes_views_of_a_packed_qkv_tensor():
+    """vLLM hands q, k, v as views of one [T, (Hq + 2 Hkv) D] projection output and writes o into a wider buffer:
+    token strides larger than the row, the matrix path must take them as they are."""
+    print("case: mfma packed qkv views", flush=True)
+    w = _ragged("natural")
+    ref = run_oracle(w)
+    g = w.to(DEV)
+    T, hq, d = g.q.shape
+    hkv = g.k.shape[1]
+    qkv = torch.empty(T, (hq + 2 * hkv) * d, dtype=g.q.dtype, device=DEV)
+    qv, kv_, vv = qkv.split([hq * d, hkv * d, hkv * d], dim=1)
+    qv = qv.view(T, hq, d); kv_ = kv_.view(T, hkv, d); vv = vv.view(T, hkv, d)
+    qv.copy_(g.q); kv_.copy_(g.k); vv.copy_(g.v)
+    obuf = torch.zeros(T, hq * d + 256, dtype=g.q.dtype, device=DEV)
+    ov = obuf[:, :hq * d].view(T, hq, d)
+    assert not qv.is_contiguous() and not ov.is_contiguous()
+    g.q, g.k, g.v = qv, kv_, vv
+    for nsplit in (1, 3):
+        got = run_op(g, kernel=_ffi.KERNEL_MFMA, num_splits=nsplit, out=ov).cpu()
+        e = _err(got, ref)
+        assert e < 2e-2, (nsplit, e)
+    assert torch.all(obuf[:, hq * d:] == 0)
+
+
 @pytest.mark.parametrize("scale", [1e-6, 3e4])
 def test_mfma_split_partials_keep_their_precision_at_any_magnitude(scale):
     """Split-KV partial rows are stored as halves with one power-of-two scale per row: values far outside
