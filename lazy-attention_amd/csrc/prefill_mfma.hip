@@ -34,8 +34,6 @@ namespace lazyattn {
 namespace {
 
 
-constexpr int D = 128;          // head_dim
-constexpr int HALF = 64;
 constexpr int BS = 16;          // page size (tokens)
 constexpr int NT = 64;          // keys per tile
 constexpr int PAGES = NT / BS;  // pages per tile
@@ -43,12 +41,17 @@ constexpr int UNIT = 32;        // query rows per wave
 // LDS tiles (bytes).  K: [page][d8 = 16][slot = 16][8 bf16].
 // V: [page][g = 2][d = 128][slots 4g..4g+3 | slots 8+4g..8+4g+3] -- the 16 bytes one lane
 // feeds to the PV MFMA as its A operand.
-constexpr int K_PAGE = 4096;
-constexpr int K_TILE = PAGES * K_PAGE;
-constexpr int V_G = 2048;
-constexpr int V_PAGE = 2 * V_G;
-constexpr int V_TILE = PAGES * V_PAGE;
-constexpr int KV_BYTES = 2 * K_TILE + 2 * V_TILE;     // K and V tiles, double-buffered: 64 KB
+// Sizes that follow from the head size HD (128 or 64); a K page is HD * 32 bytes, a V page as well.
+template <int HD> struct Geo {
+    static constexpr int K_PAGE = HD * 32, K_TILE = PAGES * K_PAGE;
+    static constexpr int V_G = HD * 16, V_PAGE = 2 * V_G, V_TILE = PAGES * V_PAGE;
+    static constexpr int KV_BYTES = 2 * K_TILE + 2 * V_TILE;      // K and V tiles, double-buffered: 64 KB at 128
+    static constexpr int Q_WAVE = HD * 64;                        // Q^T fragments of one computing wave
+    static constexpr int KS = HD / 16, DT = HD / 32;              // k-steps of K.Q^T, 32-row blocks of O^T
+    static constexpr int K_ITEMS = HD / 64, V_ITEMS = HD / 32;    // 16-byte items per gathering lane and page
+    static constexpr int PAIR = (HD / 16) * 256;                  // bytes from the chunk of d to the chunk of d + HD/2 (16-bit cache)
+    static constexpr int PAIR8 = (HD / 32) * 256;                 // ... in an fp8 page
+};
 
 enum { TILE_FULL = 0, TILE_EDGE = 1, TILE_NEW = 2 };
 
@@ -125,14 +128,17 @@ template <typename TT> struct KRegs {
 // NC = computing waves = 32-row units per workgroup: 8 (12 waves, three per SIMD) for long
 // key ranges, 4 (8 waves) when the call is small and more, lighter workgroups fill the chip
 // with fewer key-axis splits.
-constexpr int lds_bytes(int nc) { return KV_BYTES + nc * 8 * 1024 + 2 * PAGES * 4; }   // + Q^T fragments (re-read every tile) + page limits
-constexpr int KI = 2;                    // K items per gathering lane and tile: a page has 128 (8 chunks x 16 slots)
-constexpr int VI = 4;                    // V items per gathering lane and tile: a page has 256 of 16 bytes
+template <int HD> constexpr int lds_bytes(int nc) { return Geo<HD>::KV_BYTES + nc * Geo<HD>::Q_WAVE + 2 * PAGES * 4; }   // + Q^T fragments (re-read every tile) + page limits
 
 // WIN: built with the sliding-window code (calls without a window run the instantiation without it)
-template <int NC, bool FP8, bool WIN, typename T, typename TT>
+template <int NC, int HD, bool FP8, bool WIN, typename T, typename TT>
 __global__ void __launch_bounds__((NC + 4) * 64)
 prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int n_mt) {
+    using G = Geo<HD>;
+    constexpr int D = HD, HALF = HD / 2;
+    constexpr int K_PAGE = G::K_PAGE, K_TILE = G::K_TILE, V_G = G::V_G, V_PAGE = G::V_PAGE, V_TILE = G::V_TILE;
+    constexpr int KV_BYTES = G::KV_BYTES, KS = G::KS, DT = G::DT;
+    constexpr int KI = G::K_ITEMS, VI = G::V_ITEMS;   // a page has HD K items (HD/16 chunk pairs x 16 slots) and 2 HD V items
     constexpr int VI_CTX = FP8 ? VI / 2 : VI;        // an fp8 page row of 16 slots is one 16-byte item
     constexpr uint32_t TSZ = sizeof(TT);
     using E = Elem<T>;
@@ -247,7 +253,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     };
     // Valid-slot counts of the four pages of a context tile, one int per page and LDS buffer:
     // written by the gathering waves with the tile, read by the computing waves for the masks.
-    int *page_lims = reinterpret_cast<int *>(lds + KV_BYTES + NC * 8192);
+    int *page_lims = reinterpret_cast<int *>(lds + KV_BYTES + NC * G::Q_WAVE);
 
     if (gatherer) {
         // ====================================================================== gather
@@ -299,12 +305,12 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             for (int i = 0; i < KI; ++i) {
                 kr[i].lds_off = (uint32_t)(gw * K_PAGE + (lane + i * 64) * 16);
                 if (FP8) {
-                    const uint2 a = ldg8(kb, k_goff[i]), a2 = ldg8(kb, k_goff[i] + 4 * 256);
+                    const uint2 a = ldg8(kb, k_goff[i]), a2 = ldg8(kb, k_goff[i] + G::PAIR8);
                     kr[i].k1 = make_uint4(a.x, a.y, 0, 0);
                     kr[i].k2 = make_uint4(a2.x, a2.y, 0, 0);
                 } else {
                     kr[i].k1 = ldg16(kb, k_goff[i]);
-                    kr[i].k2 = ldg16(kb, k_goff[i] + 2048);
+                    kr[i].k2 = ldg16(kb, k_goff[i] + G::PAIR);
                 }
                 kr[i].c.load(tb, k_toff[i]);
                 kr[i].s.load(tb, k_toff[i] + sin_delta);
@@ -319,29 +325,34 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
 #pragma unroll
             for (int i = 0; i < KI; ++i) {
                 const int idx = lane + i * 64;
-                const int cp = idx & 7, kl = idx >> 3, m = m0 + kl;
+                const int cp = idx & (D / 16 - 1), kl = idx / (D / 16), m = m0 + kl;
                 kr[i].lds_off = (uint32_t)(gw * K_PAGE + cp * 256 + kl * 16);
-                kr[i].k1 = make_uint4(0, 0, 0, 0); kr[i].k2 = kr[i].k1;
-                kr[i].c.fill(1.f); kr[i].s.fill(0.f);
+                uint4 k1 = make_uint4(0, 0, 0, 0), k2 = k1;
+                TabVec<TT> c, sn;
+                c.fill(1.f); sn.fill(0.f);
                 if (m < t_end) {
                     const T *kn = (const T *)p.k + (qs + m) * p.k_stride[0] + (int64_t)g * p.k_stride[1] + cp * 8;
-                    kr[i].k1 = *reinterpret_cast<const uint4 *>(kn);
-                    kr[i].k2 = *reinterpret_cast<const uint4 *>(kn + HALF);
+                    k1 = *reinterpret_cast<const uint4 *>(kn);
+                    k2 = *reinterpret_cast<const uint4 *>(kn + HALF);
                     if (rot_new) {                                               // old_ops:342-343
                         const uint8_t *tb = tab_base + (int64_t)(ctx_len + m) * row_bytes;
-                        kr[i].c.load(tb, (uint32_t)cp * 8 * TSZ);
-                        kr[i].s.load(tb, (uint32_t)cp * 8 * TSZ + HALF * TSZ);
+                        c.load(tb, (uint32_t)cp * 8 * TSZ);
+                        sn.load(tb, (uint32_t)cp * 8 * TSZ + HALF * TSZ);
                     }
                 }
+                kr[i].k1 = k1; kr[i].k2 = k2; kr[i].c = c; kr[i].s = sn;
             }
 #pragma unroll
             for (int i = 0; i < VI; ++i) {
                 const int idx = lane + i * 64;
-                const int dc = idx & 15, m = m0 + (idx >> 4);
-                vr[i] = make_uint4(0, 0, 0, 0);
+                const int dc = idx & (D / 8 - 1), m = m0 + idx / (D / 8);
+                // (the value is chosen before the one store: a store under the branch lets the compiler merge
+                // the iterations' stores behind a pointer phi, and the array then stays in scratch memory)
+                uint4 t = make_uint4(0, 0, 0, 0);
                 if (m < t_end)
-                    vr[i] = *reinterpret_cast<const uint4 *>((const T *)p.v + (qs + m) * p.v_stride[0] +
-                                                             (int64_t)g * p.v_stride[1] + dc * 8);
+                    t = *reinterpret_cast<const uint4 *>((const T *)p.v + (qs + m) * p.v_stride[0] +
+                                                         (int64_t)g * p.v_stride[1] + dc * 8);
+                vr[i] = t;
             }
         };
         // kind of this wave's part of a tile, and its loads
@@ -377,7 +388,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                 }
                 *reinterpret_cast<uint4 *>(ktile + kr[i].lds_off) = make_uint4(
                     E::pack(x[0], x[1]), E::pack(x[2], x[3]), E::pack(x[4], x[5]), E::pack(x[6], x[7]));
-                *reinterpret_cast<uint4 *>(ktile + kr[i].lds_off + 8 * 256) = make_uint4(
+                *reinterpret_cast<uint4 *>(ktile + kr[i].lds_off + G::PAIR) = make_uint4(
                     E::pack(y[0], y[1]), E::pack(y[2], y[3]), E::pack(y[4], y[5]), E::pack(y[6], y[7]));
             }
         };
@@ -388,7 +399,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
 #pragma unroll
                 for (int i = 0; i < VI; ++i) {
                     const int idx = lane + i * 64;
-                    const int dc = idx & 15, slot = idx >> 4;
+                    const int dc = idx & (D / 8 - 1), slot = idx / (D / 8);
                     uint8_t *dst = vtile + gw * V_PAGE + ((slot >> 2) & 1) * V_G + (dc * 8) * 16 + (slot >> 3) * 8 +
                                    (slot & 3) * 2;
                     const uint32_t w[4] = {vr[i].x, vr[i].y, vr[i].z, vr[i].w};
@@ -510,11 +521,11 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     // reference scales the fp32 scores, old_ops:287; the extra rounding of Q is one more relative
     // 2^-9 per element, like the one the rotated K already carries).
     const float cs2 = p.sm_scale * 1.4426950408889634f;
-    uint8_t *qlds = lds + KV_BYTES + wave * 8192 + lane * 16;
+    uint8_t *qlds = lds + KV_BYTES + wave * G::Q_WAVE + lane * 16;
     {
         const T *qp = (const T *)p.q + (qs + row) * p.q_stride[0] + (int64_t)h * p.q_stride[1] + gh * 8;
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
+        for (int ks = 0; ks < KS; ++ks) {
             uint4 v = make_uint4(0, 0, 0, 0);
             if (row_ok) v = *reinterpret_cast<const uint4 *>(qp + ks * 16);
             float f[8];
@@ -535,9 +546,9 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     f32x16_t cinit;                                                 // -m_ref in every element
 #pragma unroll
     for (int i = 0; i < 16; ++i) cinit[i] = 0.f;
-    f32x16_t acc[4];
+    f32x16_t acc[DT];
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[dt][i] = 0.f;
 
@@ -559,8 +570,8 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         fetch(0);
         fetch(1);
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
-            if (ks + 2 < 8) fetch(ks + 2);
+        for (int ks = 0; ks < KS; ++ks) {
+            if (ks + 2 < KS) fetch(ks + 2);
             s0 = E::mfma(a0[ks % 3], q[ks % 3], ks ? s0 : cinit);
             s1 = E::mfma(a1[ks % 3], q[ks % 3], ks ? s1 : cinit);
             __builtin_amdgcn_sched_barrier(0);
@@ -596,7 +607,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         if (__builtin_amdgcn_ballot_w64(delta != 0.f)) {
             const float alpha = seen ? __builtin_amdgcn_exp2f(-delta) : 1.f;   // nothing accumulated before the first key
 #pragma unroll
-            for (int dt = 0; dt < 4; ++dt) acc[dt] *= alpha;
+            for (int dt = 0; dt < DT; ++dt) acc[dt] *= alpha;
             l_run *= alpha;
             l_alt *= alpha;
             s0 -= delta;
@@ -625,16 +636,16 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     // k index j of a 16-key step <-> slot 4*gh + j (j < 4), 8 + 4*gh + j - 4 (j >= 4)
     auto pv_half = [&](const uint8_t *vtile, int sub, const uint4 &p0, const uint4 &p1) {
         const uint8_t *vp = vtile + (sub * 2) * V_PAGE + gh * V_G + l32 * 16;
-        // eight MFMAs: 32-row blocks of d 0..3 for the first page of the half, then for the second;
+        // 2 DT MFMAs: the 32-row blocks of d for the first page of the half, then for the second;
         // their V^T operands are requested two MFMAs ahead
         uint4 a[3];
-        auto fetch = [&](int j) { a[j % 3] = *reinterpret_cast<const uint4 *>(vp + (j >> 2) * V_PAGE + (j & 3) * 512); };
+        auto fetch = [&](int j) { a[j % 3] = *reinterpret_cast<const uint4 *>(vp + (j / DT) * V_PAGE + (j % DT) * 512); };
         fetch(0);
         fetch(1);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            if (j + 2 < 8) fetch(j + 2);
-            acc[j & 3] = E::mfma(a[j % 3], j < 4 ? p0 : p1, acc[j & 3]);
+        for (int j = 0; j < 2 * DT; ++j) {
+            if (j + 2 < 2 * DT) fetch(j + 2);
+            acc[j % DT] = E::mfma(a[j % 3], j < DT ? p0 : p1, acc[j % DT]);
         }
     };
     auto attend = [&](const uint8_t *vtile, f32x16_t &s0, f32x16_t &s1) {
@@ -702,7 +713,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     if (nsplit == 1) {
         T *op = (T *)p.o + (qs + row) * p.o_stride[0] + (int64_t)h * p.o_stride[1];
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+        for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) {
                 const int d = dt * 32 + 8 * i4 + 4 * gh;
@@ -717,7 +728,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         // row's largest element -- an eighth of the rounding of the bf16 output.
         float am = 0.f;
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+        for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int i = 0; i < 16; i += 2) am = max3(am, fabsf(acc[dt][i]), fabsf(acc[dt][i + 1]));
         am = fmaxf(am, partner32(am, gh != 0)) * inv;
@@ -730,7 +741,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         float2 *wl = reinterpret_cast<float2 *>(wo + (int64_t)nsplit * NTOK * p.num_q_heads * D);
         const int64_t r_idx = ((int64_t)split * NTOK + (qs + row)) * p.num_q_heads + h;
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+        for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) {
                 const int d = dt * 32 + 8 * i4 + 4 * gh;
@@ -754,19 +765,20 @@ struct MergeArgs {
     int64_t o_stride[2];
     int32_t num_tokens, num_q_heads, index_bits, skip_decode;
 };
-template <typename T>
+template <typename T, int HD>
 __global__ void __launch_bounds__(256)
 prefill_combine_kernel(const MergeArgs p, const int nsplit) {
     using E = Elem<T>;
+    constexpr int D = HD, LPR = HD / 4;                       // lanes per row (4 elements each)
     const int b = blockIdx.y;
     const int64_t qs = load_index(p.b_start_loc, b, p.index_bits);
     const int64_t q_len = load_index(p.b_start_loc, b + 1, p.index_bits) - qs;
     if (q_len <= 0 || (p.skip_decode && q_len == 1)) return;
-    const int64_t r = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);
+    const int64_t r = (int64_t)blockIdx.x * (256 / LPR) + threadIdx.x / LPR;
     if (r >= q_len * p.num_q_heads) return;
     const int64_t tok = qs + r / p.num_q_heads;
     const int h = (int)(r % p.num_q_heads);
-    const int d = (threadIdx.x & 31) * 4;
+    const int d = (threadIdx.x % LPR) * 4;
     const int64_t NTOK = p.num_tokens;
     const _Float16 *wo = (const _Float16 *)p.workspace;
     const float2 *wl = reinterpret_cast<const float2 *>(wo + (int64_t)nsplit * NTOK * p.num_q_heads * D);
@@ -811,7 +823,7 @@ prefill_combine_kernel(const MergeArgs p, const int nsplit) {
 
 // ------------------------------------------------------------------ host side
 // a split-KV partial row: 128 halves + (log2-sum-exp, scale)
-constexpr size_t PARTIAL_ROW_BYTES = D * sizeof(_Float16) + 2 * sizeof(float);
+static size_t partial_row_bytes(const lazyattn_prefill_params &p) { return (size_t)p.head_dim * sizeof(_Float16) + 2 * sizeof(float); }
 static int mfma_units(const lazyattn_prefill_params &p) {
     const int group = p.num_q_heads / p.num_kv_heads;
     return ((p.max_q_len + UNIT - 1) / UNIT) * group;
@@ -845,7 +857,9 @@ bool mfma_supports(const lazyattn_prefill_params &p) {
     if (p.dtype != LAZYATTN_BF16 && p.dtype != LAZYATTN_F16) return false;
     if (!(p.cache_dtype == p.dtype || fp8)) return false;
     if (p.table_dtype != p.dtype && p.table_dtype != LAZYATTN_F32) return false;
-    if (p.head_dim != D || p.block_size != BS || p.x != (fp8 ? 16 : 8)) return false;
+    if ((p.head_dim != 128 && p.head_dim != 64) || p.rotary_dim != p.head_dim) return false;
+    if (p.head_dim == 64 && p.sliding_window > 0) return false;     // the 64-wide kernels are built without the window code
+    if (p.block_size != BS || p.x != (fp8 ? 16 : 8)) return false;
     if (p.q_stride[2] != 1 || p.k_stride[2] != 1 || p.v_stride[2] != 1 || p.o_stride[2] != 1) return false;
     if (p.kc_stride[4] != 1 || p.kc_stride[3] != p.x || p.kc_stride[2] != (int64_t)BS * p.x) return false;
     if (p.vc_stride[3] != 1 || p.vc_stride[2] != BS) return false;
@@ -865,13 +879,13 @@ size_t mfma_workspace_bytes(const lazyattn_prefill_params &p) {
     const int nw = mfma_waves(p);
     const int ns = mfma_splits(p, nw);
     if (ns <= 1) return 0;
-    return (size_t)ns * (size_t)p.num_tokens * p.num_q_heads * PARTIAL_ROW_BYTES;
+    return (size_t)ns * (size_t)p.num_tokens * p.num_q_heads * partial_row_bytes(p);
 }
 
-template <int NC, bool FP8, bool WIN, typename T, typename TT>
+template <int NC, int HD, bool FP8, bool WIN, typename T, typename TT>
 static int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt, hipStream_t stream) {
-    auto kern = prefill_mfma_kernel<NC, FP8, WIN, T, TT>;
-    constexpr int LDS_BYTES = lds_bytes(NC);
+    auto kern = prefill_mfma_kernel<NC, HD, FP8, WIN, T, TT>;
+    constexpr int LDS_BYTES = lds_bytes<HD>(NC);
     static bool attr_set = false;
     if (!attr_set) {
         if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
@@ -883,20 +897,20 @@ static int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt,
     return hipGetLastError() == hipSuccess ? LAZYATTN_OK : LAZYATTN_E_LAUNCH;
 }
 
-template <int NC, typename T>
-static int launch_mfma_nc(const lazyattn_prefill_params &p, int nsplit, int n_mt, hipStream_t stream) {
+template <int NC, int HD, bool WIN, typename T>
+static int launch_mfma_hd(const lazyattn_prefill_params &p, int nsplit, int n_mt, hipStream_t stream) {
     const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3;
     const bool t32 = p.table_dtype == LAZYATTN_F32;
-    if (p.sliding_window > 0) {
-        if (fp8) return t32 ? launch_mfma_t<NC, true, true, T, float>(p, nsplit, n_mt, stream)
-                            : launch_mfma_t<NC, true, true, T, T>(p, nsplit, n_mt, stream);
-        return t32 ? launch_mfma_t<NC, false, true, T, float>(p, nsplit, n_mt, stream)
-                   : launch_mfma_t<NC, false, true, T, T>(p, nsplit, n_mt, stream);
-    }
-    if (fp8) return t32 ? launch_mfma_t<NC, true, false, T, float>(p, nsplit, n_mt, stream)
-                        : launch_mfma_t<NC, true, false, T, T>(p, nsplit, n_mt, stream);
-    return t32 ? launch_mfma_t<NC, false, false, T, float>(p, nsplit, n_mt, stream)
-               : launch_mfma_t<NC, false, false, T, T>(p, nsplit, n_mt, stream);
+    if (fp8) return t32 ? launch_mfma_t<NC, HD, true, WIN, T, float>(p, nsplit, n_mt, stream)
+                        : launch_mfma_t<NC, HD, true, WIN, T, T>(p, nsplit, n_mt, stream);
+    return t32 ? launch_mfma_t<NC, HD, false, WIN, T, float>(p, nsplit, n_mt, stream)
+               : launch_mfma_t<NC, HD, false, WIN, T, T>(p, nsplit, n_mt, stream);
+}
+template <int NC, typename T>
+static int launch_mfma_nc(const lazyattn_prefill_params &p, int nsplit, int n_mt, hipStream_t stream) {
+    if (p.head_dim == 64) return launch_mfma_hd<NC, 64, false, T>(p, nsplit, n_mt, stream);
+    if (p.sliding_window > 0) return launch_mfma_hd<NC, 128, true, T>(p, nsplit, n_mt, stream);
+    return launch_mfma_hd<NC, 128, false, T>(p, nsplit, n_mt, stream);
 }
 
 int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
@@ -905,7 +919,7 @@ int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
     const int n_mt = mfma_mtiles(p, nw);
     const int phases = p.phases ? p.phases : LAZYATTN_PHASE_ALL;
     if (nsplit > 1) {
-        const size_t need = (size_t)nsplit * (size_t)p.num_tokens * p.num_q_heads * PARTIAL_ROW_BYTES;
+        const size_t need = (size_t)nsplit * (size_t)p.num_tokens * p.num_q_heads * partial_row_bytes(p);
         if (!p.workspace || (size_t)p.workspace_bytes < need) return LAZYATTN_E_WORKSPACE;
         if (((uintptr_t)p.workspace) & 15) return LAZYATTN_E_WORKSPACE;
     }
@@ -919,9 +933,16 @@ int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
         const int64_t rows = (int64_t)p.max_q_len * p.num_q_heads;
         const MergeArgs m{p.workspace, p.b_start_loc, p.o, {p.o_stride[0], p.o_stride[1]}, p.num_tokens, p.num_q_heads,
                           p.index_bits, p.skip_decode};
-        const dim3 grid((unsigned)((rows + 7) / 8), p.batch);
-        if (p.dtype == LAZYATTN_F16) hipLaunchKernelGGL(prefill_combine_kernel<f16_t>, grid, dim3(256), 0, stream, m, nsplit);
-        else hipLaunchKernelGGL(prefill_combine_kernel<bf16_t>, grid, dim3(256), 0, stream, m, nsplit);
+        const int rows_wg = 256 / (p.head_dim / 4);
+        const dim3 grid((unsigned)((rows + rows_wg - 1) / rows_wg), p.batch);
+        const bool f16 = p.dtype == LAZYATTN_F16;
+        if (p.head_dim == 64) {
+            if (f16) hipLaunchKernelGGL((prefill_combine_kernel<f16_t, 64>), grid, dim3(256), 0, stream, m, nsplit);
+            else hipLaunchKernelGGL((prefill_combine_kernel<bf16_t, 64>), grid, dim3(256), 0, stream, m, nsplit);
+        } else {
+            if (f16) hipLaunchKernelGGL((prefill_combine_kernel<f16_t, 128>), grid, dim3(256), 0, stream, m, nsplit);
+            else hipLaunchKernelGGL((prefill_combine_kernel<bf16_t, 128>), grid, dim3(256), 0, stream, m, nsplit);
+        }
         if (hipGetLastError() != hipSuccess) return LAZYATTN_E_LAUNCH;
     }
     return LAZYATTN_OK;

@@ -122,6 +122,22 @@ def test_mfma_takes_views_of_a_packed_qkv_tensor():
     assert torch.all(obuf[:, hq * d:] == 0)
 
 
+@pytest.mark.parametrize("variant", ["natural", "offset", "block_uniform"])
+@pytest.mark.parametrize("dtype,kv", [(torch.bfloat16, "auto"), (torch.float16, "auto"), (torch.bfloat16, "fp8")])
+def test_mfma_head_dim_64(variant, dtype, kv):
+    """Llama-3.2-1B geometry (head_dim 64, the reference's plumbing configuration) on the matrix path."""
+    print(f"case: mfma head_dim 64 {variant} {dtype} kv={kv}", flush=True)
+    w = wl.make_workload("ragged64", dtype=dtype, hq=32, hkv=8, d=64, theta=500000.0, block_size=16,
+                         doc_lens=[100, 16, 333, 70, 5, 250], requests=[[3, 1, 0], [2], [0, 2, 3, 1, 5], [4], []],
+                         q_lens=[70, 1, 9, 33, 130], variant=variant, kv_cache_dtype=kv, seed=64)
+    ref = run_oracle(w)
+    tol = 5e-2 if kv == "fp8" else (2e-2 if dtype == torch.bfloat16 else 5e-3)
+    for nsplit, kernel in ((1, _ffi.KERNEL_MFMA4), (3, _ffi.KERNEL_MFMA8)):
+        got = run_op(w.to(DEV), kernel=kernel, num_splits=nsplit).cpu()
+        e = _err(got, ref)
+        assert e < tol, (nsplit, e)
+
+
 @pytest.mark.parametrize("scale", [1e-6, 3e4])
 def test_mfma_split_partials_keep_their_precision_at_any_magnitude(scale):
     """Split-KV partial rows are stored as halves with one power-of-two scale per row: values far outside
