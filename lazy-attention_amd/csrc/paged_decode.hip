@@ -24,14 +24,13 @@
 // Slices of one request are merged by paged_decode_merge_kernel.
 #include "common.hpp"
 #include "elem16.hpp"
+#include <type_traits>
 
 namespace lazyattn {
 
 namespace {
 
 
-constexpr int D = 128;
-constexpr int HALF = 64;
 constexpr int BS = 16;
 constexpr int WAVES = 4;            // independent waves per workgroup
 
@@ -68,22 +67,25 @@ template <> struct Tab8<float> {
 };
 
 // what one page contributes, as loaded: the key side and the value side travel separately
-template <typename TT> struct KeyRegs {
-    uint4 k[4];                 // chunks grp, 4 + grp, 8 + grp, 12 + grp of token t
-    Tab8<TT> c0, s0, c1, s1;    // cos / sin for d = 8 grp .. (pair k[0], k[2]) and d = 32 + 8 grp .. (pair k[1], k[3])
+// HD = head size (128 or 64): HD/32 key chunks per lane (one per MFMA of the scores), HD/64 rotation pair
+// sets, HD/16 row blocks of V
+template <typename TT, int HD> struct KeyRegs {
+    uint4 k[HD / 32];           // chunks grp, 4 + grp, ... of token t; k[j] pairs with k[j + HD/64]
+    Tab8<TT> c[HD / 64], s[HD / 64];   // cos / sin for d = 32 j + 8 grp ..
     int lim;                    // valid slots
     int first;                  // first slot inside the sliding window (<= 0: all)
 };
-struct ValRegs {
-    uint2 v[8];                 // V[d = 16 blk + t][tokens 4 grp .. 4 grp + 3]
+template <int HD> struct ValRegs {
+    uint2 v[HD / 16];           // V[d = 16 blk + t][tokens 4 grp .. 4 grp + 3]
 };
 
 }  // namespace
 
-template <typename T, typename TT, bool FP8>
+template <typename T, typename TT, bool FP8, int HD>
 __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2)))
 paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     using E = Elem<T>;
+    constexpr int D = HD, HALF = HD / 2, NM = HD / 32, NP = HD / 64, NBLK = HD / 16;
     constexpr int TSZ = sizeof(TT);
     const int lane = threadIdx.x & 63;
     const int wave = uniform(threadIdx.x >> 6);
@@ -146,7 +148,7 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
         jc = jc < 0 ? 0 : jc;
         return bt_row[jc * bt_s1];
     };
-    auto load_keys = [&](int j, KeyRegs<TT> &r) {
+    auto load_keys = [&](int j, KeyRegs<TT, HD> &r) {
         int jc = j < n_pages ? j : n_pages - 1;
         jc = jc < 0 ? 0 : jc;
         const int bt = bt_row[jc * bt_s1];
@@ -159,7 +161,7 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
         r.first = first_key - j * BS;                                                // slots below it lie before the window
         const uint8_t *kb = kc_base + bt * kc_page_bytes;
 #pragma unroll
-        for (int m = 0; m < 4; ++m) {
+        for (int m = 0; m < NM; ++m) {
             if (FP8) {
                 const uint2 w = *reinterpret_cast<const uint2 *>(kb + k_off + m * K_STEP);
                 r.k[m] = make_uint4(w.x, w.y, 0, 0);
@@ -176,15 +178,16 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
             pos = pos < 0 ? 0 : pos;
         }
         const uint8_t *row = tab + (int64_t)pos * row_bytes;
-        r.c0.load(row, 8 * grp);
-        r.s0.load(row, HALF + 8 * grp);
-        r.c1.load(row, 32 + 8 * grp);
-        r.s1.load(row, HALF + 32 + 8 * grp);
+#pragma unroll
+        for (int j = 0; j < NP; ++j) {
+            r.c[j].load(row, 32 * j + 8 * grp);
+            r.s[j].load(row, HALF + 32 * j + 8 * grp);
+        }
     };
-    auto load_values = [&](int j, ValRegs &r) {
+    auto load_values = [&](int j, ValRegs<HD> &r) {
         const uint8_t *vb = vc_base + page_block(j) * vc_page_bytes;
 #pragma unroll
-        for (int blk = 0; blk < 8; ++blk) {
+        for (int blk = 0; blk < NBLK; ++blk) {
             if (FP8) r.v[blk] = make_uint2(*reinterpret_cast<const uint32_t *>(vb + v_off + blk * V_STEP), 0);
             else r.v[blk] = *reinterpret_cast<const uint2 *>(vb + v_off + blk * V_STEP);
         }
@@ -211,12 +214,12 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     };
 
     // Q^T: column = head = t, contraction d = 32 m + 8 grp ..
-    uint4 qf[4];
+    uint4 qf[NM];
     {
         const bool head_ok = t < group;
         const T *qp = (const T *)p.q + qs * p.q_stride[0] + (int64_t)(g * group + (head_ok ? t : 0)) * p.q_stride[1] + 8 * grp;
 #pragma unroll
-        for (int m = 0; m < 4; ++m) {
+        for (int m = 0; m < NM; ++m) {
             uint4 w = make_uint4(0, 0, 0, 0);
             if (head_ok) w = *reinterpret_cast<const uint4 *>(qp + 32 * m);
             qf[m] = w;
@@ -224,20 +227,18 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     }
     const float cs2 = p.sm_scale * 1.4426950408889634f;
     float m_run = -INFINITY, l_run = 0.f;
-    f32x4_t acc[8];
+    f32x4_t acc[NBLK];
 #pragma unroll
-    for (int blk = 0; blk < 8; ++blk) acc[blk] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int blk = 0; blk < NBLK; ++blk) acc[blk] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     // scores of one page: S^T[token 4 grp + i][head t], masked
-    auto scores = [&](const KeyRegs<TT> &r) -> f32x4_t {
-        uint4 k0, k1, k2, k3;
-        rotate(r.k[0], r.k[2], r.c0, r.s0, k0, k2);
-        rotate(r.k[1], r.k[3], r.c1, r.s1, k1, k3);
+    auto scores = [&](const KeyRegs<TT, HD> &r) -> f32x4_t {
+        uint4 kk[NM];
+#pragma unroll
+        for (int j = 0; j < NP; ++j) rotate(r.k[j], r.k[j + NP], r.c[j], r.s[j], kk[j], kk[j + NP]);
         f32x4_t s = {0.f, 0.f, 0.f, 0.f};
-        s = E::mfma16(k0, qf[0], s);
-        s = E::mfma16(k1, qf[1], s);
-        s = E::mfma16(k2, qf[2], s);
-        s = E::mfma16(k3, qf[3], s);
+#pragma unroll
+        for (int m = 0; m < NM; ++m) s = E::mfma16(kk[m], qf[m], s);
         if (r.lim < BS || r.first > 0) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) s[i] = (4 * grp + i < r.lim && 4 * grp + i >= r.first) ? s[i] : -INFINITY;
@@ -245,7 +246,7 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
         return s;
     };
     // V words of a page with the masked tokens zeroed (a masked slot may hold anything)
-    auto masked_v = [&](const ValRegs &r, int lim, int blk) -> uint2 {
+    auto masked_v = [&](const ValRegs<HD> &r, int lim, int blk) -> uint2 {
         uint2 w = r.v[blk];
         if (FP8) {
             const f32x2_t lo = __builtin_amdgcn_cvt_pk_f32_fp8(w.x, false), hi = __builtin_amdgcn_cvt_pk_f32_fp8(w.x >> 16, false);
@@ -263,13 +264,13 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     // The key side of pair i+1 is requested as soon as the scores of pair i have consumed the
     // registers it lands in, the value side of pair i at the top of its iteration: every load has
     // about half an iteration of other work between issue and use, at no extra registers.
-    KeyRegs<TT> KX, KY;
+    KeyRegs<TT, HD> KX, KY;
     if (pair_begin < pair_end) {
         load_keys(2 * pair_begin, KX);
         load_keys(2 * pair_begin + 1, KY);
     }
     for (int pr = pair_begin; pr < pair_end; ++pr) {
-        ValRegs X, Y;
+        ValRegs<HD> X, Y;
         load_values(2 * pr, X);
         load_values(2 * pr + 1, Y);
         const f32x4_t sx = scores(KX), sy = scores(KY);
@@ -287,7 +288,7 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
         const float alpha = __builtin_amdgcn_exp2f((m_run - m_safe) * cs2);
         if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
 #pragma unroll
-            for (int blk = 0; blk < 8; ++blk) acc[blk] *= alpha;
+            for (int blk = 0; blk < NBLK; ++blk) acc[blk] *= alpha;
             l_run *= alpha;
         }
         m_run = m_new;
@@ -301,7 +302,7 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
         l_run += (px[0] + px[1]) + (px[2] + px[3]) + (py[0] + py[1]) + (py[2] + py[3]);
         const uint4 pf = make_uint4(E::pack(px[0], px[1]), E::pack(px[2], px[3]), E::pack(py[0], py[1]), E::pack(py[2], py[3]));
 #pragma unroll
-        for (int blk = 0; blk < 8; ++blk) {
+        for (int blk = 0; blk < NBLK; ++blk) {
             const uint2 vx = masked_v(X, lim_x, blk), vy = masked_v(Y, lim_y, blk);
             acc[blk] = E::mfma16(make_uint4(vx.x, vx.y, vy.x, vy.y), pf, acc[blk]);
         }
@@ -316,7 +317,7 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     if (nsplit == 1) {
         T *op = (T *)p.o + qs * p.o_stride[0] + (int64_t)h * p.o_stride[1] + 4 * grp;
 #pragma unroll
-        for (int blk = 0; blk < 8; ++blk)
+        for (int blk = 0; blk < NBLK; ++blk)
             *reinterpret_cast<uint2 *>(op + 16 * blk) =
                 make_uint2(E::pack(acc[blk][0] * inv, acc[blk][1] * inv), E::pack(acc[blk][2] * inv, acc[blk][3] * inv));
         return;
@@ -326,7 +327,7 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     float *wl = wo + (int64_t)nsplit * p.batch * p.num_q_heads * D;
     const int64_t r_idx = ((int64_t)split * p.batch + b) * p.num_q_heads + h;
 #pragma unroll
-    for (int blk = 0; blk < 8; ++blk)
+    for (int blk = 0; blk < NBLK; ++blk)
         *reinterpret_cast<float4 *>(wo + r_idx * D + 16 * blk + 4 * grp) =
             make_float4(acc[blk][0] * inv, acc[blk][1] * inv, acc[blk][2] * inv, acc[blk][3] * inv);
     if (grp == 0) wl[r_idx] = l_run > 0.f ? m_run * cs2 + __builtin_amdgcn_logf(l_run) : -INFINITY;
@@ -341,16 +342,17 @@ struct DecodeMergeArgs {
     int64_t o_stride[2];
     int32_t batch, num_q_heads, index_bits;
 };
-template <typename T>
+template <typename T, int HD>
 __global__ void __launch_bounds__(256)
 paged_decode_merge_kernel(const DecodeMergeArgs p, const int nsplit) {
     using E = Elem<T>;
-    const int64_t r = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);
+    constexpr int D = HD, LPR = HD / 4;                       // lanes per row (4 elements each)
+    const int64_t r = (int64_t)blockIdx.x * (256 / LPR) + threadIdx.x / LPR;
     if (r >= (int64_t)p.batch * p.num_q_heads) return;
     const int b = (int)(r / p.num_q_heads), h = (int)(r % p.num_q_heads);
     const int64_t qs = load_index(p.b_start_loc, b, p.index_bits);
     if (load_index(p.b_start_loc, b + 1, p.index_bits) - qs != 1) return;
-    const int d = (threadIdx.x & 31) * 4;
+    const int d = (threadIdx.x % LPR) * 4;
     const float *wo = (const float *)p.workspace;
     const float *wl = wo + (int64_t)nsplit * p.batch * p.num_q_heads * D;
     const int64_t rows = (int64_t)p.batch * p.num_q_heads;
@@ -393,7 +395,8 @@ bool decode_mfma_supports(const lazyattn_prefill_params &p) {
     const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3;
     if ((p.dtype != LAZYATTN_BF16 && p.dtype != LAZYATTN_F16) || !(p.cache_dtype == p.dtype || fp8)) return false;
     if (p.table_dtype != p.dtype && p.table_dtype != LAZYATTN_F32) return false;
-    if (p.head_dim != D || p.block_size != BS || p.x != (fp8 ? 16 : 8)) return false;
+    if ((p.head_dim != 128 && p.head_dim != 64) || p.rotary_dim != p.head_dim) return false;
+    if (p.block_size != BS || p.x != (fp8 ? 16 : 8)) return false;
     if (p.pos_mode != LAZYATTN_POS_NATURAL && p.pos_mode != LAZYATTN_POS_BLOCK_UNIFORM) return false;
     if (p.num_q_heads / p.num_kv_heads > 16) return false;
     if (p.q_stride[2] != 1 || p.o_stride[2] != 1) return false;
@@ -426,14 +429,14 @@ static int decode_splits(const lazyattn_prefill_params &p) {
 size_t decode_workspace_bytes(const lazyattn_prefill_params &p) {
     const int ns = decode_splits(p);
     if (ns <= 1) return 0;
-    return (size_t)ns * (size_t)p.batch * p.num_q_heads * (D + 1) * sizeof(float);
+    return (size_t)ns * (size_t)p.batch * p.num_q_heads * (p.head_dim + 1) * sizeof(float);
 }
 
 int launch_decode_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
     int nsplit = decode_splits(p);
     if (nsplit > 1) {
         // without room for the partials the call still runs, one slice per request and kv head
-        const size_t need = (size_t)nsplit * (size_t)p.batch * p.num_q_heads * (D + 1) * sizeof(float);
+        const size_t need = (size_t)nsplit * (size_t)p.batch * p.num_q_heads * (p.head_dim + 1) * sizeof(float);
         if (!p.workspace || (size_t)p.workspace_bytes < need || (((uintptr_t)p.workspace) & 15)) nsplit = 1;
     }
     const int phases = p.phases ? p.phases : LAZYATTN_PHASE_ALL;
@@ -442,22 +445,33 @@ int launch_decode_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
     if (phases & LAZYATTN_PHASE_MAIN) {
         const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3, t32 = p.table_dtype == LAZYATTN_F32;
         const dim3 grid(nblocks), block(WAVES * 64);
-        auto launch = [&](auto elem) {
+        auto launch = [&](auto elem, auto hd) {
             using T = decltype(elem);
-            if (fp8 && t32) hipLaunchKernelGGL((paged_decode_kernel<T, float, true>), grid, block, 0, stream, p, nsplit);
-            else if (fp8) hipLaunchKernelGGL((paged_decode_kernel<T, T, true>), grid, block, 0, stream, p, nsplit);
-            else if (t32) hipLaunchKernelGGL((paged_decode_kernel<T, float, false>), grid, block, 0, stream, p, nsplit);
-            else hipLaunchKernelGGL((paged_decode_kernel<T, T, false>), grid, block, 0, stream, p, nsplit);
+            constexpr int HD = decltype(hd)::value;
+            if (fp8 && t32) hipLaunchKernelGGL((paged_decode_kernel<T, float, true, HD>), grid, block, 0, stream, p, nsplit);
+            else if (fp8) hipLaunchKernelGGL((paged_decode_kernel<T, T, true, HD>), grid, block, 0, stream, p, nsplit);
+            else if (t32) hipLaunchKernelGGL((paged_decode_kernel<T, float, false, HD>), grid, block, 0, stream, p, nsplit);
+            else hipLaunchKernelGGL((paged_decode_kernel<T, T, false, HD>), grid, block, 0, stream, p, nsplit);
         };
-        if (p.dtype == LAZYATTN_F16) launch(f16_t{}); else launch(bf16_t{});
+        using hd128 = std::integral_constant<int, 128>;
+        using hd64 = std::integral_constant<int, 64>;
+        if (p.head_dim == 64) { if (p.dtype == LAZYATTN_F16) launch(f16_t{}, hd64{}); else launch(bf16_t{}, hd64{}); }
+        else { if (p.dtype == LAZYATTN_F16) launch(f16_t{}, hd128{}); else launch(bf16_t{}, hd128{}); }
         if (hipGetLastError() != hipSuccess) return LAZYATTN_E_LAUNCH;
     }
     if (nsplit > 1 && (phases & LAZYATTN_PHASE_COMBINE)) {
         const int64_t rows = (int64_t)p.batch * p.num_q_heads;
         const DecodeMergeArgs m{p.workspace, p.b_start_loc, p.o, {p.o_stride[0], p.o_stride[1]}, p.batch, p.num_q_heads, p.index_bits};
-        const dim3 mgrid((unsigned)((rows + 7) / 8));
-        if (p.dtype == LAZYATTN_F16) hipLaunchKernelGGL(paged_decode_merge_kernel<f16_t>, mgrid, dim3(256), 0, stream, m, nsplit);
-        else hipLaunchKernelGGL(paged_decode_merge_kernel<bf16_t>, mgrid, dim3(256), 0, stream, m, nsplit);
+        const int rows_wg = 256 / (p.head_dim / 4);
+        const dim3 mgrid((unsigned)((rows + rows_wg - 1) / rows_wg));
+        const bool f16 = p.dtype == LAZYATTN_F16;
+        if (p.head_dim == 64) {
+            if (f16) hipLaunchKernelGGL((paged_decode_merge_kernel<f16_t, 64>), mgrid, dim3(256), 0, stream, m, nsplit);
+            else hipLaunchKernelGGL((paged_decode_merge_kernel<bf16_t, 64>), mgrid, dim3(256), 0, stream, m, nsplit);
+        } else {
+            if (f16) hipLaunchKernelGGL((paged_decode_merge_kernel<f16_t, 128>), mgrid, dim3(256), 0, stream, m, nsplit);
+            else hipLaunchKernelGGL((paged_decode_merge_kernel<bf16_t, 128>), mgrid, dim3(256), 0, stream, m, nsplit);
+        }
         if (hipGetLastError() != hipSuccess) return LAZYATTN_E_LAUNCH;
     }
     return LAZYATTN_OK;

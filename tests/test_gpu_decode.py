@@ -17,10 +17,9 @@ DEV = "cuda"
 
 
 def _decode_batch(variant, *, hq=8, hkv=2, q_lens=(1, 1, 1, 1, 1), table_f32=False, seed=77, kv="auto",
-                  dtype=torch.bfloat16):
+                  dtype=torch.bfloat16, d=128):
     """Ragged documents (pads at document ends), requests of 1 to 9 documents, one new token each
     (or more: such requests must be skipped)."""
-    d = 128
     w = wl.make_workload("decode", dtype=dtype, hq=hq, hkv=hkv, d=d, theta=500000.0, block_size=16,
                          doc_lens=[40, 16, 33, 70, 5, 128, 97],
                          requests=[[3, 1, 0], [2], [0, 2, 3, 1, 5, 6, 4, 5, 6], [4, 0], [6, 5, 3]],
@@ -61,7 +60,7 @@ def _run(w, *, lazy=None, num_splits=0, kernel=_ffi.KERNEL_AUTO, sliding_window=
         q=g.q, k=g.k, v=g.v, o=out, kv_cache_dtype=w.kv_cache_dtype, k_cache=g.k_cache, v_cache=g.v_cache,
         b_loc=g.block_table, b_start_loc=g.b_start_loc, b_seq_len=g.b_seq_len, max_input_len=1,
         max_seq_len=g.max_seq_len, k_scale=g.k_scale, v_scale=g.v_scale, alibi_slopes=None, sliding_window=sliding_window,
-        sm_scale=128 ** -0.5, skip_decode=False, cos_sin_cache=g.cos_sin_cache, rotary_dim=128,
+        sm_scale=g.q.shape[-1] ** -0.5, skip_decode=False, cos_sin_cache=g.cos_sin_cache, rotary_dim=g.q.shape[-1],
         is_neox_style=True, is_lazy=None if lazy is None else lazy.to(DEV),
         q_offset=g.q_offset if bu else None, q_mask=g.q_mask,
         pos_mode=_ffi.POS_BLOCK_UNIFORM if bu else _ffi.POS_NATURAL, rotate_new_k=not bu, decode=True,
@@ -154,6 +153,20 @@ def test_decode_sliding_window(variant, window):
         got = _run(w, num_splits=nsplit, sliding_window=window)
         assert _err(got, ref) < 2e-2, (nsplit, _err(got, ref))
     same = _run(w, kernel=_ffi.KERNEL_GENERIC, sliding_window=window)
+    assert _err(got, same) < 2e-2, _err(got, same)
+
+
+@pytest.mark.parametrize("variant", ["natural", "block_uniform"])
+@pytest.mark.parametrize("dtype,kv", [(torch.bfloat16, "auto"), (torch.float16, "auto"), (torch.bfloat16, "fp8")])
+def test_decode_head_dim_64(variant, dtype, kv):
+    print(f"case: decode head_dim 64 {variant} {dtype} kv={kv}", flush=True)
+    w = _decode_batch(variant, hq=16, hkv=4, kv=kv, dtype=dtype, d=64)
+    ref = _oracle(w)
+    tol = 5e-2 if kv == "fp8" else (2e-2 if dtype == torch.bfloat16 else 5e-3)
+    for nsplit in (1, 3):
+        got = _run(w, num_splits=nsplit)
+        assert _err(got, ref) < tol, (nsplit, _err(got, ref))
+    same = _run(w, kernel=_ffi.KERNEL_GENERIC)
     assert _err(got, same) < 2e-2, _err(got, same)
 
 
