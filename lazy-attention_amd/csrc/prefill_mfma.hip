@@ -299,7 +299,10 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             // set, else natural (old_ops:186-191); block-uniform: q_offset-1 if set, else 0 (ops:180-186);
             // un-rotated requests read row 0 of the table (cos 1, sin 0): exact identity.  pm.qo is 0
             // wherever q_offset is not consulted, nat_step is 0 wherever the fallback is row 0.
-            const int pos0 = pm.qo ? pm.qo - 1 : j * nat_step;
+            // A page past the context (its slots are all masked) takes the last page's position: the
+            // table only has to cover the positions of real keys.
+            const int jp = j < n_pages ? j : n_pages - 1;
+            const int pos0 = pm.qo ? pm.qo - 1 : jp * nat_step;
             const uint8_t *tb = ctab_base + (int64_t)pos0 * pos_bytes;
 #pragma unroll
             for (int i = 0; i < KI; ++i) {

@@ -149,14 +149,15 @@ def packed_cos_sin(table: torch.Tensor) -> Optional[torch.Tensor]:
     hit = _packed_tables.get(key)
     if hit is not None and hit[0] == table._version:
         return hit[1]
-    if len(_packed_tables) > 16:
+    if len(_packed_tables) >= 4:
         _packed_tables.clear()
     packed = torch.empty(table.shape[0] * table.shape[1], dtype=table.dtype, device=table.device)
     rc = lib().lazyattn_pack_cos_sin_cache(table.data_ptr(), packed.data_ptr(), dtype_code(table.dtype),
                                            table.stride(0), table.shape[0], table.shape[1],
                                            torch.cuda.current_stream(table.device).cuda_stream)
     check(rc, "lazyattn_pack_cos_sin_cache")
-    _packed_tables[key] = (table._version, packed)
+    # the entry holds the table too: while it is cached its address cannot be handed to another tensor
+    _packed_tables[key] = (table._version, packed, table)
     return packed
 
 

@@ -88,7 +88,7 @@ def launch_prefill(*, q, k, v, o, kv_cache_dtype, k_cache, v_cache, b_loc, b_sta
         k_scale = v_scale = None
     b_loc, q_offset, q_mask = _i32(b_loc), _i32(q_offset), _i32(q_mask)
     packed = None
-    if not decode and q.dtype == torch.bfloat16 and pos_mode != _ffi.POS_BLOCK_UNIFORM:
+    if not decode and q.dtype in (torch.bfloat16, torch.float16) and pos_mode != _ffi.POS_BLOCK_UNIFORM:
         packed = _ffi.packed_cos_sin(cos_sin_cache)      # built once per table
     p = _ffi.fill_params(
         q=q, k=k, v=v, o=o, k_cache=k_cache, v_cache=v_cache, block_table=b_loc,

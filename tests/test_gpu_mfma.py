@@ -98,6 +98,26 @@ def test_mfma_sliding_window(variant, window):
         assert e < 2e-2, (nsplit, e)
 
 
+@pytest.mark.parametrize("variant", ["natural", "offset"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_mfma_without_the_packed_table_and_a_table_of_exact_size(variant, dtype, monkeypatch):
+    """A C-ABI caller that passes no packed table: the per-token rotation reads the plain [rows, D]
+    table.  The table ends at the last real position (context 336 + 7 new tokens), while the last
+    context tile reaches slot 383: pages past the context must not read rows the table does not have."""
+    print(f"case: mfma unpacked table {variant} {dtype}", flush=True)
+    w = wl.make_workload("unpacked", dtype=dtype, **GEOM, doc_lens=[100, 5, 200, 65], requests=[[3], [0, 1, 2]],
+                         q_lens=[40, 7], variant=variant, seed=41)
+    rows = int(w.b_seq_len.max())
+    if variant == "natural":
+        w.cos_sin_cache = w.cos_sin_cache[:rows].clone()
+    ref = run_oracle(w)
+    monkeypatch.setattr(_ffi, "packed_cos_sin", lambda table: None)
+    for nsplit in (1, 2):
+        got = run_op(w.to(DEV), kernel=_ffi.KERNEL_MFMA, num_splits=nsplit).cpu()
+        e = _err(got, ref)
+        assert e < 2e-2, (nsplit, e)
+
+
 def test_mfma_takes_views_of_a_packed_qkv_tensor():
     """vLLM hands q, k, v as views of one [T, (Hq + 2 Hkv) D] projection output and writes o into a wider buffer:
     token strides larger than the row, the matrix path must take them as they are."""

@@ -33,7 +33,10 @@ def _draw(seed):
     kernel = r.choice([_ffi.KERNEL_MFMA4, _ffi.KERNEL_MFMA8, _ffi.KERNEL_AUTO])
     dtype = r.choice([torch.bfloat16, torch.bfloat16, torch.float16])
     window = r.choice([0, 0, 7, 50, 300])
-    return dict(dtype=dtype, window=window, hq=hkv * group, hkv=hkv, doc_lens=doc_lens, requests=requests, q_lens=q_lens, variant=variant,
+    d = r.choice([128, 128, 64])
+    if d == 64:
+        window = 0               # the 64-wide matrix kernels are built without the window code
+    return dict(dtype=dtype, window=window, d=d, hq=hkv * group, hkv=hkv, doc_lens=doc_lens, requests=requests, q_lens=q_lens, variant=variant,
                 kv=kv, nsplit=nsplit, kernel=kernel)
 
 
@@ -41,7 +44,7 @@ def _draw(seed):
 def test_random_ragged_batch(seed):
     c = _draw(1000 + seed)
     print(f"case: random batch seed={seed} {c}", flush=True)
-    w = wl.make_workload("rand", dtype=c["dtype"], hq=c["hq"], hkv=c["hkv"], d=128, theta=500000.0, block_size=16,
+    w = wl.make_workload("rand", dtype=c["dtype"], hq=c["hq"], hkv=c["hkv"], d=c["d"], theta=500000.0, block_size=16,
                          doc_lens=c["doc_lens"], requests=c["requests"], q_lens=c["q_lens"], variant=c["variant"],
                          kv_cache_dtype=c["kv"], seed=seed)
     lazy = None
