@@ -861,7 +861,6 @@ bool mfma_supports(const lazyattn_prefill_params &p) {
     if (!(p.cache_dtype == p.dtype || fp8)) return false;
     if (p.table_dtype != p.dtype && p.table_dtype != LAZYATTN_F32) return false;
     if ((p.head_dim != 128 && p.head_dim != 64) || p.rotary_dim != p.head_dim) return false;
-    if (p.head_dim == 64 && p.sliding_window > 0) return false;     // the 64-wide kernels are built without the window code
     if (p.block_size != BS || p.x != (fp8 ? 16 : 8)) return false;
     if (p.q_stride[2] != 1 || p.k_stride[2] != 1 || p.v_stride[2] != 1 || p.o_stride[2] != 1) return false;
     if (p.kc_stride[4] != 1 || p.kc_stride[3] != p.x || p.kc_stride[2] != (int64_t)BS * p.x) return false;
@@ -911,7 +910,9 @@ static int launch_mfma_hd(const lazyattn_prefill_params &p, int nsplit, int n_mt
 }
 template <int NC, typename T>
 static int launch_mfma_nc(const lazyattn_prefill_params &p, int nsplit, int n_mt, hipStream_t stream) {
-    if (p.head_dim == 64) return launch_mfma_hd<NC, 64, false, T>(p, nsplit, n_mt, stream);
+    if (p.head_dim == 64)
+        return p.sliding_window > 0 ? launch_mfma_hd<NC, 64, true, T>(p, nsplit, n_mt, stream)
+                                    : launch_mfma_hd<NC, 64, false, T>(p, nsplit, n_mt, stream);
     if (p.sliding_window > 0) return launch_mfma_hd<NC, 128, true, T>(p, nsplit, n_mt, stream);
     return launch_mfma_hd<NC, 128, false, T>(p, nsplit, n_mt, stream);
 }

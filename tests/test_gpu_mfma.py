@@ -17,8 +17,8 @@ def _err(a, b):
     return (a.float() - b.float()).abs().max().item()
 
 
-def _ragged(variant, kv="auto", seed=31, table_f32=False):
-    w = wl.make_workload("ragged", dtype=torch.bfloat16, **GEOM,
+def _ragged(variant, kv="auto", seed=31, table_f32=False, d=128):
+    w = wl.make_workload("ragged", dtype=torch.bfloat16, **{**GEOM, "d": d},
                          doc_lens=[100, 16, 333, 70, 5, 250], requests=[[3, 1, 0], [2], [0, 2, 3, 1, 5], [4], []],
                          q_lens=[70, 1, 9, 33, 130], variant=variant, kv_cache_dtype=kv, seed=seed)
     if table_f32:
@@ -85,12 +85,12 @@ def test_mfma_float16_operands(variant, kv):
 
 
 @pytest.mark.parametrize("variant", ["natural", "block_uniform"])
-@pytest.mark.parametrize("window", [5, 37, 200, 4096])
-def test_mfma_sliding_window(variant, window):
+@pytest.mark.parametrize("window,d", [(5, 128), (37, 128), (200, 128), (4096, 128), (37, 64), (200, 64)])
+def test_mfma_sliding_window(variant, window, d):
     """Sliding windows shorter than a page, than a tile, of several tiles, and longer than every context
     (old_ops/prefix_prefill.py:270-284, 373-376); the tiles before a workgroup's first window are skipped."""
-    print(f"case: mfma sliding window {window} {variant}", flush=True)
-    w = _ragged(variant)
+    print(f"case: mfma sliding window {window} {variant} head {d}", flush=True)
+    w = _ragged(variant, d=d)
     ref = run_oracle(w, sliding_window=window)
     for nsplit, kernel in ((1, _ffi.KERNEL_MFMA4), (3, _ffi.KERNEL_MFMA8)):
         got = run_op(w.to(DEV), kernel=kernel, num_splits=nsplit, sliding_window=window).cpu()

@@ -34,8 +34,6 @@ def _draw(seed):
     dtype = r.choice([torch.bfloat16, torch.bfloat16, torch.float16])
     window = r.choice([0, 0, 7, 50, 300])
     d = r.choice([128, 128, 64])
-    if d == 64:
-        window = 0               # the 64-wide matrix kernels are built without the window code
     return dict(dtype=dtype, window=window, d=d, hq=hkv * group, hkv=hkv, doc_lens=doc_lens, requests=requests, q_lens=q_lens, variant=variant,
                 kv=kv, nsplit=nsplit, kernel=kernel)
 
