@@ -109,7 +109,7 @@ def test_decode_vanilla_requests_and_fp32_table():
     assert _err(got, ref) < 2e-2, _err(got, ref)
 
 
-@pytest.mark.parametrize("hq,hkv", [(4, 4), (16, 2), (32, 2)])
+@pytest.mark.parametrize("hq,hkv", [(4, 4), (16, 2), (32, 2), (3, 1), (28, 4), (24, 2)])
 def test_decode_group_sizes(hq, hkv):
     print(f"case: decode group {hq // hkv}", flush=True)
     w = _decode_batch("natural", hq=hq, hkv=hkv)

@@ -118,6 +118,38 @@ def test_mfma_without_the_packed_table_and_a_table_of_exact_size(variant, dtype,
         assert e < 2e-2, (nsplit, e)
 
 
+@pytest.mark.parametrize("hq,hkv", [(3, 1), (12, 4), (28, 4), (14, 2), (48, 4)])
+def test_mfma_group_sizes_that_do_not_divide_a_workgroup(hq, hkv):
+    """Query heads per kv head of 3, 7 and 12 (Qwen2-7B has 28/4): a 32-row unit is one (chunk, head) pair and
+    a workgroup's 4 or 8 units straddle chunks."""
+    print(f"case: mfma group {hq}/{hkv}", flush=True)
+    w = wl.make_workload("groups", dtype=torch.bfloat16, hq=hq, hkv=hkv, d=128, theta=500000.0, block_size=16,
+                         doc_lens=[100, 16, 333, 70], requests=[[3, 1, 0], [2], [0, 2, 3, 1]],
+                         q_lens=[70, 33, 130], variant="offset", seed=hq)
+    ref = run_oracle(w)
+    for nsplit, kernel in ((1, _ffi.KERNEL_MFMA4), (3, _ffi.KERNEL_MFMA8), (0, _ffi.KERNEL_AUTO)):
+        got = run_op(w.to(DEV), kernel=kernel, num_splits=nsplit).cpu()
+        e = _err(got, ref)
+        assert e < 2e-2, (nsplit, e)
+
+
+@pytest.mark.parametrize("n_req,hkv", [(257, 1), (67, 8), (130, 2)])
+def test_mfma_many_requests(n_req, hkv):
+    """Hundreds of short requests, in counts that exercise each of the three workgroup-to-XCD mappings; every
+    fifth request has a single new token, every seventh no cached document."""
+    print(f"case: mfma many requests {n_req} x {hkv} kv heads", flush=True)
+    docs = [16, 40, 5, 64, 33]
+    requests = [[] if b % 7 == 0 else [b % 5, (b + 2) % 5][: 1 + b % 2] for b in range(n_req)]
+    q_lens = [1 if b % 5 == 0 else 3 + b % 37 for b in range(n_req)]
+    w = wl.make_workload("many", dtype=torch.bfloat16, hq=2 * hkv, hkv=hkv, d=128, theta=500000.0, block_size=16,
+                         doc_lens=docs, requests=requests, q_lens=q_lens, variant="block_uniform", seed=n_req)
+    ref = run_oracle(w)
+    for nsplit in (0, 2):
+        got = run_op(w.to(DEV), kernel=_ffi.KERNEL_MFMA, num_splits=nsplit).cpu()
+        e = _err(got, ref)
+        assert e < 2e-2, (nsplit, e)
+
+
 def test_mfma_takes_views_of_a_packed_qkv_tensor():
     """vLLM hands q, k, v as views of one [T, (Hq + 2 Hkv) D] projection output and writes o into a wider buffer:
     token strides larger than the row, the matrix path must take them as they are."""
