@@ -888,11 +888,14 @@ template <int NC, int HD, bool FP8, bool WIN, typename T, typename TT>
 static int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt, hipStream_t stream) {
     auto kern = prefill_mfma_kernel<NC, HD, FP8, WIN, T, TT>;
     constexpr int LDS_BYTES = lds_bytes<HD>(NC);
-    static bool attr_set = false;
-    if (!attr_set) {
+    // the attribute belongs to the device's copy of the kernel: once per device, on the caller's current device
+    static bool attr_set[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return LAZYATTN_E_LAUNCH;
+    if (!attr_set[dev]) {
         if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
             return LAZYATTN_E_LAUNCH;
-        attr_set = true;
+        attr_set[dev] = true;
     }
     const unsigned nblocks = (unsigned)(p.batch * p.num_kv_heads * nsplit * n_mt);
     hipLaunchKernelGGL(kern, dim3(nblocks), dim3((NC + 4) * 64), LDS_BYTES, stream, p, nsplit, n_mt);
