@@ -150,6 +150,19 @@ def test_mfma_many_requests(n_req, hkv):
         assert e < 2e-2, (nsplit, e)
 
 
+@pytest.mark.parametrize("kernel", [_ffi.KERNEL_MFMA, _ffi.KERNEL_GENERIC, _ffi.KERNEL_AUTO])
+def test_request_without_new_tokens_is_passed_over(kernel):
+    """b_start_loc may repeat a value: that request has a context but nothing to compute."""
+    print(f"case: zero-length request, kernel {kernel}", flush=True)
+    w = wl.make_workload("zero_len", dtype=torch.bfloat16, **GEOM, doc_lens=[40, 16, 70],
+                         requests=[[0, 1], [2], [1, 2]], q_lens=[33, 0, 5], variant="natural", seed=3)
+    ref = run_oracle(w)
+    for nsplit in (0, 2):
+        got = run_op(w.to(DEV), kernel=kernel, num_splits=nsplit).cpu()
+        e = _err(got, ref)
+        assert e < 2e-2, (nsplit, e)
+
+
 def test_mfma_takes_views_of_a_packed_qkv_tensor():
     """vLLM hands q, k, v as views of one [T, (Hq + 2 Hkv) D] projection output and writes o into a wider buffer:
     token strides larger than the row, the matrix path must take them as they are."""
