@@ -759,7 +759,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     }
 }
 
-// ---- merge split-KV partials: one 32-lane group per (token, q-head) row ----
+// ---- merge split-KV partials: one 16-lane group (head size 128) per (token, q-head) row ----
 // The few fields the merge needs, not the whole parameter block: a launch with ~450 bytes of kernel
 // arguments costs about a microsecond more than one with 64 on this part.
 struct MergeArgs {
@@ -768,11 +768,12 @@ struct MergeArgs {
     int64_t o_stride[2];
     int32_t num_tokens, num_q_heads, index_bits, skip_decode;
 };
-template <typename T, int HD>
+// NB = splits taken per batch of loads: 2, 4 or 8, the smallest that covers nsplit (more only when nsplit > 8)
+template <typename T, int HD, int NB>
 __global__ void __launch_bounds__(256)
 prefill_combine_kernel(const MergeArgs p, const int nsplit) {
     using E = Elem<T>;
-    constexpr int D = HD, LPR = HD / 4;                       // lanes per row (4 elements each)
+    constexpr int D = HD, LPR = HD / 8;                       // lanes per row (8 elements = one 16-byte load each)
     const int b = blockIdx.y;
     const int64_t qs = load_index(p.b_start_loc, b, p.index_bits);
     const int64_t q_len = load_index(p.b_start_loc, b + 1, p.index_bits) - qs;
@@ -781,47 +782,55 @@ prefill_combine_kernel(const MergeArgs p, const int nsplit) {
     if (r >= q_len * p.num_q_heads) return;
     const int64_t tok = qs + r / p.num_q_heads;
     const int h = (int)(r % p.num_q_heads);
-    const int d = (threadIdx.x % LPR) * 4;
+    const int d = (threadIdx.x % LPR) * 8;
     const int64_t NTOK = p.num_tokens;
     const _Float16 *wo = (const _Float16 *)p.workspace;
     const float2 *wl = reinterpret_cast<const float2 *>(wo + (int64_t)nsplit * NTOK * p.num_q_heads * D);
-    // Splits are taken eight at a time, log-sum-exps and partial rows of a batch requested together and
-    // before the first use: one memory round trip per eight splits.  Batches are chained like the
-    // tiles of the main kernel, by a running maximum.
+    // Log-sum-exps and partial rows of a batch of splits are requested together and before the first use:
+    // one memory round trip per batch.  Batches are chained like the tiles of the main kernel, by a running
+    // maximum.
     const int64_t row0 = tok * p.num_q_heads + h, split_rows = NTOK * p.num_q_heads;
     float mx = -INFINITY, wsum = 0.f;
-    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int s0 = 0; s0 < nsplit; s0 += 8) {
-        float2 e[8];                                         // (log2-sum-exp, scale of the row's halves)
-        uint2 v[8];
+    float o[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+    for (int i = 0; i < 8; ++i) o[i] = 0.f;
+    for (int s0 = 0; s0 < nsplit; s0 += NB) {
+        float2 e[NB];                                        // (log2-sum-exp, scale of the row's halves)
+        uint4 v[NB];
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
             const int64_t ri = (int64_t)(s0 + j < nsplit ? s0 + j : nsplit - 1) * split_rows + row0;
             e[j] = wl[ri];
-            v[j] = *reinterpret_cast<const uint2 *>(wo + ri * D + d);
+            v[j] = *reinterpret_cast<const uint4 *>(wo + ri * D + d);
         }
         float bm = e[0].x;
 #pragma unroll
-        for (int j = 1; j < 8; ++j) bm = fmaxf(bm, e[j].x);
+        for (int j = 1; j < NB; ++j) bm = fmaxf(bm, e[j].x);
         const float m_new = fmaxf(mx, bm);
         if (m_new == -INFINITY) continue;                    // nothing visible so far
         const float keep = __builtin_amdgcn_exp2f(mx - m_new);   // mx = -inf -> 0
-        o.x *= keep; o.y *= keep; o.z *= keep; o.w *= keep;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] *= keep;
         wsum *= keep;
         mx = m_new;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < NB; ++j) {
             const float w = s0 + j < nsplit ? __builtin_amdgcn_exp2f(e[j].x - mx) : 0.f;
             const float ws = w * e[j].y;
-            const f16x2_t lo = *reinterpret_cast<const f16x2_t *>(&v[j].x), hi = *reinterpret_cast<const f16x2_t *>(&v[j].y);
-            o.x = fmaf(ws, (float)lo[0], o.x); o.y = fmaf(ws, (float)lo[1], o.y);
-            o.z = fmaf(ws, (float)hi[0], o.z); o.w = fmaf(ws, (float)hi[1], o.w);
+            const uint32_t u[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const f16x2_t hh = *reinterpret_cast<const f16x2_t *>(&u[i]);
+                o[2 * i] = fmaf(ws, (float)hh[0], o[2 * i]);
+                o[2 * i + 1] = fmaf(ws, (float)hh[1], o[2 * i + 1]);
+            }
             wsum += w;
         }
     }
     const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
     T *op = (T *)p.o + tok * p.o_stride[0] + (int64_t)h * p.o_stride[1] + d;
-    *reinterpret_cast<uint2 *>(op) = make_uint2(E::pack(o.x * inv, o.y * inv), E::pack(o.z * inv, o.w * inv));
+    *reinterpret_cast<uint4 *>(op) = make_uint4(E::pack(o[0] * inv, o[1] * inv), E::pack(o[2] * inv, o[3] * inv),
+                                                E::pack(o[4] * inv, o[5] * inv), E::pack(o[6] * inv, o[7] * inv));
 }
 
 // ------------------------------------------------------------------ host side
@@ -940,16 +949,20 @@ int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
         const int64_t rows = (int64_t)p.max_q_len * p.num_q_heads;
         const MergeArgs m{p.workspace, p.b_start_loc, p.o, {p.o_stride[0], p.o_stride[1]}, p.num_tokens, p.num_q_heads,
                           p.index_bits, p.skip_decode};
-        const int rows_wg = 256 / (p.head_dim / 4);
+        const int rows_wg = 256 / (p.head_dim / 8);
         const dim3 grid((unsigned)((rows + rows_wg - 1) / rows_wg), p.batch);
         const bool f16 = p.dtype == LAZYATTN_F16;
+#define LAZYATTN_COMBINE(HD, NB)                                                                              \
+    {                                                                                                         \
+        if (f16) hipLaunchKernelGGL((prefill_combine_kernel<f16_t, HD, NB>), grid, dim3(256), 0, stream, m, nsplit); \
+        else hipLaunchKernelGGL((prefill_combine_kernel<bf16_t, HD, NB>), grid, dim3(256), 0, stream, m, nsplit);    \
+    }
         if (p.head_dim == 64) {
-            if (f16) hipLaunchKernelGGL((prefill_combine_kernel<f16_t, 64>), grid, dim3(256), 0, stream, m, nsplit);
-            else hipLaunchKernelGGL((prefill_combine_kernel<bf16_t, 64>), grid, dim3(256), 0, stream, m, nsplit);
+            if (nsplit <= 2) LAZYATTN_COMBINE(64, 2) else if (nsplit <= 4) LAZYATTN_COMBINE(64, 4) else LAZYATTN_COMBINE(64, 8)
         } else {
-            if (f16) hipLaunchKernelGGL((prefill_combine_kernel<f16_t, 128>), grid, dim3(256), 0, stream, m, nsplit);
-            else hipLaunchKernelGGL((prefill_combine_kernel<bf16_t, 128>), grid, dim3(256), 0, stream, m, nsplit);
+            if (nsplit <= 2) LAZYATTN_COMBINE(128, 2) else if (nsplit <= 4) LAZYATTN_COMBINE(128, 4) else LAZYATTN_COMBINE(128, 8)
         }
+#undef LAZYATTN_COMBINE
         if (hipGetLastError() != hipSuccess) return LAZYATTN_E_LAUNCH;
     }
     return LAZYATTN_OK;
