@@ -30,7 +30,8 @@ def _decode_batch(variant, *, hq=8, hkv=2, q_lens=(1, 1, 1, 1, 1), table_f32=Fal
     fp8 = "fp8" in kv
 
     def to_cache(t, scale):
-        return (t.float() / scale).to(torch.float8_e4m3fn).view(torch.uint8) if fp8 else t
+        # a cache write saturates: a new token may exceed the range the scale was chosen for
+        return (t.float() / scale).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8) if fp8 else t
     for b in range(len(q_lens)):
         qs, qe = int(w.b_start_loc[b]), int(w.b_start_loc[b + 1])
         ctx = int(w.b_seq_len[b]) - (qe - qs)

@@ -3,6 +3,7 @@ composition, new-token counts, GQA group, split count, position mode and cache t
 seeded generator (the reference's own tests sweep fixed grids, tests/kernels/test_prefix_prefill.py:27-60;
 the draws here reach the corners in between: documents shorter than a page, requests with no context,
 one-token requests next to long ones, tiles that end inside a page)."""
+import os
 import random
 
 import pytest
@@ -13,6 +14,16 @@ from opcall import run_op, run_oracle
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
+# LAZYATTN_RANDOM_CASES=N widens both sweeps to N draws (the default keeps the suite short)
+N_PREFILL = int(os.environ.get("LAZYATTN_RANDOM_CASES", 64))
+N_DECODE = int(os.environ.get("LAZYATTN_RANDOM_CASES", 24))
+
+
+def _excess(got, ref, dtype):
+    """Largest |got - ref| beyond one unit in the last place of ref: both are rounded to the operand type, and
+    a row that sees a handful of keys can have outputs above 4, where one bf16 step is 2^-5."""
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    return ((got.float() - ref.float()).abs() - ulp * ref.float().abs()).clamp(min=0).max().item()
 
 
 def _draw(seed):
@@ -38,7 +49,7 @@ def _draw(seed):
                 kv=kv, nsplit=nsplit, kernel=kernel)
 
 
-@pytest.mark.parametrize("seed", range(64))
+@pytest.mark.parametrize("seed", range(N_PREFILL))
 def test_random_ragged_batch(seed):
     c = _draw(1000 + seed)
     print(f"case: random batch seed={seed} {c}", flush=True)
@@ -52,11 +63,11 @@ def test_random_ragged_batch(seed):
     got = run_op(w.to(DEV), kernel=c["kernel"], num_splits=c["nsplit"], sliding_window=c["window"] or None,
                  is_lazy=None if lazy is None else lazy.to(DEV)).cpu()
     assert torch.isfinite(got.float()).all()
-    err = (got.float() - ref.float()).abs().max().item()
+    err = _excess(got, ref, c["dtype"])
     assert err < (5e-2 if c["kv"] == "fp8" else 2e-2 if c["dtype"] == torch.bfloat16 else 5e-3), err
 
 
-@pytest.mark.parametrize("seed", range(24))
+@pytest.mark.parametrize("seed", range(N_DECODE))
 def test_random_decode_batch(seed):
     """The q_len == 1 rows through the decode launch: every key, the new token included, sits in the paged
     cache when the call is made; requests with more than one new token must be left alone."""
