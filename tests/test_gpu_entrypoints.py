@@ -71,3 +71,49 @@ def test_entry_block_uniform_mixed_batch_with_packed_table(dtype, d, tol):
                         q_mask=None, packed_block_table=packed)
     err = (out.cpu().float() - ref.float()).abs().max().item()
     assert err < tol, err
+
+
+@pytest.mark.parametrize("block_size", [32, 16])
+@pytest.mark.parametrize("head_size", [128, 96, 24])
+@pytest.mark.parametrize("queries_per_kv", [1, 8, 64])
+def test_reference_kernel_test_grid(head_size, queries_per_kv, block_size):
+    """The grid of the reference's own kernel test (tests/kernels/test_prefix_prefill.py:37-48, 85-93, with
+    vLLM's NUM_HEADS = 64, NUM_QUERIES_PER_KV = 1 / 8 / 64, HEAD_SIZES = 128 / 96 / 24, float16, pages of 32
+    tokens, ten requests the last of which has one new token), lengths cut so that the CPU oracle takes
+    well under a second, through both entry points of the un-rotated-cache variant; pages of 16 added."""
+    import random
+    from lazy_amd.attention.old_ops.prefix_prefill import context_attention_fwd
+    print(f"case: reference grid head {head_size} group {queries_per_kv} page {block_size}", flush=True)
+    r = random.Random(0)
+    q_lens = [r.randint(16, 128) for _ in range(10)]
+    q_lens[-1] = 1
+    docs = [r.randint(16, 256) for _ in range(10)]
+    d, hkv = head_size, 64 // queries_per_kv
+    w = wl.make_workload("refgrid", dtype=torch.float16, hq=64, hkv=hkv, d=d, theta=10000.0, block_size=block_size,
+                         doc_lens=docs, requests=[[i] for i in range(10)], q_lens=q_lens, variant="natural", seed=0)
+    # the decode request's token is in the cache when the backend calls (backends/triton_attn.py:100-109)
+    x = w.k_cache.shape[4]
+    qs = int(w.b_start_loc[9]); n = int(w.b_seq_len[9]) - 1
+    pb = int(w.block_table[9, n // block_size]); o_ = n % block_size
+    w.k_cache[pb, :, :, o_, :] = w.k[qs].view(hkv, d // x, x)
+    w.v_cache[pb, :, :, o_] = w.v[qs]
+    prefill_only = torch.full_like(w.q, 5.0)
+    orc.prefix_prefill(w.q, w.k, w.v, w.k_cache, w.v_cache, w.block_table, w.b_start_loc, w.b_seq_len,
+                       w.cos_sin_cache, w.q_offset, w.q_mask, pos_mode=w.pos_mode, rotate_new_k=w.rotate_new_k,
+                       out=prefill_only)
+    both = _expected(w)
+    g = w.to(DEV)
+    out = torch.full_like(g.q, 5.0)
+    context_attention_fwd(g.q, g.k, g.v, out, "auto", g.k_cache, g.v_cache, g.block_table, g.b_start_loc, g.b_seq_len,
+                          g.max_seq_len, g.max_query_len, g.k_scale, g.v_scale, rotary_dim=d,
+                          cos_sin_cache=g.cos_sin_cache, q_mask=g.q_mask)
+    err = (out.cpu().float() - prefill_only.float()).abs().max().item()
+    assert err < 5e-3, err
+    # the scale is passed, as the backend does: this entry point's default is 1/sqrt(number of heads), like the
+    # reference's (old_ops/chunked_prefill_paged_decode.py:311-312)
+    out = torch.full_like(g.q, 5.0)
+    entry_unrotated(g.q, g.k, g.v, out, "auto", g.k_cache, g.v_cache, g.block_table, g.b_start_loc, g.b_seq_len,
+                    g.max_seq_len, g.max_query_len, g.k_scale, g.v_scale, sm_scale=d ** -0.5, rotary_dim=d,
+                    cos_sin_cache=g.cos_sin_cache, q_mask=g.q_mask)
+    err = (out.cpu().float() - both.float()).abs().max().item()
+    assert err < 5e-3, err
