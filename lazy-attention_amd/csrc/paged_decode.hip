@@ -135,31 +135,37 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     const float k_scale = FP8 ? *p.k_scale : 1.f, v_scale = FP8 ? *p.v_scale : 1.f;
     const uint8_t *tab = (const uint8_t *)p.cos_sin_cache;
     const int64_t row_bytes = p.table_stride * TSZ;
-    // bf16: chunk 4 m + grp of token t at (4 m + grp) * 256 + t * 16, 16 bytes
-    // fp8 : the same 8 d are half (grp & 1) of 16-d chunk 2 m + grp / 2: (2 m + grp / 2) * 256 + t * 16 + (grp & 1) * 8
-    const uint32_t k_off = FP8 ? (uint32_t)((grp >> 1) * 256 + t * 16 + (grp & 1) * 8) : (uint32_t)(grp * 256 + t * 16);
-    constexpr uint32_t K_STEP = FP8 ? 512 : 1024;                // per m
+    // A cache page of 32 slots is read as two parts of 16: "page" j below is the j-th run of 16 slots of the
+    // sequence, part j & 1 of cache page j >> 1 (pshift = 1); with pages of 16 slots the two coincide.
+    const int pshift = p.block_size == 2 * BS ? 1 : 0;
+    const int cache_bs = BS << pshift;
+    // bf16: chunk 4 m + grp of token t at ((4 m + grp) * slots + t) * 16, 16 bytes
+    // fp8 : the same 8 d are half (grp & 1) of 16-d chunk 2 m + grp / 2: ((2 m + grp / 2) * slots + t) * 16 + (grp & 1) * 8
+    const uint32_t k_off = FP8 ? (uint32_t)(((grp >> 1) * cache_bs + t) * 16 + (grp & 1) * 8) : (uint32_t)((grp * cache_bs + t) * 16);
+    const uint32_t K_STEP = (FP8 ? 512u : 1024u) << pshift;      // per m
     // V[d = 16 blk + t][tokens 4 grp ..]: 8 bytes (bf16) or 4 bytes (fp8) of the row
-    const uint32_t v_off = FP8 ? (uint32_t)(t * 16 + grp * 4) : (uint32_t)(t * 32 + grp * 8);
-    constexpr uint32_t V_STEP = FP8 ? 256 : 512;                 // per blk
+    const uint32_t v_off = FP8 ? (uint32_t)(t * cache_bs + grp * 4) : (uint32_t)(t * cache_bs * 2 + grp * 8);
+    const uint32_t V_STEP = (FP8 ? 256u : 512u) << pshift;       // per blk
 
     auto page_block = [&](int j) -> int {
         int jc = j < n_pages ? j : n_pages - 1;
         jc = jc < 0 ? 0 : jc;
-        return bt_row[jc * bt_s1];
+        return bt_row[(jc >> pshift) * bt_s1];
     };
     auto load_keys = [&](int j, KeyRegs<TT, HD> &r) {
         int jc = j < n_pages ? j : n_pages - 1;
         jc = jc < 0 ? 0 : jc;
-        const int bt = bt_row[jc * bt_s1];
-        const int qo = qo_row[jc * qo_s1] & qo_and;
-        const int qm = qm_row[jc * qm_s1] & qm_and;                                  // old_ops/chunked...:165-167 analogue
+        const int pj = jc >> pshift, part = jc & pshift;
+        const int bt = bt_row[pj * bt_s1];
+        const int qo = qo_row[pj * qo_s1] & qo_and;
+        const int qm = qm_row[pj * qm_s1] & qm_and;                                  // old_ops/chunked...:165-167 analogue
+        const int ql = cache_bs - qm - (j & pshift) * BS;                            // valid slots of this part
         int l = seq_len - j * BS;
-        l = l < BS - qm ? l : BS - qm;
+        l = l < ql ? l : ql;
         l = l > BS ? BS : l;
         r.lim = l < 0 ? 0 : l;
         r.first = first_key - j * BS;                                                // slots below it lie before the window
-        const uint8_t *kb = kc_base + bt * kc_page_bytes;
+        const uint8_t *kb = kc_base + bt * kc_page_bytes + part * (BS * 16);
 #pragma unroll
         for (int m = 0; m < NM; ++m) {
             if (FP8) {
@@ -185,7 +191,9 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
         }
     };
     auto load_values = [&](int j, ValRegs<HD> &r) {
-        const uint8_t *vb = vc_base + page_block(j) * vc_page_bytes;
+        int jv = j < n_pages ? j : n_pages - 1;
+        jv = jv < 0 ? 0 : jv;
+        const uint8_t *vb = vc_base + page_block(j) * vc_page_bytes + (jv & pshift) * (BS * CSZ);
 #pragma unroll
         for (int blk = 0; blk < NBLK; ++blk) {
             if (FP8) r.v[blk] = make_uint2(*reinterpret_cast<const uint32_t *>(vb + v_off + blk * V_STEP), 0);
@@ -396,12 +404,12 @@ bool decode_mfma_supports(const lazyattn_prefill_params &p) {
     if ((p.dtype != LAZYATTN_BF16 && p.dtype != LAZYATTN_F16) || !(p.cache_dtype == p.dtype || fp8)) return false;
     if (p.table_dtype != p.dtype && p.table_dtype != LAZYATTN_F32) return false;
     if ((p.head_dim != 128 && p.head_dim != 64) || p.rotary_dim != p.head_dim) return false;
-    if (p.block_size != BS || p.x != (fp8 ? 16 : 8)) return false;
+    if ((p.block_size != BS && p.block_size != 2 * BS) || p.x != (fp8 ? 16 : 8)) return false;
     if (p.pos_mode != LAZYATTN_POS_NATURAL && p.pos_mode != LAZYATTN_POS_BLOCK_UNIFORM) return false;
     if (p.num_q_heads / p.num_kv_heads > 16) return false;
     if (p.q_stride[2] != 1 || p.o_stride[2] != 1) return false;
-    if (p.kc_stride[4] != 1 || p.kc_stride[3] != p.x || p.kc_stride[2] != (int64_t)BS * p.x) return false;
-    if (p.vc_stride[3] != 1 || p.vc_stride[2] != BS) return false;
+    if (p.kc_stride[4] != 1 || p.kc_stride[3] != p.x || p.kc_stride[2] != (int64_t)p.block_size * p.x) return false;
+    if (p.vc_stride[3] != 1 || p.vc_stride[2] != p.block_size) return false;
     const int64_t al[] = {p.q_stride[0], p.q_stride[1], p.o_stride[0], p.o_stride[1], p.kc_stride[0], p.kc_stride[1],
                           p.vc_stride[0], p.vc_stride[1], p.table_stride};
     for (int64_t s : al)

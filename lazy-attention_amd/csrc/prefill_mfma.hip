@@ -238,15 +238,21 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     const int64_t qo_s1 = use_qo ? p.qo_stride[1] : p.bt_stride[1];
     const int64_t qm_s1 = use_qmask ? p.qm_stride[1] : p.bt_stride[1];
     const int qo_and = use_qo ? -1 : 0, qm_and = use_qmask ? -1 : 0;
+    // A cache page of 32 slots is handled as two parts of 16: "page" j below is the j-th run of 16 context
+    // slots, part j & 1 of cache page j >> 1.  Its valid slots follow from the page's pad count.
+    const int pshift = p.block_size == 2 * BS ? 1 : 0, part_mask = pshift;
+    const int cache_bs = BS << pshift;
     auto load_page = [&](int j) -> PageMeta {
         PageMeta m;
         int jc = j < n_pages ? j : n_pages - 1;
         jc = jc < 0 ? 0 : jc;
-        m.bt = bt_row[jc * bt_s1];
-        m.qo = qo_row[jc * qo_s1] & qo_and;
-        const int qm = qm_row[jc * qm_s1] & qm_and;                                  // old_ops:165-167
+        const int pj = jc >> pshift;
+        m.bt = bt_row[pj * bt_s1];
+        m.qo = qo_row[pj * qo_s1] & qo_and;
+        const int qm = qm_row[pj * qm_s1] & qm_and;                                  // old_ops:165-167
+        const int ql = cache_bs - qm - (j & part_mask) * BS;                         // valid slots of this part
         int l = ctx_len - j * BS;
-        l = l < BS - qm ? l : BS - qm;
+        l = l < ql ? l : ql;
         l = l > BS ? BS : l;
         m.lim = l < 0 ? 0 : l;
         return m;
@@ -275,15 +281,29 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         const uint8_t *ctab_base = packed_tab ? (const uint8_t *)p.cos_sin_packed : tab_base;
         const uint32_t pos_bytes = packed_tab ? 8 * TSZ : row_bytes;       // bytes per unit of position
         const uint32_t sin_delta = packed_tab ? (uint32_t)(HALF / 8) * (uint32_t)p.packed_rows * 8 * TSZ : HALF * TSZ;
+        // this wave's part of its cache pages (pages of 32 slots: the tile's pages 0, 1 are the two parts of
+        // one cache page, 2, 3 of the next): first slot, and the position step that goes with it
+        const int slot0 = (gw & part_mask) * BS;
+        const int part_pos = nat_step ? slot0 : 0;               // block-uniform: one position for the whole page
         // K items of a page: 128 = (8 chunks of 8 (d, d+64) pairs) x 16 slots, two per lane
-        uint32_t k_goff[KI], k_toff[KI];
+        uint32_t k_toff[KI];
+        // Cache offsets of a lane's items: item i = item 0 + i * (a wave-uniform stride), so one offset register
+        // serves all of them and the strides go into the scalar page base.
+        // K bf16: [D/8][slots][8] -> item (cp, o) at (cp*slots + o)*16 bytes, cp = lane/16 + 4 i
+        //   fp8 : [D/16][slots][16] -> 8 bytes at chunk cp/2, half cp&1
+        // V bf16: row d = lane/2 + 32 i of `slots` slots, 8 slots (16 bytes) per item; fp8: row d = lane + 64 i, 16 slots
+        const uint32_t k_goff = FP8 ? (uint32_t)(((lane >> 5) * cache_bs + slot0 + (lane & 15)) * 16 + ((lane >> 4) & 1) * 8)
+                                    : (uint32_t)(((lane >> 4) * cache_bs + slot0 + (lane & 15)) * 16);
+        const uint32_t k_item = (uint32_t)((FP8 ? 2 : 4) * cache_bs * 16);
+        const uint32_t v_goff = FP8 ? (uint32_t)(lane * cache_bs + slot0)
+                                    : (uint32_t)((lane >> 1) * cache_bs * 2 + slot0 * 2 + (lane & 1) * 16);
+        const uint32_t v_item = (uint32_t)(64 * cache_bs);
+        // bytes from the chunk of d to the chunk of d + HD/2 in the cache page
+        const uint32_t pair = (uint32_t)(FP8 ? G::PAIR8 : G::PAIR) << pshift;
 #pragma unroll
         for (int i = 0; i < KI; ++i) {
             const int idx = lane + i * 64;
             const int o = idx & 15, cp = idx >> 4;
-            // bf16: [D/8][16][8] -> item (cp, o) at (cp*16 + o)*16 bytes, pair chunk +2048
-            // fp8 : [D/16][16][16] -> 8 bytes at chunk cp/2, half cp&1, pair chunk +4*256
-            k_goff[i] = FP8 ? (uint32_t)((cp >> 1) * 256 + o * 16 + (cp & 1) * 8) : (uint32_t)(idx * 16);
             // block-uniform rotation and un-rotated requests use one table row for the whole page
             k_toff[i] = packed_tab ? ((uint32_t)cp * (uint32_t)p.packed_rows + (uint32_t)o) * 8 * TSZ
                                    : (per_token ? (uint32_t)o * row_bytes : 0u) + (uint32_t)cp * 8 * TSZ;
@@ -302,25 +322,25 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             // A page past the context (its slots are all masked) takes the last page's position: the
             // table only has to cover the positions of real keys.
             const int jp = j < n_pages ? j : n_pages - 1;
-            const int pos0 = pm.qo ? pm.qo - 1 : jp * nat_step;
+            const int pos0 = pm.qo ? pm.qo - 1 + part_pos : jp * nat_step;
             const uint8_t *tb = ctab_base + (int64_t)pos0 * pos_bytes;
 #pragma unroll
             for (int i = 0; i < KI; ++i) {
                 kr[i].lds_off = (uint32_t)(gw * K_PAGE + (lane + i * 64) * 16);
                 if (FP8) {
-                    const uint2 a = ldg8(kb, k_goff[i]), a2 = ldg8(kb, k_goff[i] + G::PAIR8);
+                    const uint2 a = ldg8(kb + i * k_item, k_goff), a2 = ldg8(kb + i * k_item + pair, k_goff);
                     kr[i].k1 = make_uint4(a.x, a.y, 0, 0);
                     kr[i].k2 = make_uint4(a2.x, a2.y, 0, 0);
                 } else {
-                    kr[i].k1 = ldg16(kb, k_goff[i]);
-                    kr[i].k2 = ldg16(kb, k_goff[i] + G::PAIR);
+                    kr[i].k1 = ldg16(kb + i * k_item, k_goff);
+                    kr[i].k2 = ldg16(kb + i * k_item + pair, k_goff);
                 }
                 kr[i].c.load(tb, k_toff[i]);
                 kr[i].s.load(tb, k_toff[i] + sin_delta);
             }
             const uint8_t *vb = vc_base + pm.bt * vc_page_bytes;
 #pragma unroll
-            for (int i = 0; i < VI_CTX; ++i) vr[i] = ldg16(vb, (uint32_t)((lane + i * 64) * 16));
+            for (int i = 0; i < VI_CTX; ++i) vr[i] = ldg16(vb + i * v_item, v_goff);
         };
         // ---- loads of this wave's 16 keys of a new-token tile ----
         auto issue_loads_new = [&](int tile) {
@@ -870,10 +890,10 @@ bool mfma_supports(const lazyattn_prefill_params &p) {
     if (!(p.cache_dtype == p.dtype || fp8)) return false;
     if (p.table_dtype != p.dtype && p.table_dtype != LAZYATTN_F32) return false;
     if ((p.head_dim != 128 && p.head_dim != 64) || p.rotary_dim != p.head_dim) return false;
-    if (p.block_size != BS || p.x != (fp8 ? 16 : 8)) return false;
+    if ((p.block_size != BS && p.block_size != 2 * BS) || p.x != (fp8 ? 16 : 8)) return false;
     if (p.q_stride[2] != 1 || p.k_stride[2] != 1 || p.v_stride[2] != 1 || p.o_stride[2] != 1) return false;
-    if (p.kc_stride[4] != 1 || p.kc_stride[3] != p.x || p.kc_stride[2] != (int64_t)BS * p.x) return false;
-    if (p.vc_stride[3] != 1 || p.vc_stride[2] != BS) return false;
+    if (p.kc_stride[4] != 1 || p.kc_stride[3] != p.x || p.kc_stride[2] != (int64_t)p.block_size * p.x) return false;
+    if (p.vc_stride[3] != 1 || p.vc_stride[2] != p.block_size) return false;
     const int64_t al[] = {p.q_stride[0], p.q_stride[1], p.k_stride[0], p.k_stride[1], p.v_stride[0], p.v_stride[1],
                           p.o_stride[0], p.o_stride[1], p.kc_stride[0], p.kc_stride[1], p.vc_stride[0], p.vc_stride[1],
                           p.table_stride};

@@ -17,10 +17,10 @@ DEV = "cuda"
 
 
 def _decode_batch(variant, *, hq=8, hkv=2, q_lens=(1, 1, 1, 1, 1), table_f32=False, seed=77, kv="auto",
-                  dtype=torch.bfloat16, d=128):
+                  dtype=torch.bfloat16, d=128, bs=16):
     """Ragged documents (pads at document ends), requests of 1 to 9 documents, one new token each
     (or more: such requests must be skipped)."""
-    w = wl.make_workload("decode", dtype=dtype, hq=hq, hkv=hkv, d=d, theta=500000.0, block_size=16,
+    w = wl.make_workload("decode", dtype=dtype, hq=hq, hkv=hkv, d=d, theta=500000.0, block_size=bs,
                          doc_lens=[40, 16, 33, 70, 5, 128, 97],
                          requests=[[3, 1, 0], [2], [0, 2, 3, 1, 5, 6, 4, 5, 6], [4, 0], [6, 5, 3]],
                          q_lens=list(q_lens), variant=variant, seed=seed, kv_cache_dtype=kv)
@@ -37,7 +37,7 @@ def _decode_batch(variant, *, hq=8, hkv=2, q_lens=(1, 1, 1, 1, 1), table_f32=Fal
         ctx = int(w.b_seq_len[b]) - (qe - qs)
         for t in range(qe - qs):
             n = ctx + t
-            pb = int(w.block_table[b, n // 16]); o_ = n % 16
+            pb = int(w.block_table[b, n // bs]); o_ = n % bs
             w.k_cache[pb, :, :, o_, :] = to_cache(w.k[qs + t], w.k_scale).view(hkv, d // x, x)
             w.v_cache[pb, :, :, o_] = to_cache(w.v[qs + t], w.v_scale)
     return w
@@ -117,6 +117,23 @@ def test_decode_group_sizes(hq, hkv):
     ref = _oracle(w)
     got = _run(w)
     assert _err(got, ref) < 2e-2, _err(got, ref)
+
+
+@pytest.mark.parametrize("variant", ["natural", "block_uniform"])
+@pytest.mark.parametrize("dtype,kv,d", [(torch.bfloat16, "auto", 128), (torch.float16, "fp8", 128), (torch.bfloat16, "auto", 64)])
+def test_decode_pages_of_32_slots(variant, dtype, kv, d):
+    """Cache pages of 32 slots (the page size of the reference's kernel test, tests/kernels/test_prefix_prefill.py:86):
+    read as two parts of 16; pads at the end of a document span parts."""
+    print(f"case: decode pages of 32 {variant} {dtype} kv={kv} d={d}", flush=True)
+    w = _decode_batch(variant, dtype=dtype, kv=kv, d=d, bs=32)
+    lazy = torch.tensor([True, False, True, True, True]) if variant == "block_uniform" else None
+    ref = _oracle(w, lazy)
+    for nsplit in (0, 1, 3):
+        got = _run(w, lazy=lazy, num_splits=nsplit, kernel=_ffi.KERNEL_MFMA)
+        assert _err(got, ref) < (5e-2 if kv == "fp8" else 2e-2), (nsplit, _err(got, ref))
+    ref = _oracle(w, lazy, sliding_window=20)
+    got = _run(w, lazy=lazy, sliding_window=20, kernel=_ffi.KERNEL_MFMA)
+    assert _err(got, ref) < (5e-2 if kv == "fp8" else 2e-2), _err(got, ref)
 
 
 @pytest.mark.parametrize("variant,table_f32", [("natural", False), ("block_uniform", True)])

@@ -163,6 +163,24 @@ def test_request_without_new_tokens_is_passed_over(kernel):
         assert e < 2e-2, (nsplit, e)
 
 
+@pytest.mark.parametrize("variant", ["natural", "offset", "block_uniform"])
+@pytest.mark.parametrize("dtype,kv,d", [(torch.bfloat16, "auto", 128), (torch.float16, "fp8", 128), (torch.bfloat16, "auto", 64)])
+def test_mfma_pages_of_32_slots(variant, dtype, kv, d):
+    """Cache pages of 32 slots (the page size of the reference's kernel test, tests/kernels/test_prefix_prefill.py:86):
+    the gather reads them as two parts of 16; document pads span parts and q_offset counts from the page's first slot."""
+    print(f"case: mfma pages of 32 {variant} {dtype} kv={kv} d={d}", flush=True)
+    w = wl.make_workload("page32", dtype=dtype, hq=32, hkv=8, d=d, theta=500000.0, block_size=32,
+                         doc_lens=[100, 16, 333, 70, 5, 250, 47], requests=[[3, 1, 0], [2], [0, 2, 3, 1, 5], [4, 6], []],
+                         q_lens=[70, 1, 9, 33, 130], variant=variant, kv_cache_dtype=kv, seed=32)
+    tol = 5e-2 if kv == "fp8" else 2e-2
+    for window in (0, 50):
+        ref = run_oracle(w, sliding_window=window)
+        for nsplit, kernel in ((1, _ffi.KERNEL_MFMA4), (3, _ffi.KERNEL_MFMA8)):
+            got = run_op(w.to(DEV), kernel=kernel, num_splits=nsplit, sliding_window=window or None).cpu()
+            e = _err(got, ref)
+            assert e < tol, (window, nsplit, e)
+
+
 def test_mfma_takes_views_of_a_packed_qkv_tensor():
     """vLLM hands q, k, v as views of one [T, (Hq + 2 Hkv) D] projection output and writes o into a wider buffer:
     token strides larger than the row, the matrix path must take them as they are."""

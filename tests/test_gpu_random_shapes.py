@@ -45,7 +45,8 @@ def _draw(seed):
     dtype = r.choice([torch.bfloat16, torch.bfloat16, torch.float16])
     window = r.choice([0, 0, 7, 50, 300])
     d = r.choice([128, 128, 64])
-    return dict(dtype=dtype, window=window, d=d, hq=hkv * group, hkv=hkv, doc_lens=doc_lens, requests=requests, q_lens=q_lens, variant=variant,
+    page = r.choice([16, 16, 32])
+    return dict(page=page, dtype=dtype, window=window, d=d, hq=hkv * group, hkv=hkv, doc_lens=doc_lens, requests=requests, q_lens=q_lens, variant=variant,
                 kv=kv, nsplit=nsplit, kernel=kernel)
 
 
@@ -53,7 +54,7 @@ def _draw(seed):
 def test_random_ragged_batch(seed):
     c = _draw(1000 + seed)
     print(f"case: random batch seed={seed} {c}", flush=True)
-    w = wl.make_workload("rand", dtype=c["dtype"], hq=c["hq"], hkv=c["hkv"], d=c["d"], theta=500000.0, block_size=16,
+    w = wl.make_workload("rand", dtype=c["dtype"], hq=c["hq"], hkv=c["hkv"], d=c["d"], theta=500000.0, block_size=c["page"],
                          doc_lens=c["doc_lens"], requests=c["requests"], q_lens=c["q_lens"], variant=c["variant"],
                          kv_cache_dtype=c["kv"], seed=seed)
     lazy = None
@@ -80,9 +81,10 @@ def test_random_decode_batch(seed):
     kv = r.choice(["auto", "auto", "fp8"])
     q_lens = tuple(r.choice([1, 1, 1, 3]) for _ in range(5))
     nsplit = r.choice([0, 1, 2, 5, 9])
-    print(f"case: random decode seed={seed} hkv={hkv} group={group} {variant} kv={kv} q_lens={q_lens} nsplit={nsplit}",
-          flush=True)
-    w = dec._decode_batch(variant, hq=hkv * group, hkv=hkv, q_lens=q_lens, seed=seed, kv=kv)
+    page = r.choice([16, 16, 32])
+    print(f"case: random decode seed={seed} hkv={hkv} group={group} {variant} kv={kv} q_lens={q_lens} nsplit={nsplit} "
+          f"page={page}", flush=True)
+    w = dec._decode_batch(variant, hq=hkv * group, hkv=hkv, q_lens=q_lens, seed=seed, kv=kv, bs=page)
     lazy = torch.tensor([(seed + b) % 4 != 0 for b in range(5)]) if variant == "block_uniform" else None
     ref = dec._oracle(w, lazy)
     got = dec._run(w, lazy=lazy, num_splits=nsplit)
