@@ -35,9 +35,9 @@ __device__ __forceinline__ uint8_t to_fp8_e4m3(float x, float inv_scale) {
 //   [.., + Hkv * C)        k chunk pairs: rotate (optional) + cache write of both chunks
 //   [.., + Hkv * P)        k pass-through chunks (head_dim > rotary_dim): cache write only
 // then, per run of RUN = 16 consecutive tokens: Hkv * D items, one (head, d) each, that move the
-// run's V column.  The V cache keeps the token axis innermost; when the run fills one page in order
-// (the usual case: a prefill chunk is written page by page) the column is one 32-byte store and a
-// wave writes 2 KB contiguously, otherwise the item falls back to one store per token.
+// run's V column.  The V cache keeps the token axis innermost; when the run fills 16 aligned slots of one
+// page in order (the usual case: a prefill chunk is written page by page; pages of 16, 32, ... slots) the
+// column is one 32-byte store, otherwise the item falls back to one store per token.
 constexpr int RUN = 16;
 template <typename T, typename TT, bool FP8>
 __global__ void __launch_bounds__(256)
@@ -67,12 +67,13 @@ rope_cache_write_kernel(const lazyattn_rope_write_params p) {
         const float v_inv = FP8 ? 1.f / *p.v_scale : 1.f;
         const T *src = (const T *)p.v + t0 * p.v_stride[0] + (int64_t)h * p.v_stride[1] + d;
         const int64_t s0 = slot_of(t0);
-        bool page = n == RUN && p.block_size == RUN && s0 >= 0 && s0 % RUN == 0 && p.vc_stride[3] == 1 &&
+        bool page = n == RUN && p.block_size % RUN == 0 && s0 >= 0 && s0 % RUN == 0 && p.vc_stride[3] == 1 &&
                     (((uintptr_t)p.v_cache | (uintptr_t)(p.vc_stride[0] * CSZ) | (uintptr_t)(p.vc_stride[1] * CSZ) |
                       (uintptr_t)(p.vc_stride[2] * CSZ)) & 15) == 0;
         for (int i = 1; page && i < RUN; ++i) page = slot_of(t0 + i) == s0 + i;
         if (page) {
-            uint8_t *dst = (uint8_t *)p.v_cache + ((s0 / RUN) * p.vc_stride[0] + (int64_t)h * p.vc_stride[1] + (int64_t)d * p.vc_stride[2]) * CSZ;
+            uint8_t *dst = (uint8_t *)p.v_cache + ((s0 / p.block_size) * p.vc_stride[0] + (int64_t)h * p.vc_stride[1] +
+                                               (int64_t)d * p.vc_stride[2] + s0 % p.block_size) * CSZ;
             if (FP8) {
                 __attribute__((aligned(16))) uint8_t b[RUN];
 #pragma unroll

@@ -101,16 +101,17 @@ def test_written_cache_feeds_the_attention_oracle_layout():
     assert torch.equal(kb, k) and torch.equal(vb, v)
 
 
+@pytest.mark.parametrize("bs", [16, 32])
 @pytest.mark.parametrize("dtype,fp8", [(torch.bfloat16, False), (torch.float32, False), (torch.bfloat16, True)])
-def test_page_ordered_runs_and_broken_runs(dtype, fp8):
-    """A prefill chunk is written page by page (whole 16-token runs land in one page, in order);
-    runs broken by a skipped token or ending short take the per-token route."""
-    print(f"case: page-ordered slots {dtype} fp8={fp8}", flush=True)
+def test_page_ordered_runs_and_broken_runs(dtype, fp8, bs):
+    """A prefill chunk is written page by page (whole 16-token runs land in 16 aligned slots of one page, in
+    order); runs broken by a skipped token or ending short take the per-token route."""
+    print(f"case: page-ordered slots {dtype} fp8={fp8} page={bs}", flush=True)
     d, t = 64 if dtype == torch.float32 else 128, 70
-    table, q, k, v, pos, slots, kc, vc = _case(dtype, d, 4, 2, t, fp8=fp8, seed=21)
+    table, q, k, v, pos, slots, kc, vc = _case(dtype, d, 4, 2, t, fp8=fp8, seed=21, bs=bs)
     nb = kc.shape[0]
     pages = torch.randperm(nb)[:5]
-    slots = (pages[:, None] * 16 + torch.arange(16)[None, :]).flatten()[:t].clone()
+    slots = (pages[:, None] * bs + torch.arange(bs)[None, :]).flatten()[:t].clone()
     slots[37] = -1                                                # breaks the third run
     ks, vs = (0.02, 0.01) if fp8 else (1.0, 1.0)
     kc_ref, vc_ref = kc.clone(), vc.clone()
