@@ -133,7 +133,7 @@ template <int HD> constexpr int lds_bytes(int nc) { return Geo<HD>::KV_BYTES + n
 // WIN: built with the sliding-window code (calls without a window run the instantiation without it)
 template <int NC, int HD, bool FP8, bool WIN, typename T, typename TT>
 __global__ void __launch_bounds__((NC + 4) * 64)
-prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int n_mt) {
+prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int n_mt, const int mt_total) {
     using G = Geo<HD>;
     constexpr int D = HD, HALF = HD / 2;
     constexpr int K_PAGE = G::K_PAGE, K_TILE = G::K_TILE, V_G = G::V_G, V_PAGE = G::V_PAGE, V_TILE = G::V_TILE;
@@ -149,9 +149,63 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     const bool gatherer = wave >= NC;
 
     // ---- work item: the m-tiles of one (request, kv-head, split) land on the same XCD ----
-    const int n_groups = p.batch * p.num_kv_heads * nsplit;
-    int mt, kvgrp;
-    {
+    const int group = p.num_q_heads / p.num_kv_heads;
+    int mt, split, g, b;
+    if (mt_total > 0) {
+        // Compact list: the grid holds (kv head, split, I) for I below a host-side bound on the number of m-tiles
+        // of all requests together; I is resolved to (request, m-tile) here from the token offsets.  Used when
+        // most (request, m-tile) pairs of the plain mapping would be empty: requests with one new token next to
+        // a long one.  Workgroups of one kv head stay on one XCD.
+        const int L = blockIdx.x, hkv = p.num_kv_heads;
+        int q;
+        if ((hkv & 7) == 0) { g = (L & 7) + 8 * ((L >> 3) % (hkv >> 3)); q = (L >> 3) / (hkv >> 3); }
+        else { g = L % hkv; q = L / hkv; }
+        split = q % nsplit;
+        const int item = q / nsplit;
+        int base = 0;
+        b = -1; mt = 0;
+        // 256 requests per round, four per lane: their offsets are requested together (one memory round trip),
+        // the m-tile counts are summed per lane, scanned over the wave, and the hit is located inside its lane
+        for (int c = 0; c < p.batch; c += 256) {
+            const int r0 = c + lane * 4;
+            int64_t off[5];
+#pragma unroll
+            for (int j = 0; j < 5; ++j) {
+                const int rb = r0 + j;
+                off[j] = load_index(p.b_start_loc, rb < p.batch ? rb : p.batch, p.index_bits);
+            }
+            int cn[4], tot = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int ql = r0 + j < p.batch ? (int)(off[j + 1] - off[j]) : 0;
+                cn[j] = (ql > 0 && !(p.skip_decode && ql == 1)) ? (((ql + UNIT - 1) / UNIT) * group + NC - 1) / NC : 0;
+                tot += cn[j];
+            }
+            int incl = tot;                                       // inclusive prefix sum over the wave
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const int up = __shfl_up(incl, d);
+                if (lane >= d) incl += up;
+            }
+            const uint64_t hit = __builtin_amdgcn_ballot_w64(base + incl > item);
+            if (hit) {
+                const int idx = __builtin_ctzll(hit);
+                int rem = item - (base + __builtin_amdgcn_readlane(incl - tot, idx));
+                const int c0 = __builtin_amdgcn_readlane(cn[0], idx), c1 = __builtin_amdgcn_readlane(cn[1], idx),
+                          c2 = __builtin_amdgcn_readlane(cn[2], idx);
+                int j = 0;
+                if (rem >= c0) { rem -= c0; j = 1; if (rem >= c1) { rem -= c1; j = 2; if (rem >= c2) { rem -= c2; j = 3; } } }
+                b = c + idx * 4 + j;
+                mt = rem;
+                break;
+            }
+            base += __builtin_amdgcn_readlane(incl, 63);
+        }
+        if (b < 0) return;
+        b = uniform(b); mt = uniform(mt);
+    } else {
+        const int n_groups = p.batch * p.num_kv_heads * nsplit;
+        int kvgrp;
         const int L = blockIdx.x;
         if (((p.batch * p.num_kv_heads) & 7) == 0) {
             // every split and m-tile of one (request, kv-head) on one XCD: they share K/V through its L2
@@ -167,11 +221,10 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             mt = L % n_mt;
             kvgrp = L / n_mt;
         }
+        split = kvgrp % nsplit;
+        g = (kvgrp / nsplit) % p.num_kv_heads;
+        b = kvgrp / (nsplit * p.num_kv_heads);
     }
-    const int split = kvgrp % nsplit;
-    const int g = (kvgrp / nsplit) % p.num_kv_heads;
-    const int b = kvgrp / (nsplit * p.num_kv_heads);
-    const int group = p.num_q_heads / p.num_kv_heads;
 
     const int64_t qs = load_index(p.b_start_loc, b, p.index_bits);
     const int q_len = (int)(load_index(p.b_start_loc, b + 1, p.index_bits) - qs);
@@ -860,6 +913,33 @@ static int mfma_units(const lazyattn_prefill_params &p) {
     const int group = p.num_q_heads / p.num_kv_heads;
     return ((p.max_q_len + UNIT - 1) / UNIT) * group;
 }
+static int mfma_mtiles(const lazyattn_prefill_params &p, int nw) { return (mfma_units(p) + nw - 1) / nw; }
+
+// M-tiles (workgroups per kv head and split) the call has, estimated from what the host knows -- the token
+// count, the request count and the longest request -- by taking every request to have either one new token or
+// max_q_len of them.  Exact for uniform batches and for one long request among one-token requests, the two
+// shapes a serving batch usually has; it only steers the split count and the workgroup shape.
+static int64_t mfma_mtiles_estimate(const lazyattn_prefill_params &p, int nw) {
+    const int64_t per_req = mfma_mtiles(p, nw);
+    if (p.batch <= 1 || p.max_q_len <= 1) return (int64_t)p.batch * per_req;
+    int64_t longs = ((int64_t)p.num_tokens - p.batch + p.max_q_len - 2) / (p.max_q_len - 1);
+    longs = longs < 1 ? 1 : (longs > p.batch ? p.batch : longs);
+    const int group = p.num_q_heads / p.num_kv_heads;
+    const int64_t per_short = (group + nw - 1) / nw;             // a one-token request, unless it is skipped
+    return longs * per_req + (p.skip_decode ? 0 : (p.batch - longs) * per_short);
+}
+// Upper bound on the same number: every request may end with a partly filled 32-row chunk and a partly filled
+// m-tile.  The compact work list is sized by it.
+static int64_t mfma_mtiles_bound(const lazyattn_prefill_params &p, int nw) {
+    const int group = p.num_q_heads / p.num_kv_heads;
+    const int64_t chunks = ((int64_t)p.num_tokens + UNIT - 1) / UNIT + p.batch;
+    return (chunks * group + nw - 1) / nw + p.batch;
+}
+// The compact list pays a scan of the token offsets per workgroup: taken when it at least halves the grid.
+static bool mfma_compact(const lazyattn_prefill_params &p, int nw) {
+    return p.batch > 1 && mfma_mtiles_bound(p, nw) * 2 <= (int64_t)p.batch * mfma_mtiles(p, nw);
+}
+
 // units (computing waves) per workgroup
 static int mfma_waves(const lazyattn_prefill_params &p) {
     if (p.kernel == LAZYATTN_KERNEL_MFMA4) return 4;
@@ -867,16 +947,14 @@ static int mfma_waves(const lazyattn_prefill_params &p) {
     const int units = mfma_units(p);
     if (units <= 4) return 4;
     // 64-key tiles of work per CU if the 8-unit kernel is used: small calls take the lighter one
-    const int64_t wgs8 = (int64_t)p.batch * p.num_kv_heads * ((units + 7) / 8);
+    const int64_t wgs8 = p.num_kv_heads * mfma_mtiles_estimate(p, 8);
     const int64_t tiles = p.max_seq_len > 0 ? (p.max_seq_len + NT - 1) / NT : 64;
     return wgs8 * tiles >= 16 * 256 ? 8 : 4;
 }
 
-static int mfma_mtiles(const lazyattn_prefill_params &p, int nw) { return (mfma_units(p) + nw - 1) / nw; }
-
 static int mfma_splits(const lazyattn_prefill_params &p, int nw) {
     if (p.num_splits > 0) return p.num_splits > 64 ? 64 : p.num_splits;
-    const int64_t natural = (int64_t)p.batch * p.num_kv_heads * mfma_mtiles(p, nw);
+    const int64_t natural = p.num_kv_heads * mfma_mtiles_estimate(p, nw);
     const int64_t ctx_tiles = p.max_seq_len > 0 ? (p.max_seq_len + NT - 1) / NT : 1;
     int64_t s = (256 + natural - 1) / natural;        // one workgroup per CU
     if (s > ctx_tiles / 2) s = ctx_tiles / 2;        // at least two tiles per split
@@ -914,7 +992,7 @@ size_t mfma_workspace_bytes(const lazyattn_prefill_params &p) {
 }
 
 template <int NC, int HD, bool FP8, bool WIN, typename T, typename TT>
-static int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt, hipStream_t stream) {
+static int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt, int mt_total, hipStream_t stream) {
     auto kern = prefill_mfma_kernel<NC, HD, FP8, WIN, T, TT>;
     constexpr int LDS_BYTES = lds_bytes<HD>(NC);
     // the attribute belongs to the device's copy of the kernel: once per device, on the caller's current device
@@ -926,33 +1004,36 @@ static int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt,
             return LAZYATTN_E_LAUNCH;
         attr_set[dev] = true;
     }
-    const unsigned nblocks = (unsigned)(p.batch * p.num_kv_heads * nsplit * n_mt);
-    hipLaunchKernelGGL(kern, dim3(nblocks), dim3((NC + 4) * 64), LDS_BYTES, stream, p, nsplit, n_mt);
+    const int64_t nb = (int64_t)p.num_kv_heads * nsplit * (mt_total > 0 ? (int64_t)mt_total : (int64_t)p.batch * n_mt);
+    if (nb <= 0 || nb > 0x7fffffff) return LAZYATTN_E_SHAPE;
+    hipLaunchKernelGGL(kern, dim3((unsigned)nb), dim3((NC + 4) * 64), LDS_BYTES, stream, p, nsplit, n_mt, mt_total);
     return hipGetLastError() == hipSuccess ? LAZYATTN_OK : LAZYATTN_E_LAUNCH;
 }
 
 template <int NC, int HD, bool WIN, typename T>
-static int launch_mfma_hd(const lazyattn_prefill_params &p, int nsplit, int n_mt, hipStream_t stream) {
+static int launch_mfma_hd(const lazyattn_prefill_params &p, int nsplit, int n_mt, int mt_total, hipStream_t stream) {
     const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3;
     const bool t32 = p.table_dtype == LAZYATTN_F32;
-    if (fp8) return t32 ? launch_mfma_t<NC, HD, true, WIN, T, float>(p, nsplit, n_mt, stream)
-                        : launch_mfma_t<NC, HD, true, WIN, T, T>(p, nsplit, n_mt, stream);
-    return t32 ? launch_mfma_t<NC, HD, false, WIN, T, float>(p, nsplit, n_mt, stream)
-               : launch_mfma_t<NC, HD, false, WIN, T, T>(p, nsplit, n_mt, stream);
+    if (fp8) return t32 ? launch_mfma_t<NC, HD, true, WIN, T, float>(p, nsplit, n_mt, mt_total, stream)
+                        : launch_mfma_t<NC, HD, true, WIN, T, T>(p, nsplit, n_mt, mt_total, stream);
+    return t32 ? launch_mfma_t<NC, HD, false, WIN, T, float>(p, nsplit, n_mt, mt_total, stream)
+               : launch_mfma_t<NC, HD, false, WIN, T, T>(p, nsplit, n_mt, mt_total, stream);
 }
 template <int NC, typename T>
-static int launch_mfma_nc(const lazyattn_prefill_params &p, int nsplit, int n_mt, hipStream_t stream) {
+static int launch_mfma_nc(const lazyattn_prefill_params &p, int nsplit, int n_mt, int mt_total, hipStream_t stream) {
     if (p.head_dim == 64)
-        return p.sliding_window > 0 ? launch_mfma_hd<NC, 64, true, T>(p, nsplit, n_mt, stream)
-                                    : launch_mfma_hd<NC, 64, false, T>(p, nsplit, n_mt, stream);
-    if (p.sliding_window > 0) return launch_mfma_hd<NC, 128, true, T>(p, nsplit, n_mt, stream);
-    return launch_mfma_hd<NC, 128, false, T>(p, nsplit, n_mt, stream);
+        return p.sliding_window > 0 ? launch_mfma_hd<NC, 64, true, T>(p, nsplit, n_mt, mt_total, stream)
+                                    : launch_mfma_hd<NC, 64, false, T>(p, nsplit, n_mt, mt_total, stream);
+    if (p.sliding_window > 0) return launch_mfma_hd<NC, 128, true, T>(p, nsplit, n_mt, mt_total, stream);
+    return launch_mfma_hd<NC, 128, false, T>(p, nsplit, n_mt, mt_total, stream);
 }
 
 int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
     const int nw = mfma_waves(p);
     const int nsplit = mfma_splits(p, nw);
     const int n_mt = mfma_mtiles(p, nw);
+    const int64_t bound = mfma_mtiles_bound(p, nw);
+    const int mt_total = mfma_compact(p, nw) && bound <= 0x7fffffff ? (int)bound : 0;
     const int phases = p.phases ? p.phases : LAZYATTN_PHASE_ALL;
     if (nsplit > 1) {
         const size_t need = (size_t)nsplit * (size_t)p.num_tokens * p.num_q_heads * partial_row_bytes(p);
@@ -961,8 +1042,8 @@ int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
     }
     if (phases & LAZYATTN_PHASE_MAIN) {
         const bool f16 = p.dtype == LAZYATTN_F16;
-        const int rc = nw == 8 ? (f16 ? launch_mfma_nc<8, f16_t>(p, nsplit, n_mt, stream) : launch_mfma_nc<8, bf16_t>(p, nsplit, n_mt, stream))
-                               : (f16 ? launch_mfma_nc<4, f16_t>(p, nsplit, n_mt, stream) : launch_mfma_nc<4, bf16_t>(p, nsplit, n_mt, stream));
+        const int rc = nw == 8 ? (f16 ? launch_mfma_nc<8, f16_t>(p, nsplit, n_mt, mt_total, stream) : launch_mfma_nc<8, bf16_t>(p, nsplit, n_mt, mt_total, stream))
+                               : (f16 ? launch_mfma_nc<4, f16_t>(p, nsplit, n_mt, mt_total, stream) : launch_mfma_nc<4, bf16_t>(p, nsplit, n_mt, mt_total, stream));
         if (rc != LAZYATTN_OK) return rc;
     }
     if (nsplit > 1 && (phases & LAZYATTN_PHASE_COMBINE)) {
