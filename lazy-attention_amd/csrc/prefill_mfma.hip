@@ -840,6 +840,7 @@ struct MergeArgs {
     void *o;
     int64_t o_stride[2];
     int32_t num_tokens, num_q_heads, index_bits, skip_decode;
+    int32_t batch, token_grid;      // token_grid: rows are numbered over all tokens instead of per request
 };
 // NB = splits taken per batch of loads: 2, 4 or 8, the smallest that covers nsplit (more only when nsplit > 8)
 template <typename T, int HD, int NB>
@@ -847,13 +848,30 @@ __global__ void __launch_bounds__(256)
 prefill_combine_kernel(const MergeArgs p, const int nsplit) {
     using E = Elem<T>;
     constexpr int D = HD, LPR = HD / 8;                       // lanes per row (8 elements = one 16-byte load each)
-    const int b = blockIdx.y;
-    const int64_t qs = load_index(p.b_start_loc, b, p.index_bits);
-    const int64_t q_len = load_index(p.b_start_loc, b + 1, p.index_bits) - qs;
-    if (q_len <= 0 || (p.skip_decode && q_len == 1)) return;
     const int64_t r = (int64_t)blockIdx.x * (256 / LPR) + threadIdx.x / LPR;
-    if (r >= q_len * p.num_q_heads) return;
-    const int64_t tok = qs + r / p.num_q_heads;
+    int64_t tok;
+    if (p.token_grid) {
+        // Rows over all tokens of the call: no workgroup is launched for rows a request does not have (a grid
+        // of batch x longest request is mostly empty when one long request sits among one-token requests).
+        // Only the skipping of one-token requests needs the row's request: a binary search of the offsets.
+        tok = r / p.num_q_heads;
+        if (tok >= load_index(p.b_start_loc, p.batch, p.index_bits)) return;
+        if (p.skip_decode) {
+            int lo = 0, hi = p.batch;                         // offsets[lo] <= tok < offsets[hi]
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) >> 1;
+                if (load_index(p.b_start_loc, mid, p.index_bits) <= tok) lo = mid; else hi = mid;
+            }
+            if (load_index(p.b_start_loc, lo + 1, p.index_bits) - load_index(p.b_start_loc, lo, p.index_bits) == 1) return;
+        }
+    } else {
+        const int b = blockIdx.y;
+        const int64_t qs = load_index(p.b_start_loc, b, p.index_bits);
+        const int64_t q_len = load_index(p.b_start_loc, b + 1, p.index_bits) - qs;
+        if (q_len <= 0 || (p.skip_decode && q_len == 1)) return;
+        if (r >= q_len * p.num_q_heads) return;
+        tok = qs + r / p.num_q_heads;
+    }
     const int h = (int)(r % p.num_q_heads);
     const int d = (threadIdx.x % LPR) * 8;
     const int64_t NTOK = p.num_tokens;
@@ -1047,11 +1065,13 @@ int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
         if (rc != LAZYATTN_OK) return rc;
     }
     if (nsplit > 1 && (phases & LAZYATTN_PHASE_COMBINE)) {
-        const int64_t rows = (int64_t)p.max_q_len * p.num_q_heads;
+        // rows per request x requests, or rows over all tokens when that is at most half as many
+        const int token_grid = p.batch > 1 && 2 * (int64_t)p.num_tokens <= (int64_t)p.batch * p.max_q_len;
+        const int64_t rows = (int64_t)(token_grid ? p.num_tokens : p.max_q_len) * p.num_q_heads;
         const MergeArgs m{p.workspace, p.b_start_loc, p.o, {p.o_stride[0], p.o_stride[1]}, p.num_tokens, p.num_q_heads,
-                          p.index_bits, p.skip_decode};
+                          p.index_bits, p.skip_decode, p.batch, token_grid};
         const int rows_wg = 256 / (p.head_dim / 8);
-        const dim3 grid((unsigned)((rows + rows_wg - 1) / rows_wg), p.batch);
+        const dim3 grid((unsigned)((rows + rows_wg - 1) / rows_wg), token_grid ? 1 : p.batch);
         const bool f16 = p.dtype == LAZYATTN_F16;
 #define LAZYATTN_COMBINE(HD, NB)                                                                              \
     {                                                                                                         \
