@@ -13,7 +13,8 @@
 //     v_mfma_f32_16x16x32_bf16 for S^T = K . Q^T, and holds both halves (d, d + 64) of its
 //     rotation pairs, so the rotation happens in place;
 //   * the query heads of the group are the 16 columns of the MFMA (heads beyond the group are
-//     zero columns): the matrix pipe is mostly idle here and that is fine;
+//     zero columns; a group above 16 is cut into blocks of 16 heads, one wave each): the matrix
+//     pipe is mostly idle here and that is fine;
 //   * S^T comes out as (4 tokens per lane) x (head = lane % 16): each lane runs the online
 //     softmax of one head, lanes 16 apart share a head and exchange the row max;
 //   * P^T (two pages = 32 tokens) is the B operand of O^T += V^T . P^T as it stands if the
@@ -90,13 +91,18 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     const int lane = threadIdx.x & 63;
     const int wave = uniform(threadIdx.x >> 6);
     const int W = blockIdx.x * WAVES + wave;
-    if (W >= p.batch * p.num_kv_heads * nsplit) return;
-    // kv heads vary fastest: the waves of a workgroup walk the same pages, whose heads are
-    // adjacent 4 KB pieces of one cache block
-    const int g = W % p.num_kv_heads;
-    const int split = (W / p.num_kv_heads) % nsplit;
-    const int b = W / (nsplit * p.num_kv_heads);
     const int group = p.num_q_heads / p.num_kv_heads;
+    // a wave takes 16 query heads of a kv head (the columns of its MFMAs): groups above 16 are cut into blocks
+    // that walk the same pages side by side
+    const int hblocks = (group + 15) >> 4;
+    const int kvh = p.num_kv_heads * hblocks;
+    if (W >= p.batch * kvh * nsplit) return;
+    // (head block, then) kv heads vary fastest: the waves of a workgroup walk the same pages, whose heads are
+    // adjacent 4 KB pieces of one cache block
+    const int hb0 = (W % hblocks) * 16;                          // first head of this wave's block within the group
+    const int g = (W % kvh) / hblocks;
+    const int split = (W / kvh) % nsplit;
+    const int b = W / (nsplit * kvh);
 
     const int64_t qs = load_index(p.b_start_loc, b, p.index_bits);
     const int q_len = (int)(load_index(p.b_start_loc, b + 1, p.index_bits) - qs);
@@ -224,8 +230,8 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     // Q^T: column = head = t, contraction d = 32 m + 8 grp ..
     uint4 qf[NM];
     {
-        const bool head_ok = t < group;
-        const T *qp = (const T *)p.q + qs * p.q_stride[0] + (int64_t)(g * group + (head_ok ? t : 0)) * p.q_stride[1] + 8 * grp;
+        const bool head_ok = hb0 + t < group;
+        const T *qp = (const T *)p.q + qs * p.q_stride[0] + (int64_t)(g * group + (head_ok ? hb0 + t : 0)) * p.q_stride[1] + 8 * grp;
 #pragma unroll
         for (int m = 0; m < NM; ++m) {
             uint4 w = make_uint4(0, 0, 0, 0);
@@ -319,8 +325,8 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     // ---- epilogue: lane (head t, grp) holds O^T[d = 16 blk + 4 grp + i][head t] ----
     l_run += __shfl_xor(l_run, 16);
     l_run += __shfl_xor(l_run, 32);
-    if (t >= group) return;
-    const int h = g * group + t;
+    if (hb0 + t >= group) return;
+    const int h = g * group + hb0 + t;
     const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
     if (nsplit == 1) {
         T *op = (T *)p.o + qs * p.o_stride[0] + (int64_t)h * p.o_stride[1] + 4 * grp;
@@ -406,7 +412,6 @@ bool decode_mfma_supports(const lazyattn_prefill_params &p) {
     if ((p.head_dim != 128 && p.head_dim != 64) || p.rotary_dim != p.head_dim) return false;
     if ((p.block_size != BS && p.block_size != 2 * BS) || p.x != (fp8 ? 16 : 8)) return false;
     if (p.pos_mode != LAZYATTN_POS_NATURAL && p.pos_mode != LAZYATTN_POS_BLOCK_UNIFORM) return false;
-    if (p.num_q_heads / p.num_kv_heads > 16) return false;
     if (p.q_stride[2] != 1 || p.o_stride[2] != 1) return false;
     if (p.kc_stride[4] != 1 || p.kc_stride[3] != p.x || p.kc_stride[2] != (int64_t)p.block_size * p.x) return false;
     if (p.vc_stride[3] != 1 || p.vc_stride[2] != p.block_size) return false;
@@ -425,7 +430,7 @@ bool decode_mfma_supports(const lazyattn_prefill_params &p) {
 // than they gain in parallelism (5 K keys, one request: 16-32 slices 32 us, 64 slices 43 us)
 static int decode_splits(const lazyattn_prefill_params &p) {
     if (p.num_splits > 0) return p.num_splits > 64 ? 64 : p.num_splits;
-    const int64_t natural = (int64_t)p.batch * p.num_kv_heads;
+    const int64_t natural = (int64_t)p.batch * p.num_kv_heads * ((p.num_q_heads / p.num_kv_heads + 15) / 16);
     if (natural <= 0) return 1;
     int64_t s = (256 * 8 + natural - 1) / natural;
     const int64_t pages = p.max_seq_len > 0 ? (p.max_seq_len + BS - 1) / BS : 64;
@@ -448,7 +453,7 @@ int launch_decode_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
         if (!p.workspace || (size_t)p.workspace_bytes < need || (((uintptr_t)p.workspace) & 15)) nsplit = 1;
     }
     const int phases = p.phases ? p.phases : LAZYATTN_PHASE_ALL;
-    const int64_t waves = (int64_t)p.batch * p.num_kv_heads * nsplit;
+    const int64_t waves = (int64_t)p.batch * p.num_kv_heads * ((p.num_q_heads / p.num_kv_heads + 15) / 16) * nsplit;
     const unsigned nblocks = (unsigned)((waves + WAVES - 1) / WAVES);
     if (phases & LAZYATTN_PHASE_MAIN) {
         const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3, t32 = p.table_dtype == LAZYATTN_F32;

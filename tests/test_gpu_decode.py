@@ -110,13 +110,14 @@ def test_decode_vanilla_requests_and_fp32_table():
     assert _err(got, ref) < 2e-2, _err(got, ref)
 
 
-@pytest.mark.parametrize("hq,hkv", [(4, 4), (16, 2), (32, 2), (3, 1), (28, 4), (24, 2)])
+@pytest.mark.parametrize("hq,hkv", [(4, 4), (16, 2), (32, 2), (3, 1), (28, 4), (24, 2), (64, 1), (40, 2), (34, 2)])
 def test_decode_group_sizes(hq, hkv):
     print(f"case: decode group {hq // hkv}", flush=True)
     w = _decode_batch("natural", hq=hq, hkv=hkv)
     ref = _oracle(w)
-    got = _run(w)
-    assert _err(got, ref) < 2e-2, _err(got, ref)
+    for nsplit in (0, 1, 3):
+        got = _run(w, num_splits=nsplit, kernel=_ffi.KERNEL_MFMA)      # groups above 16: blocks of 16 heads
+        assert _err(got, ref) < 2e-2, (nsplit, _err(got, ref))
 
 
 @pytest.mark.parametrize("variant", ["natural", "block_uniform"])
