@@ -73,9 +73,10 @@ typedef struct lazyattn_prefill_params {
                                    LAZYATTN_POS_BLOCK_UNIFORM (ops/prefix_prefill.py:98) */
     const void *b_start_loc;    /* [B+1] int32 or int64, see index_bits */
     const void *b_seq_len;      /* [B] */
-    const void *cos_sin_cache;  /* [max_pos, rotary_dim]: row p = cos(p*inv) | sin(p*inv); only rows of
-                                   positions that real keys take are read (max_pos >= the longest
-                                   b_seq_len suffices for LAZYATTN_POS_NATURAL) */
+    const void *cos_sin_cache;  /* [max_pos, rotary_dim]: row p = cos(p*inv) | sin(p*inv); rows are read
+                                   for the 16-slot runs that hold real keys and for the new tokens
+                                   (LAZYATTN_POS_NATURAL: max_pos >= the longest context rounded up to
+                                   16 and >= the longest b_seq_len), like the reference's kernels */
     const void *cos_sin_packed; /* optional: the same table re-laid out by lazyattn_pack_cos_sin_cache()
                                    as [2][rotary_dim/16][packed_rows][8], so that the 16 slots of a page
                                    read 16 consecutive 16-byte chunks; NULL = read the row-major table */
