@@ -131,11 +131,14 @@ template <typename TT> struct KRegs {
 template <int HD> constexpr int lds_bytes(int nc) { return Geo<HD>::KV_BYTES + nc * Geo<HD>::Q_WAVE + 2 * PAGES * 4; }   // + Q^T fragments (re-read every tile) + page limits
 
 // WIN: built with the sliding-window code (calls without a window run the instantiation without it)
-template <int NC, int HD, bool FP8, bool WIN, typename T, typename TT>
+// PAD: the head size is a multiple of 16 below HD = 128: Q, K and V sit zero-padded in the 128-wide tiles, the two
+// halves of the real head at (0 .., 64 ..) so that the rotation pairs stay (d, 64 + d)
+template <int NC, int HD, bool FP8, bool WIN, bool PAD, typename T, typename TT>
 __global__ void __launch_bounds__((NC + 4) * 64)
 prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int n_mt, const int mt_total) {
     using G = Geo<HD>;
     constexpr int D = HD, HALF = HD / 2;
+    const int Dr = PAD ? p.head_dim : D, HALFr = Dr / 2, CPr = Dr / 16;   // real head size, its half, its chunk pairs
     constexpr int K_PAGE = G::K_PAGE, K_TILE = G::K_TILE, V_G = G::V_G, V_PAGE = G::V_PAGE, V_TILE = G::V_TILE;
     constexpr int KV_BYTES = G::KV_BYTES, KS = G::KS, DT = G::DT;
     constexpr int KI = G::K_ITEMS, VI = G::V_ITEMS;   // a page has HD K items (HD/16 chunk pairs x 16 slots) and 2 HD V items
@@ -333,7 +336,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         const bool packed_tab = p.cos_sin_packed != nullptr && per_token;
         const uint8_t *ctab_base = packed_tab ? (const uint8_t *)p.cos_sin_packed : tab_base;
         const uint32_t pos_bytes = packed_tab ? 8 * TSZ : row_bytes;       // bytes per unit of position
-        const uint32_t sin_delta = packed_tab ? (uint32_t)(HALF / 8) * (uint32_t)p.packed_rows * 8 * TSZ : HALF * TSZ;
+        const uint32_t sin_delta = packed_tab ? (uint32_t)(HALFr / 8) * (uint32_t)p.packed_rows * 8 * TSZ : HALFr * TSZ;
         // this wave's part of its cache pages (pages of 32 slots: the tile's pages 0, 1 are the two parts of
         // one cache page, 2, 3 of the next): first slot, and the position step that goes with it
         const int slot0 = (gw & part_mask) * BS;
@@ -356,10 +359,32 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
 #pragma unroll
         for (int i = 0; i < KI; ++i) {
             const int idx = lane + i * 64;
-            const int o = idx & 15, cp = idx >> 4;
+            const int o = idx & 15, cp = PAD && (idx >> 4) >= CPr ? 0 : idx >> 4;   // (a padded chunk reads chunk 0 and is zeroed)
             // block-uniform rotation and un-rotated requests use one table row for the whole page
             k_toff[i] = packed_tab ? ((uint32_t)cp * (uint32_t)p.packed_rows + (uint32_t)o) * 8 * TSZ
                                    : (per_token ? (uint32_t)o * row_bytes : 0u) + (uint32_t)cp * 8 * TSZ;
+        }
+        // PAD: per-item cache offsets (the chunk of d + Dr/2 is not a fixed distance away in an fp8 page) and
+        // which of the lane's items exist
+        uint32_t pk1[PAD ? KI : 1], pk2[PAD ? KI : 1], pv[PAD ? VI_CTX : 1];
+        bool pk_ok[PAD ? KI : 1], pv_ok[PAD ? VI_CTX : 1];
+        if constexpr (PAD) {
+#pragma unroll
+            for (int i = 0; i < KI; ++i) {
+                const int idx = lane + i * 64, o = idx & 15;
+                pk_ok[i] = (idx >> 4) < CPr;
+                const int c1 = pk_ok[i] ? idx >> 4 : 0, c2 = CPr + c1;                  // 8-element chunks of d and d + Dr/2
+                pk1[i] = FP8 ? (uint32_t)(((c1 >> 1) * cache_bs + slot0 + o) * 16 + (c1 & 1) * 8) : (uint32_t)((c1 * cache_bs + slot0 + o) * 16);
+                pk2[i] = FP8 ? (uint32_t)(((c2 >> 1) * cache_bs + slot0 + o) * 16 + (c2 & 1) * 8) : (uint32_t)((c2 * cache_bs + slot0 + o) * 16);
+            }
+#pragma unroll
+            for (int i = 0; i < VI_CTX; ++i) {
+                const int idx = lane + i * 64;
+                const int d = FP8 ? idx : idx >> 1;
+                pv_ok[i] = d < Dr;
+                const int dc = pv_ok[i] ? d : 0;
+                pv[i] = FP8 ? (uint32_t)(dc * cache_bs + slot0) : (uint32_t)(dc * cache_bs * 2 + slot0 * 2 + (idx & 1) * 16);
+            }
         }
         KRegs<TT> kr[KI];
         uint4 vr[VI];
@@ -380,7 +405,20 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
 #pragma unroll
             for (int i = 0; i < KI; ++i) {
                 kr[i].lds_off = (uint32_t)(gw * K_PAGE + (lane + i * 64) * 16);
-                if (FP8) {
+                if constexpr (PAD) {
+                    uint4 k1, k2;
+                    if (FP8) {
+                        const uint2 a = ldg8(kb, pk1[i]), a2 = ldg8(kb, pk2[i]);
+                        k1 = make_uint4(a.x, a.y, 0, 0);
+                        k2 = make_uint4(a2.x, a2.y, 0, 0);
+                    } else {
+                        k1 = ldg16(kb, pk1[i]);
+                        k2 = ldg16(kb, pk2[i]);
+                    }
+                    const uint4 z = make_uint4(0, 0, 0, 0);
+                    kr[i].k1 = pk_ok[i] ? k1 : z;
+                    kr[i].k2 = pk_ok[i] ? k2 : z;
+                } else if (FP8) {
                     const uint2 a = ldg8(kb + i * k_item, k_goff), a2 = ldg8(kb + i * k_item + pair, k_goff);
                     kr[i].k1 = make_uint4(a.x, a.y, 0, 0);
                     kr[i].k2 = make_uint4(a2.x, a2.y, 0, 0);
@@ -393,7 +431,14 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             }
             const uint8_t *vb = vc_base + pm.bt * vc_page_bytes;
 #pragma unroll
-            for (int i = 0; i < VI_CTX; ++i) vr[i] = ldg16(vb + i * v_item, v_goff);
+            for (int i = 0; i < VI_CTX; ++i) {
+                if constexpr (PAD) {
+                    const uint4 t = ldg16(vb, pv[i]);
+                    vr[i] = pv_ok[i] ? t : make_uint4(0, 0, 0, 0);
+                } else {
+                    vr[i] = ldg16(vb + i * v_item, v_goff);
+                }
+            }
         };
         // ---- loads of this wave's 16 keys of a new-token tile ----
         auto issue_loads_new = [&](int tile) {
@@ -406,14 +451,14 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                 uint4 k1 = make_uint4(0, 0, 0, 0), k2 = k1;
                 TabVec<TT> c, sn;
                 c.fill(1.f); sn.fill(0.f);
-                if (m < t_end) {
+                if (m < t_end && (!PAD || cp < CPr)) {
                     const T *kn = (const T *)p.k + (qs + m) * p.k_stride[0] + (int64_t)g * p.k_stride[1] + cp * 8;
                     k1 = *reinterpret_cast<const uint4 *>(kn);
-                    k2 = *reinterpret_cast<const uint4 *>(kn + HALF);
+                    k2 = *reinterpret_cast<const uint4 *>(kn + HALFr);
                     if (rot_new) {                                               // old_ops:342-343
                         const uint8_t *tb = tab_base + (int64_t)(ctx_len + m) * row_bytes;
                         c.load(tb, (uint32_t)cp * 8 * TSZ);
-                        sn.load(tb, (uint32_t)cp * 8 * TSZ + HALF * TSZ);
+                        sn.load(tb, (uint32_t)cp * 8 * TSZ + HALFr * TSZ);
                     }
                 }
                 kr[i].k1 = k1; kr[i].k2 = k2; kr[i].c = c; kr[i].s = sn;
@@ -425,7 +470,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                 // (the value is chosen before the one store: a store under the branch lets the compiler merge
                 // the iterations' stores behind a pointer phi, and the array then stays in scratch memory)
                 uint4 t = make_uint4(0, 0, 0, 0);
-                if (m < t_end)
+                if (m < t_end && (!PAD || dc * 8 < Dr))
                     t = *reinterpret_cast<const uint4 *>((const T *)p.v + (qs + m) * p.v_stride[0] +
                                                          (int64_t)g * p.v_stride[1] + dc * 8);
                 vr[i] = t;
@@ -603,7 +648,13 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             uint4 v = make_uint4(0, 0, 0, 0);
-            if (row_ok) v = *reinterpret_cast<const uint4 *>(qp + ks * 16);
+            if constexpr (PAD) {
+                // tile column c = ks*16 + gh*8: real element c (first half of the head) or Dr/2 + c - 64 (second)
+                const int c = ks * 16 + gh * 8, lo = c & 63;
+                if (row_ok && lo < HALFr) v = *reinterpret_cast<const uint4 *>(qp - gh * 8 + (c < 64 ? lo : HALFr + lo));
+            } else {
+                if (row_ok) v = *reinterpret_cast<const uint4 *>(qp + ks * 16);
+            }
             float f[8];
             unpack8<T>(v, f);
             *reinterpret_cast<uint4 *>(qlds + ks * 1024) =
@@ -793,6 +844,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) {
                 const int d = dt * 32 + 8 * i4 + 4 * gh;
+                if (PAD && d >= Dr) continue;                                  // padding columns of the tile
                 *reinterpret_cast<uint2 *>(op + d) =
                     make_uint2(E::pack(acc[dt][4 * i4] * inv, acc[dt][4 * i4 + 1] * inv),
                                E::pack(acc[dt][4 * i4 + 2] * inv, acc[dt][4 * i4 + 3] * inv));
@@ -841,6 +893,7 @@ struct MergeArgs {
     int64_t o_stride[2];
     int32_t num_tokens, num_q_heads, index_bits, skip_decode;
     int32_t batch, token_grid;      // token_grid: rows are numbered over all tokens instead of per request
+    int32_t head_dim;               // elements of an output row (below HD when the partial rows are padded)
 };
 // NB = splits taken per batch of loads: 2, 4 or 8, the smallest that covers nsplit (more only when nsplit > 8)
 template <typename T, int HD, int NB>
@@ -874,6 +927,7 @@ prefill_combine_kernel(const MergeArgs p, const int nsplit) {
     }
     const int h = (int)(r % p.num_q_heads);
     const int d = (threadIdx.x % LPR) * 8;
+    if (d >= p.head_dim) return;
     const int64_t NTOK = p.num_tokens;
     const _Float16 *wo = (const _Float16 *)p.workspace;
     const float2 *wl = reinterpret_cast<const float2 *>(wo + (int64_t)nsplit * NTOK * p.num_q_heads * D);
@@ -926,7 +980,9 @@ prefill_combine_kernel(const MergeArgs p, const int nsplit) {
 
 // ------------------------------------------------------------------ host side
 // a split-KV partial row: 128 halves + (log2-sum-exp, scale)
-static size_t partial_row_bytes(const lazyattn_prefill_params &p) { return (size_t)p.head_dim * sizeof(_Float16) + 2 * sizeof(float); }
+// width of the tiles and of a partial row: the head size, or 128 for the head sizes that are padded to it
+static int tile_dim(const lazyattn_prefill_params &p) { return p.head_dim == 64 ? 64 : 128; }
+static size_t partial_row_bytes(const lazyattn_prefill_params &p) { return (size_t)tile_dim(p) * sizeof(_Float16) + 2 * sizeof(float); }
 static int mfma_units(const lazyattn_prefill_params &p) {
     const int group = p.num_q_heads / p.num_kv_heads;
     return ((p.max_q_len + UNIT - 1) / UNIT) * group;
@@ -985,7 +1041,8 @@ bool mfma_supports(const lazyattn_prefill_params &p) {
     if (p.dtype != LAZYATTN_BF16 && p.dtype != LAZYATTN_F16) return false;
     if (!(p.cache_dtype == p.dtype || fp8)) return false;
     if (p.table_dtype != p.dtype && p.table_dtype != LAZYATTN_F32) return false;
-    if ((p.head_dim != 128 && p.head_dim != 64) || p.rotary_dim != p.head_dim) return false;
+    // 128, 64, or a multiple of 16 below 128 (padded to 128)
+    if (p.head_dim < 16 || p.head_dim > 128 || p.head_dim % 16 || p.rotary_dim != p.head_dim) return false;
     if ((p.block_size != BS && p.block_size != 2 * BS) || p.x != (fp8 ? 16 : 8)) return false;
     if (p.q_stride[2] != 1 || p.k_stride[2] != 1 || p.v_stride[2] != 1 || p.o_stride[2] != 1) return false;
     if (p.kc_stride[4] != 1 || p.kc_stride[3] != p.x || p.kc_stride[2] != (int64_t)p.block_size * p.x) return false;
@@ -1009,9 +1066,9 @@ size_t mfma_workspace_bytes(const lazyattn_prefill_params &p) {
     return (size_t)ns * (size_t)p.num_tokens * p.num_q_heads * partial_row_bytes(p);
 }
 
-template <int NC, int HD, bool FP8, bool WIN, typename T, typename TT>
+template <int NC, int HD, bool FP8, bool WIN, bool PAD, typename T, typename TT>
 static int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt, int mt_total, hipStream_t stream) {
-    auto kern = prefill_mfma_kernel<NC, HD, FP8, WIN, T, TT>;
+    auto kern = prefill_mfma_kernel<NC, HD, FP8, WIN, PAD, T, TT>;
     constexpr int LDS_BYTES = lds_bytes<HD>(NC);
     // the attribute belongs to the device's copy of the kernel: once per device, on the caller's current device
     static bool attr_set[64] = {};
@@ -1028,22 +1085,24 @@ static int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt,
     return hipGetLastError() == hipSuccess ? LAZYATTN_OK : LAZYATTN_E_LAUNCH;
 }
 
-template <int NC, int HD, bool WIN, typename T>
+template <int NC, int HD, bool WIN, bool PAD, typename T>
 static int launch_mfma_hd(const lazyattn_prefill_params &p, int nsplit, int n_mt, int mt_total, hipStream_t stream) {
     const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3;
     const bool t32 = p.table_dtype == LAZYATTN_F32;
-    if (fp8) return t32 ? launch_mfma_t<NC, HD, true, WIN, T, float>(p, nsplit, n_mt, mt_total, stream)
-                        : launch_mfma_t<NC, HD, true, WIN, T, T>(p, nsplit, n_mt, mt_total, stream);
-    return t32 ? launch_mfma_t<NC, HD, false, WIN, T, float>(p, nsplit, n_mt, mt_total, stream)
-               : launch_mfma_t<NC, HD, false, WIN, T, T>(p, nsplit, n_mt, mt_total, stream);
+    if (fp8) return t32 ? launch_mfma_t<NC, HD, true, WIN, PAD, T, float>(p, nsplit, n_mt, mt_total, stream)
+                        : launch_mfma_t<NC, HD, true, WIN, PAD, T, T>(p, nsplit, n_mt, mt_total, stream);
+    return t32 ? launch_mfma_t<NC, HD, false, WIN, PAD, T, float>(p, nsplit, n_mt, mt_total, stream)
+               : launch_mfma_t<NC, HD, false, WIN, PAD, T, T>(p, nsplit, n_mt, mt_total, stream);
 }
 template <int NC, typename T>
 static int launch_mfma_nc(const lazyattn_prefill_params &p, int nsplit, int n_mt, int mt_total, hipStream_t stream) {
     if (p.head_dim == 64)
-        return p.sliding_window > 0 ? launch_mfma_hd<NC, 64, true, T>(p, nsplit, n_mt, mt_total, stream)
-                                    : launch_mfma_hd<NC, 64, false, T>(p, nsplit, n_mt, mt_total, stream);
-    if (p.sliding_window > 0) return launch_mfma_hd<NC, 128, true, T>(p, nsplit, n_mt, mt_total, stream);
-    return launch_mfma_hd<NC, 128, false, T>(p, nsplit, n_mt, mt_total, stream);
+        return p.sliding_window > 0 ? launch_mfma_hd<NC, 64, true, false, T>(p, nsplit, n_mt, mt_total, stream)
+                                    : launch_mfma_hd<NC, 64, false, false, T>(p, nsplit, n_mt, mt_total, stream);
+    // other head sizes: the 128-wide kernel with padding (built with the window code, which a window of 0 switches off)
+    if (p.head_dim != 128) return launch_mfma_hd<NC, 128, true, true, T>(p, nsplit, n_mt, mt_total, stream);
+    if (p.sliding_window > 0) return launch_mfma_hd<NC, 128, true, false, T>(p, nsplit, n_mt, mt_total, stream);
+    return launch_mfma_hd<NC, 128, false, false, T>(p, nsplit, n_mt, mt_total, stream);
 }
 
 int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
@@ -1069,8 +1128,8 @@ int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
         const int token_grid = p.batch > 1 && 2 * (int64_t)p.num_tokens <= (int64_t)p.batch * p.max_q_len;
         const int64_t rows = (int64_t)(token_grid ? p.num_tokens : p.max_q_len) * p.num_q_heads;
         const MergeArgs m{p.workspace, p.b_start_loc, p.o, {p.o_stride[0], p.o_stride[1]}, p.num_tokens, p.num_q_heads,
-                          p.index_bits, p.skip_decode, p.batch, token_grid};
-        const int rows_wg = 256 / (p.head_dim / 8);
+                          p.index_bits, p.skip_decode, p.batch, token_grid, p.head_dim};
+        const int rows_wg = 256 / (tile_dim(p) / 8);
         const dim3 grid((unsigned)((rows + rows_wg - 1) / rows_wg), token_grid ? 1 : p.batch);
         const bool f16 = p.dtype == LAZYATTN_F16;
 #define LAZYATTN_COMBINE(HD, NB)                                                                              \

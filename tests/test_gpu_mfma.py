@@ -203,6 +203,26 @@ def test_mfma_one_long_request_among_short_requests(n_short, q_short, skip, kern
         assert e < 2e-2, (nsplit, e)
 
 
+@pytest.mark.parametrize("d", [96, 80, 112, 48, 32, 16])
+@pytest.mark.parametrize("variant", ["natural", "offset", "block_uniform"])
+@pytest.mark.parametrize("dtype,kv,page", [(torch.bfloat16, "auto", 16), (torch.float16, "auto", 32), (torch.bfloat16, "fp8", 16)])
+def test_mfma_head_sizes_padded_to_128(d, variant, dtype, kv, page):
+    """Head sizes that are multiples of 16 below 128 (96 is in the reference's test grid, tests/kernels/
+    test_prefix_prefill.py:41 with vLLM's HEAD_SIZES) run the 128-wide kernel with Q, K and V zero-padded in its
+    tiles; forcing the matrix kernel fails if it does not take them."""
+    print(f"case: mfma head size {d} {variant} {dtype} kv={kv} page={page}", flush=True)
+    w = wl.make_workload("pad", dtype=dtype, hq=32, hkv=8, d=d, theta=500000.0, block_size=page,
+                         doc_lens=[100, 16, 333, 70, 5, 250], requests=[[3, 1, 0], [2], [0, 2, 3, 1, 5], [4], []],
+                         q_lens=[70, 1, 9, 33, 130], variant=variant, kv_cache_dtype=kv, seed=d)
+    tol = 5e-2 if kv == "fp8" else (2e-2 if dtype == torch.bfloat16 else 5e-3)
+    for window in (0, 50):
+        ref = run_oracle(w, sliding_window=window)
+        for nsplit, kernel in ((1, _ffi.KERNEL_MFMA4), (3, _ffi.KERNEL_MFMA8)):
+            got = run_op(w.to(DEV), kernel=kernel, num_splits=nsplit, sliding_window=window or None).cpu()
+            e = _err(got, ref)
+            assert e < tol, (window, nsplit, e)
+
+
 def test_mfma_takes_views_of_a_packed_qkv_tensor():
     """vLLM hands q, k, v as views of one [T, (Hq + 2 Hkv) D] projection output and writes o into a wider buffer:
     token strides larger than the row, the matrix path must take them as they are."""

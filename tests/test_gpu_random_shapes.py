@@ -46,6 +46,8 @@ def _draw(seed):
     window = r.choice([0, 0, 7, 50, 300])
     d = r.choice([128, 128, 64])
     page = r.choice([16, 16, 32])
+    if r.random() < 0.25:
+        d = r.choice([96, 80, 48, 112])     # padded to 128 inside the matrix kernel
     return dict(page=page, dtype=dtype, window=window, d=d, hq=hkv * group, hkv=hkv, doc_lens=doc_lens, requests=requests, q_lens=q_lens, variant=variant,
                 kv=kv, nsplit=nsplit, kernel=kernel)
 
