@@ -35,7 +35,7 @@ enum {
 enum {
     LAZYATTN_KERNEL_AUTO = 0,
     LAZYATTN_KERNEL_GENERIC = 1, /* fp32 arithmetic, any geometry */
-    LAZYATTN_KERNEL_MFMA = 2,    /* bf16 / fp16 MFMA, head_dim 128 or 64, pages of 16 or 32 slots; workgroup shape chosen */
+    LAZYATTN_KERNEL_MFMA = 2,    /* bf16 / fp16 MFMA, head_dim 128, 64 or a multiple of 16 below 128, pages of 16 or 32 slots; workgroup shape chosen */
     LAZYATTN_KERNEL_MFMA4 = 3,   /* ... with 4 x 32 query rows per workgroup */
     LAZYATTN_KERNEL_MFMA8 = 4    /* ... with 8 x 32 query rows per workgroup */
 };
