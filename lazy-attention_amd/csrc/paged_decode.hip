@@ -1,4 +1,5 @@
-// q_len == 1 rows with the rotation fused in: bf16 (cache bf16 or fp8 e4m3), head_dim 128, 16-token pages, gfx950.
+// q_len == 1 rows with the rotation fused in: bf16 / float16 (cache of the same type or fp8 e4m3), head sizes 128, 64 and
+// other multiples of 16 below 128 (padded), pages of 16 or 32 slots, gfx950.
 //
 // Follows old_ops/chunked_prefill_paged_decode.py:23-280 (un-rotated cache, key n rotated
 // at position n) and ops/models/llama_v1.py:18-637 (block-uniform rotation by q_offset-1,
@@ -82,12 +83,15 @@ template <int HD> struct ValRegs {
 
 }  // namespace
 
-template <typename T, typename TT, bool FP8, int HD>
+// PAD: the head size is a multiple of 16 below HD = 128; the lane's chunks, the query and the V rows are laid out as
+// for 128 with the two halves of the real head at (0 .., 64 ..) and zeros in between
+template <typename T, typename TT, bool FP8, int HD, bool PAD>
 __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2)))
 paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     using E = Elem<T>;
-    constexpr int D = HD, HALF = HD / 2, NM = HD / 32, NP = HD / 64, NBLK = HD / 16;
+    constexpr int D = HD, NM = HD / 32, NP = HD / 64, NBLK = HD / 16;
     constexpr int TSZ = sizeof(TT);
+    const int Dr = PAD ? p.head_dim : D, HALFr = Dr / 2, CPr = Dr / 16, NBr = Dr / 16;   // real sizes
     const int lane = threadIdx.x & 63;
     const int wave = uniform(threadIdx.x >> 6);
     const int W = blockIdx.x * WAVES + wave;
@@ -153,6 +157,19 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     const uint32_t v_off = FP8 ? (uint32_t)(t * cache_bs + grp * 4) : (uint32_t)(t * cache_bs * 2 + grp * 8);
     const uint32_t V_STEP = (FP8 ? 256u : 512u) << pshift;       // per blk
 
+    // PAD: chunk 4 m + grp of the 128-wide layout is real chunk c (first half) or Dr/16 + c - 8 (second half), if c % 8
+    // is below Dr/16; the others are read from chunk 0 and zeroed
+    uint32_t pk_off[PAD ? NM : 1];
+    bool pk_ok[PAD ? NM : 1];
+    if constexpr (PAD) {
+#pragma unroll
+        for (int m = 0; m < NM; ++m) {
+            const int c = 4 * m + grp;
+            pk_ok[m] = (c & 7) < CPr;
+            const int rc = pk_ok[m] ? (c < 8 ? c : CPr + c - 8) : 0;
+            pk_off[m] = FP8 ? (uint32_t)(((rc >> 1) * cache_bs + t) * 16 + (rc & 1) * 8) : (uint32_t)((rc * cache_bs + t) * 16);
+        }
+    }
     auto page_block = [&](int j) -> int {
         int jc = j < n_pages ? j : n_pages - 1;
         jc = jc < 0 ? 0 : jc;
@@ -174,7 +191,16 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
         const uint8_t *kb = kc_base + bt * kc_page_bytes + part * (BS * 16);
 #pragma unroll
         for (int m = 0; m < NM; ++m) {
-            if (FP8) {
+            if constexpr (PAD) {
+                uint4 w4;
+                if (FP8) {
+                    const uint2 w = *reinterpret_cast<const uint2 *>(kb + pk_off[m]);
+                    w4 = make_uint4(w.x, w.y, 0, 0);
+                } else {
+                    w4 = *reinterpret_cast<const uint4 *>(kb + pk_off[m]);
+                }
+                r.k[m] = pk_ok[m] ? w4 : make_uint4(0, 0, 0, 0);
+            } else if (FP8) {
                 const uint2 w = *reinterpret_cast<const uint2 *>(kb + k_off + m * K_STEP);
                 r.k[m] = make_uint4(w.x, w.y, 0, 0);
             } else {
@@ -192,8 +218,9 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
         const uint8_t *row = tab + (int64_t)pos * row_bytes;
 #pragma unroll
         for (int j = 0; j < NP; ++j) {
-            r.c[j].load(row, 32 * j + 8 * grp);
-            r.s[j].load(row, HALF + 32 * j + 8 * grp);
+            const int e = PAD && 32 * j + 8 * grp >= HALFr ? 0 : 32 * j + 8 * grp;   // (a padded chunk is zero: any angle will do)
+            r.c[j].load(row, e);
+            r.s[j].load(row, HALFr + e);
         }
     };
     auto load_values = [&](int j, ValRegs<HD> &r) {
@@ -202,8 +229,11 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
         const uint8_t *vb = vc_base + page_block(j) * vc_page_bytes + (jv & pshift) * (BS * CSZ);
 #pragma unroll
         for (int blk = 0; blk < NBLK; ++blk) {
-            if (FP8) r.v[blk] = make_uint2(*reinterpret_cast<const uint32_t *>(vb + v_off + blk * V_STEP), 0);
-            else r.v[blk] = *reinterpret_cast<const uint2 *>(vb + v_off + blk * V_STEP);
+            const uint32_t vo = v_off + (PAD && blk >= NBr ? 0 : blk) * V_STEP;      // rows 16 blk .. of V; past the head: zeros
+            uint2 w;
+            if (FP8) w = make_uint2(*reinterpret_cast<const uint32_t *>(vb + vo), 0);
+            else w = *reinterpret_cast<const uint2 *>(vb + vo);
+            r.v[blk] = PAD && blk >= NBr ? make_uint2(0, 0) : w;
         }
     };
     // rotate the pair (lo, hi) = (d, d + 64) in fp32, one rounding to bf16
@@ -235,7 +265,12 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
 #pragma unroll
         for (int m = 0; m < NM; ++m) {
             uint4 w = make_uint4(0, 0, 0, 0);
-            if (head_ok) w = *reinterpret_cast<const uint4 *>(qp + 32 * m);
+            if constexpr (PAD) {
+                const int c = 32 * m + 8 * grp, lo = c & 63;               // column of the 128-wide layout
+                if (head_ok && lo < HALFr) w = *reinterpret_cast<const uint4 *>(qp - 8 * grp + (c < 64 ? lo : HALFr + lo));
+            } else {
+                if (head_ok) w = *reinterpret_cast<const uint4 *>(qp + 32 * m);
+            }
             qf[m] = w;
         }
     }
@@ -331,9 +366,11 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     if (nsplit == 1) {
         T *op = (T *)p.o + qs * p.o_stride[0] + (int64_t)h * p.o_stride[1] + 4 * grp;
 #pragma unroll
-        for (int blk = 0; blk < NBLK; ++blk)
+        for (int blk = 0; blk < NBLK; ++blk) {
+            if (PAD && blk >= NBr) continue;
             *reinterpret_cast<uint2 *>(op + 16 * blk) =
                 make_uint2(E::pack(acc[blk][0] * inv, acc[blk][1] * inv), E::pack(acc[blk][2] * inv, acc[blk][3] * inv));
+        }
         return;
     }
     // partial of this slice: normalised O and log2-sum-exp, indexed by (slice, request, head)
@@ -355,6 +392,7 @@ struct DecodeMergeArgs {
     void *o;
     int64_t o_stride[2];
     int32_t batch, num_q_heads, index_bits;
+    int32_t head_dim;              // elements of an output row (below HD when the partial rows are padded)
 };
 template <typename T, int HD>
 __global__ void __launch_bounds__(256)
@@ -367,6 +405,7 @@ paged_decode_merge_kernel(const DecodeMergeArgs p, const int nsplit) {
     const int64_t qs = load_index(p.b_start_loc, b, p.index_bits);
     if (load_index(p.b_start_loc, b + 1, p.index_bits) - qs != 1) return;
     const int d = (threadIdx.x % LPR) * 4;
+    if (d >= p.head_dim) return;
     const float *wo = (const float *)p.workspace;
     const float *wl = wo + (int64_t)nsplit * p.batch * p.num_q_heads * D;
     const int64_t rows = (int64_t)p.batch * p.num_q_heads;
@@ -405,11 +444,15 @@ paged_decode_merge_kernel(const DecodeMergeArgs p, const int nsplit) {
 }
 
 // ------------------------------------------------------------------ host side
+// width of the lane layout and of a partial row: the head size, or 128 for the head sizes that are padded to it
+static int decode_tile_dim(const lazyattn_prefill_params &p) { return p.head_dim == 64 ? 64 : 128; }
+
 bool decode_mfma_supports(const lazyattn_prefill_params &p) {
     const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3;
     if ((p.dtype != LAZYATTN_BF16 && p.dtype != LAZYATTN_F16) || !(p.cache_dtype == p.dtype || fp8)) return false;
     if (p.table_dtype != p.dtype && p.table_dtype != LAZYATTN_F32) return false;
-    if ((p.head_dim != 128 && p.head_dim != 64) || p.rotary_dim != p.head_dim) return false;
+    // 128, 64, or a multiple of 16 below 128 (padded to 128)
+    if (p.head_dim < 16 || p.head_dim > 128 || p.head_dim % 16 || p.rotary_dim != p.head_dim) return false;
     if ((p.block_size != BS && p.block_size != 2 * BS) || p.x != (fp8 ? 16 : 8)) return false;
     if (p.pos_mode != LAZYATTN_POS_NATURAL && p.pos_mode != LAZYATTN_POS_BLOCK_UNIFORM) return false;
     if (p.q_stride[2] != 1 || p.o_stride[2] != 1) return false;
@@ -442,14 +485,14 @@ static int decode_splits(const lazyattn_prefill_params &p) {
 size_t decode_workspace_bytes(const lazyattn_prefill_params &p) {
     const int ns = decode_splits(p);
     if (ns <= 1) return 0;
-    return (size_t)ns * (size_t)p.batch * p.num_q_heads * (p.head_dim + 1) * sizeof(float);
+    return (size_t)ns * (size_t)p.batch * p.num_q_heads * (decode_tile_dim(p) + 1) * sizeof(float);
 }
 
 int launch_decode_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
     int nsplit = decode_splits(p);
     if (nsplit > 1) {
         // without room for the partials the call still runs, one slice per request and kv head
-        const size_t need = (size_t)nsplit * (size_t)p.batch * p.num_q_heads * (p.head_dim + 1) * sizeof(float);
+        const size_t need = (size_t)nsplit * (size_t)p.batch * p.num_q_heads * (decode_tile_dim(p) + 1) * sizeof(float);
         if (!p.workspace || (size_t)p.workspace_bytes < need || (((uintptr_t)p.workspace) & 15)) nsplit = 1;
     }
     const int phases = p.phases ? p.phases : LAZYATTN_PHASE_ALL;
@@ -458,24 +501,28 @@ int launch_decode_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
     if (phases & LAZYATTN_PHASE_MAIN) {
         const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3, t32 = p.table_dtype == LAZYATTN_F32;
         const dim3 grid(nblocks), block(WAVES * 64);
-        auto launch = [&](auto elem, auto hd) {
+        auto launch = [&](auto elem, auto hd, auto pad) {
             using T = decltype(elem);
             constexpr int HD = decltype(hd)::value;
-            if (fp8 && t32) hipLaunchKernelGGL((paged_decode_kernel<T, float, true, HD>), grid, block, 0, stream, p, nsplit);
-            else if (fp8) hipLaunchKernelGGL((paged_decode_kernel<T, T, true, HD>), grid, block, 0, stream, p, nsplit);
-            else if (t32) hipLaunchKernelGGL((paged_decode_kernel<T, float, false, HD>), grid, block, 0, stream, p, nsplit);
-            else hipLaunchKernelGGL((paged_decode_kernel<T, T, false, HD>), grid, block, 0, stream, p, nsplit);
+            constexpr bool PAD = decltype(pad)::value;
+            if (fp8 && t32) hipLaunchKernelGGL((paged_decode_kernel<T, float, true, HD, PAD>), grid, block, 0, stream, p, nsplit);
+            else if (fp8) hipLaunchKernelGGL((paged_decode_kernel<T, T, true, HD, PAD>), grid, block, 0, stream, p, nsplit);
+            else if (t32) hipLaunchKernelGGL((paged_decode_kernel<T, float, false, HD, PAD>), grid, block, 0, stream, p, nsplit);
+            else hipLaunchKernelGGL((paged_decode_kernel<T, T, false, HD, PAD>), grid, block, 0, stream, p, nsplit);
         };
         using hd128 = std::integral_constant<int, 128>;
         using hd64 = std::integral_constant<int, 64>;
-        if (p.head_dim == 64) { if (p.dtype == LAZYATTN_F16) launch(f16_t{}, hd64{}); else launch(bf16_t{}, hd64{}); }
-        else { if (p.dtype == LAZYATTN_F16) launch(f16_t{}, hd128{}); else launch(bf16_t{}, hd128{}); }
+        using yes = std::true_type;
+        using no = std::false_type;
+        if (p.head_dim == 64) { if (p.dtype == LAZYATTN_F16) launch(f16_t{}, hd64{}, no{}); else launch(bf16_t{}, hd64{}, no{}); }
+        else if (p.head_dim == 128) { if (p.dtype == LAZYATTN_F16) launch(f16_t{}, hd128{}, no{}); else launch(bf16_t{}, hd128{}, no{}); }
+        else { if (p.dtype == LAZYATTN_F16) launch(f16_t{}, hd128{}, yes{}); else launch(bf16_t{}, hd128{}, yes{}); }
         if (hipGetLastError() != hipSuccess) return LAZYATTN_E_LAUNCH;
     }
     if (nsplit > 1 && (phases & LAZYATTN_PHASE_COMBINE)) {
         const int64_t rows = (int64_t)p.batch * p.num_q_heads;
-        const DecodeMergeArgs m{p.workspace, p.b_start_loc, p.o, {p.o_stride[0], p.o_stride[1]}, p.batch, p.num_q_heads, p.index_bits};
-        const int rows_wg = 256 / (p.head_dim / 4);
+        const DecodeMergeArgs m{p.workspace, p.b_start_loc, p.o, {p.o_stride[0], p.o_stride[1]}, p.batch, p.num_q_heads, p.index_bits, p.head_dim};
+        const int rows_wg = 256 / (decode_tile_dim(p) / 4);
         const dim3 mgrid((unsigned)((rows + rows_wg - 1) / rows_wg));
         const bool f16 = p.dtype == LAZYATTN_F16;
         if (p.head_dim == 64) {

@@ -137,6 +137,22 @@ def test_decode_pages_of_32_slots(variant, dtype, kv, d):
     assert _err(got, ref) < (5e-2 if kv == "fp8" else 2e-2), _err(got, ref)
 
 
+@pytest.mark.parametrize("d", [96, 80, 112, 48, 16])
+@pytest.mark.parametrize("variant", ["natural", "block_uniform"])
+@pytest.mark.parametrize("dtype,kv,page", [(torch.bfloat16, "auto", 16), (torch.float16, "auto", 32), (torch.bfloat16, "fp8", 16)])
+def test_decode_head_sizes_padded_to_128(d, variant, dtype, kv, page):
+    """Head sizes that are multiples of 16 below 128 run the 128-wide kernel with the lane's chunks, the query and
+    the V rows zero-padded; forcing the fast kernel fails if it does not take them."""
+    print(f"case: decode head size {d} {variant} {dtype} kv={kv} page={page}", flush=True)
+    w = _decode_batch(variant, dtype=dtype, kv=kv, d=d, bs=page, seed=d)
+    lazy = torch.tensor([True, False, True, True, True]) if variant == "block_uniform" else None
+    for window in (0, 20):
+        ref = _oracle(w, lazy, sliding_window=window)
+        for nsplit in (0, 1, 3):
+            got = _run(w, lazy=lazy, num_splits=nsplit, sliding_window=window, kernel=_ffi.KERNEL_MFMA)
+            assert _err(got, ref) < (5e-2 if kv == "fp8" else 2e-2), (window, nsplit, _err(got, ref))
+
+
 @pytest.mark.parametrize("variant,table_f32", [("natural", False), ("block_uniform", True)])
 def test_decode_fp8_cache(variant, table_f32):
     print(f"case: decode fp8 {variant} table_f32={table_f32}", flush=True)
