@@ -84,9 +84,12 @@ def test_random_decode_batch(seed):
     q_lens = tuple(r.choice([1, 1, 1, 3]) for _ in range(5))
     nsplit = r.choice([0, 1, 2, 5, 9])
     page = r.choice([16, 16, 32])
+    d = r.choice([128, 128, 64, 96, 80, 48])
+    if r.random() < 0.2:
+        group = r.choice([24, 40, 64])        # above 16: several head blocks per kv head
     print(f"case: random decode seed={seed} hkv={hkv} group={group} {variant} kv={kv} q_lens={q_lens} nsplit={nsplit} "
-          f"page={page}", flush=True)
-    w = dec._decode_batch(variant, hq=hkv * group, hkv=hkv, q_lens=q_lens, seed=seed, kv=kv, bs=page)
+          f"page={page} d={d}", flush=True)
+    w = dec._decode_batch(variant, hq=hkv * group, hkv=hkv, q_lens=q_lens, seed=seed, kv=kv, bs=page, d=d)
     lazy = torch.tensor([(seed + b) % 4 != 0 for b in range(5)]) if variant == "block_uniform" else None
     ref = dec._oracle(w, lazy)
     got = dec._run(w, lazy=lazy, num_splits=nsplit)
