@@ -42,10 +42,15 @@ template <typename T> __device__ __forceinline__ void unpack8(const uint4 &w, fl
     f[4] = Elem<T>::lo(w.z); f[5] = Elem<T>::hi(w.z); f[6] = Elem<T>::lo(w.w); f[7] = Elem<T>::hi(w.w);
 }
 
-// 8 fp8 e4m3 bytes -> (float * scale) rounded to the query type, as floats
-template <typename T> __device__ __forceinline__ void unpack8_fp8(uint32_t lo, uint32_t hi, float scale, float *f) {
-    const f32x2_t a = __builtin_amdgcn_cvt_pk_f32_fp8(lo, false), b = __builtin_amdgcn_cvt_pk_f32_fp8(lo >> 16, false);
-    const f32x2_t c = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false), d = __builtin_amdgcn_cvt_pk_f32_fp8(hi >> 16, false);
+// two fp8 bytes (the low 16 bits of w) -> two floats; KIND 1: e4m3, 2: e5m2
+template <int KIND> __device__ __forceinline__ f32x2_t cvt_fp8x2(uint32_t w) {
+    if constexpr (KIND == 2) return __builtin_amdgcn_cvt_pk_f32_bf8(w, false);
+    else return __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
+}
+// 8 fp8 bytes -> (float * scale) rounded to the query type, as floats
+template <typename T, int KIND> __device__ __forceinline__ void unpack8_fp8(uint32_t lo, uint32_t hi, float scale, float *f) {
+    const f32x2_t a = cvt_fp8x2<KIND>(lo), b = cvt_fp8x2<KIND>(lo >> 16);
+    const f32x2_t c = cvt_fp8x2<KIND>(hi), d = cvt_fp8x2<KIND>(hi >> 16);
     const float t[8] = {a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
 #pragma unroll
     for (int i = 0; i < 8; ++i) f[i] = round_to<T>(t[i] * scale);
@@ -85,7 +90,7 @@ template <int HD> struct ValRegs {
 
 // PAD: the head size is a multiple of 16 below HD = 128; the lane's chunks, the query and the V rows are laid out as
 // for 128 with the two halves of the real head at (0 .., 64 ..) and zeros in between
-template <typename T, typename TT, bool FP8, int HD, bool PAD>
+template <typename T, typename TT, int FP8, int HD, bool PAD>
 __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2)))
 paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     using E = Elem<T>;
@@ -240,8 +245,8 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     auto rotate = [&](const uint4 &lo, const uint4 &hi, const Tab8<TT> &c, const Tab8<TT> &s, uint4 &xo, uint4 &yo) {
         float a[8], bb[8], cs[8], sn[8], x[8], y[8];
         if (FP8) {
-            unpack8_fp8<T>(lo.x, lo.y, k_scale, a);
-            unpack8_fp8<T>(hi.x, hi.y, k_scale, bb);
+            unpack8_fp8<T, FP8>(lo.x, lo.y, k_scale, a);
+            unpack8_fp8<T, FP8>(hi.x, hi.y, k_scale, bb);
         } else {
             unpack8<T>(lo, a);
             unpack8<T>(hi, bb);
@@ -298,7 +303,7 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     auto masked_v = [&](const ValRegs<HD> &r, int lim, int blk) -> uint2 {
         uint2 w = r.v[blk];
         if (FP8) {
-            const f32x2_t lo = __builtin_amdgcn_cvt_pk_f32_fp8(w.x, false), hi = __builtin_amdgcn_cvt_pk_f32_fp8(w.x >> 16, false);
+            const f32x2_t lo = cvt_fp8x2<FP8>(w.x), hi = cvt_fp8x2<FP8>(w.x >> 16);
             w = make_uint2(E::pack(lo[0] * v_scale, lo[1] * v_scale), E::pack(hi[0] * v_scale, hi[1] * v_scale));
         }
         if (lim < BS) {
@@ -448,7 +453,7 @@ paged_decode_merge_kernel(const DecodeMergeArgs p, const int nsplit) {
 static int decode_tile_dim(const lazyattn_prefill_params &p) { return p.head_dim == 64 ? 64 : 128; }
 
 bool decode_mfma_supports(const lazyattn_prefill_params &p) {
-    const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3;
+    const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3 || p.cache_dtype == LAZYATTN_FP8_E5M2;
     if ((p.dtype != LAZYATTN_BF16 && p.dtype != LAZYATTN_F16) || !(p.cache_dtype == p.dtype || fp8)) return false;
     if (p.table_dtype != p.dtype && p.table_dtype != LAZYATTN_F32) return false;
     // 128, 64, or a multiple of 16 below 128 (padded to 128)
@@ -499,16 +504,19 @@ int launch_decode_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
     const int64_t waves = (int64_t)p.batch * p.num_kv_heads * ((p.num_q_heads / p.num_kv_heads + 15) / 16) * nsplit;
     const unsigned nblocks = (unsigned)((waves + WAVES - 1) / WAVES);
     if (phases & LAZYATTN_PHASE_MAIN) {
-        const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3, t32 = p.table_dtype == LAZYATTN_F32;
+        const bool t32 = p.table_dtype == LAZYATTN_F32;
+        const int fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3 ? 1 : p.cache_dtype == LAZYATTN_FP8_E5M2 ? 2 : 0;   // kind of cache page
         const dim3 grid(nblocks), block(WAVES * 64);
         auto launch = [&](auto elem, auto hd, auto pad) {
             using T = decltype(elem);
             constexpr int HD = decltype(hd)::value;
             constexpr bool PAD = decltype(pad)::value;
-            if (fp8 && t32) hipLaunchKernelGGL((paged_decode_kernel<T, float, true, HD, PAD>), grid, block, 0, stream, p, nsplit);
-            else if (fp8) hipLaunchKernelGGL((paged_decode_kernel<T, T, true, HD, PAD>), grid, block, 0, stream, p, nsplit);
-            else if (t32) hipLaunchKernelGGL((paged_decode_kernel<T, float, false, HD, PAD>), grid, block, 0, stream, p, nsplit);
-            else hipLaunchKernelGGL((paged_decode_kernel<T, T, false, HD, PAD>), grid, block, 0, stream, p, nsplit);
+            if (fp8 == 1 && t32) hipLaunchKernelGGL((paged_decode_kernel<T, float, 1, HD, PAD>), grid, block, 0, stream, p, nsplit);
+            else if (fp8 == 1) hipLaunchKernelGGL((paged_decode_kernel<T, T, 1, HD, PAD>), grid, block, 0, stream, p, nsplit);
+            else if (fp8 == 2 && t32) hipLaunchKernelGGL((paged_decode_kernel<T, float, 2, HD, PAD>), grid, block, 0, stream, p, nsplit);
+            else if (fp8 == 2) hipLaunchKernelGGL((paged_decode_kernel<T, T, 2, HD, PAD>), grid, block, 0, stream, p, nsplit);
+            else if (t32) hipLaunchKernelGGL((paged_decode_kernel<T, float, 0, HD, PAD>), grid, block, 0, stream, p, nsplit);
+            else hipLaunchKernelGGL((paged_decode_kernel<T, T, 0, HD, PAD>), grid, block, 0, stream, p, nsplit);
         };
         using hd128 = std::integral_constant<int, 128>;
         using hd64 = std::integral_constant<int, 64>;

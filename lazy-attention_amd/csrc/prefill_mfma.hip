@@ -102,10 +102,15 @@ template <typename T> __device__ __forceinline__ void unpack8(const uint4 &w, fl
     f[0] = Elem<T>::lo(w.x); f[1] = Elem<T>::hi(w.x); f[2] = Elem<T>::lo(w.y); f[3] = Elem<T>::hi(w.y);
     f[4] = Elem<T>::lo(w.z); f[5] = Elem<T>::hi(w.z); f[6] = Elem<T>::lo(w.w); f[7] = Elem<T>::hi(w.w);
 }
-// 8 fp8 e4m3 bytes -> (float * scale) rounded to the query type, as floats  (old_ops:239-241)
-template <typename T> __device__ __forceinline__ void unpack8_fp8(uint32_t lo, uint32_t hi, float scale, float *f) {
-    const f32x2_t a = __builtin_amdgcn_cvt_pk_f32_fp8(lo, false), b = __builtin_amdgcn_cvt_pk_f32_fp8(lo >> 16, false);
-    const f32x2_t c = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false), d = __builtin_amdgcn_cvt_pk_f32_fp8(hi >> 16, false);
+// two fp8 bytes (the low 16 bits of w) -> two floats; KIND 1: e4m3, 2: e5m2
+template <int KIND> __device__ __forceinline__ f32x2_t cvt_fp8x2(uint32_t w) {
+    if constexpr (KIND == 2) return __builtin_amdgcn_cvt_pk_f32_bf8(w, false);
+    else return __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
+}
+// 8 fp8 bytes -> (float * scale) rounded to the query type, as floats  (old_ops:239-241)
+template <typename T, int KIND> __device__ __forceinline__ void unpack8_fp8(uint32_t lo, uint32_t hi, float scale, float *f) {
+    const f32x2_t a = cvt_fp8x2<KIND>(lo), b = cvt_fp8x2<KIND>(lo >> 16);
+    const f32x2_t c = cvt_fp8x2<KIND>(hi), d = cvt_fp8x2<KIND>(hi >> 16);
     const float t[8] = {a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
 #pragma unroll
     for (int i = 0; i < 8; ++i) f[i] = round_to<T>(t[i] * scale);
@@ -133,7 +138,7 @@ template <int HD> constexpr int lds_bytes(int nc) { return Geo<HD>::KV_BYTES + n
 // WIN: built with the sliding-window code (calls without a window run the instantiation without it)
 // PAD: the head size is a multiple of 16 below HD = 128: Q, K and V sit zero-padded in the 128-wide tiles, the two
 // halves of the real head at (0 .., 64 ..) so that the rotation pairs stay (d, 64 + d)
-template <int NC, int HD, bool FP8, bool WIN, bool PAD, typename T, typename TT>
+template <int NC, int HD, int FP8, bool WIN, bool PAD, typename T, typename TT>
 __global__ void __launch_bounds__((NC + 4) * 64)
 prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int n_mt, const int mt_total) {
     using G = Geo<HD>;
@@ -493,8 +498,8 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             for (int i = 0; i < KI; ++i) {
                 float a[8], bb[8], cs[8], sn[8];
                 if (FP8 && kind != TILE_NEW) {
-                    unpack8_fp8<T>(kr[i].k1.x, kr[i].k1.y, k_scale, a);
-                    unpack8_fp8<T>(kr[i].k2.x, kr[i].k2.y, k_scale, bb);
+                    unpack8_fp8<T, FP8>(kr[i].k1.x, kr[i].k1.y, k_scale, a);
+                    unpack8_fp8<T, FP8>(kr[i].k2.x, kr[i].k2.y, k_scale, bb);
                 } else {
                     unpack8<T>(kr[i].k1, a);
                     unpack8<T>(kr[i].k2, bb);
@@ -542,8 +547,8 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                     uint32_t o2[4][2];
 #pragma unroll
                     for (int q4 = 0; q4 < 4; ++q4) {
-                        const f32x2_t lo = __builtin_amdgcn_cvt_pk_f32_fp8(w[q4], false);
-                        const f32x2_t hi = __builtin_amdgcn_cvt_pk_f32_fp8(w[q4] >> 16, false);
+                        const f32x2_t lo = cvt_fp8x2<FP8>(w[q4]);
+                        const f32x2_t hi = cvt_fp8x2<FP8>(w[q4] >> 16);
                         float f[4] = {lo[0] * v_scale, lo[1] * v_scale, hi[0] * v_scale, hi[1] * v_scale};
                         if (kind == TILE_EDGE) {
 #pragma unroll
@@ -1037,7 +1042,7 @@ static int mfma_splits(const lazyattn_prefill_params &p, int nw) {
 }
 
 bool mfma_supports(const lazyattn_prefill_params &p) {
-    const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3;
+    const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3 || p.cache_dtype == LAZYATTN_FP8_E5M2;
     if (p.dtype != LAZYATTN_BF16 && p.dtype != LAZYATTN_F16) return false;
     if (!(p.cache_dtype == p.dtype || fp8)) return false;
     if (p.table_dtype != p.dtype && p.table_dtype != LAZYATTN_F32) return false;
@@ -1066,7 +1071,7 @@ size_t mfma_workspace_bytes(const lazyattn_prefill_params &p) {
     return (size_t)ns * (size_t)p.num_tokens * p.num_q_heads * partial_row_bytes(p);
 }
 
-template <int NC, int HD, bool FP8, bool WIN, bool PAD, typename T, typename TT>
+template <int NC, int HD, int FP8, bool WIN, bool PAD, typename T, typename TT>
 static int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt, int mt_total, hipStream_t stream) {
     auto kern = prefill_mfma_kernel<NC, HD, FP8, WIN, PAD, T, TT>;
     constexpr int LDS_BYTES = lds_bytes<HD>(NC);
@@ -1087,12 +1092,16 @@ static int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt,
 
 template <int NC, int HD, bool WIN, bool PAD, typename T>
 static int launch_mfma_hd(const lazyattn_prefill_params &p, int nsplit, int n_mt, int mt_total, hipStream_t stream) {
-    const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3;
     const bool t32 = p.table_dtype == LAZYATTN_F32;
-    if (fp8) return t32 ? launch_mfma_t<NC, HD, true, WIN, PAD, T, float>(p, nsplit, n_mt, mt_total, stream)
-                        : launch_mfma_t<NC, HD, true, WIN, PAD, T, T>(p, nsplit, n_mt, mt_total, stream);
-    return t32 ? launch_mfma_t<NC, HD, false, WIN, PAD, T, float>(p, nsplit, n_mt, mt_total, stream)
-               : launch_mfma_t<NC, HD, false, WIN, PAD, T, T>(p, nsplit, n_mt, mt_total, stream);
+    // cache pages: 0 the element type, 1 fp8 e4m3, 2 fp8 e5m2
+    if (p.cache_dtype == LAZYATTN_FP8_E4M3)
+        return t32 ? launch_mfma_t<NC, HD, 1, WIN, PAD, T, float>(p, nsplit, n_mt, mt_total, stream)
+                   : launch_mfma_t<NC, HD, 1, WIN, PAD, T, T>(p, nsplit, n_mt, mt_total, stream);
+    if (p.cache_dtype == LAZYATTN_FP8_E5M2)
+        return t32 ? launch_mfma_t<NC, HD, 2, WIN, PAD, T, float>(p, nsplit, n_mt, mt_total, stream)
+                   : launch_mfma_t<NC, HD, 2, WIN, PAD, T, T>(p, nsplit, n_mt, mt_total, stream);
+    return t32 ? launch_mfma_t<NC, HD, 0, WIN, PAD, T, float>(p, nsplit, n_mt, mt_total, stream)
+               : launch_mfma_t<NC, HD, 0, WIN, PAD, T, T>(p, nsplit, n_mt, mt_total, stream);
 }
 template <int NC, typename T>
 static int launch_mfma_nc(const lazyattn_prefill_params &p, int nsplit, int n_mt, int mt_total, hipStream_t stream) {

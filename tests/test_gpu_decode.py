@@ -153,6 +153,27 @@ def test_decode_head_sizes_padded_to_128(d, variant, dtype, kv, page):
             assert _err(got, ref) < (5e-2 if kv == "fp8" else 2e-2), (window, nsplit, _err(got, ref))
 
 
+@pytest.mark.parametrize("d,page", [(128, 16), (64, 32), (96, 16)])
+@pytest.mark.parametrize("variant", ["natural", "block_uniform"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_decode_fp8_e5m2_cache(d, page, variant, dtype):
+    """kv_cache_dtype "fp8_e5m2" (ops/chunked_prefill_paged_decode.py:123-124) on the fast kernel: the e4m3 bytes of
+    the batch read as e5m2, exponents kept below inf/NaN; outputs reach 14, so one unit in the last place is allowed."""
+    print(f"case: decode fp8_e5m2 d={d} page={page} {variant} {dtype}", flush=True)
+    w = _decode_batch(variant, dtype=dtype, kv="fp8", d=d, bs=page, seed=d)
+    w.kv_cache_dtype = "fp8_e5m2"
+    w.k_cache &= 0x7B
+    w.v_cache &= 0x7B
+    w.k_scale = torch.tensor(2.0 ** -12)
+    w.v_scale = torch.tensor(2.0 ** -12)
+    lazy = torch.tensor([True, False, True, True, True]) if variant == "block_uniform" else None
+    ref = _oracle(w, lazy).float()
+    for nsplit in (0, 1, 3):
+        got = _run(w, lazy=lazy, num_splits=nsplit, kernel=_ffi.KERNEL_MFMA).float()
+        e = ((got.cpu() - ref).abs() - 2.0 ** -7 * ref.abs()).clamp(min=0).max().item()
+        assert e < 5e-2, (nsplit, e)
+
+
 @pytest.mark.parametrize("variant,table_f32", [("natural", False), ("block_uniform", True)])
 def test_decode_fp8_cache(variant, table_f32):
     print(f"case: decode fp8 {variant} table_f32={table_f32}", flush=True)

@@ -223,6 +223,33 @@ def test_mfma_head_sizes_padded_to_128(d, variant, dtype, kv, page):
             assert e < tol, (window, nsplit, e)
 
 
+def _as_e5m2(w):
+    """The e4m3 bytes of a workload read as e5m2 (exponents kept below inf/NaN, scales to match): still a valid cache."""
+    w.kv_cache_dtype = "fp8_e5m2"
+    w.k_cache &= 0x7B
+    w.v_cache &= 0x7B
+    w.k_scale = torch.tensor(2.0 ** -12)
+    w.v_scale = torch.tensor(2.0 ** -12)
+    return w
+
+
+@pytest.mark.parametrize("d,page", [(128, 16), (64, 32), (96, 16)])
+@pytest.mark.parametrize("variant", ["natural", "offset", "block_uniform"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_mfma_fp8_e5m2_cache(d, page, variant, dtype):
+    """kv_cache_dtype "fp8_e5m2" (ops/prefix_prefill.py:643-644): the second fp8 format the entry points accept.
+    The outputs reach 14 here, so the bound allows one unit in the last place of the reference."""
+    print(f"case: mfma fp8_e5m2 d={d} page={page} {variant} {dtype}", flush=True)
+    w = _as_e5m2(wl.make_workload("e5m2", dtype=dtype, hq=32, hkv=8, d=d, theta=500000.0, block_size=page,
+                                  doc_lens=[100, 16, 333, 70, 5, 250], requests=[[3, 1, 0], [2], [0, 2, 3, 1, 5], [4], []],
+                                  q_lens=[70, 1, 9, 33, 130], variant=variant, kv_cache_dtype="fp8", seed=d))
+    ref = run_oracle(w).float()
+    for nsplit, kernel in ((1, _ffi.KERNEL_MFMA4), (3, _ffi.KERNEL_MFMA8)):
+        got = run_op(w.to(DEV), kernel=kernel, num_splits=nsplit).cpu().float()
+        e = ((got - ref).abs() - 2.0 ** -7 * ref.abs()).clamp(min=0).max().item()
+        assert e < 5e-2, (nsplit, e)
+
+
 def test_mfma_takes_views_of_a_packed_qkv_tensor():
     """vLLM hands q, k, v as views of one [T, (Hq + 2 Hkv) D] projection output and writes o into a wider buffer:
     token strides larger than the row, the matrix path must take them as they are."""
