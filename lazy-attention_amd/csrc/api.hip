@@ -122,7 +122,7 @@ extern "C" int lazyattn_rope_and_cache_write(const lazyattn_rope_write_params *p
         (p->table_stride % (p->table_dtype == LAZYATTN_F32 ? 4 : 8) || ((uintptr_t)p->cos_sin_cache & 15)))
         return LAZYATTN_E_UNSUPPORTED;
     if (write) {
-        const bool fp8 = p->cache_dtype == LAZYATTN_FP8_E4M3;
+        const bool fp8 = p->cache_dtype == LAZYATTN_FP8_E4M3 || p->cache_dtype == LAZYATTN_FP8_E5M2;
         if (!fp8 && p->cache_dtype != p->dtype) return LAZYATTN_E_DTYPE;
         if (fp8 && (!p->k_scale || !p->v_scale)) return LAZYATTN_E_NULL;
         if (p->slot_bits != 32 && p->slot_bits != 64) return LAZYATTN_E_DTYPE;

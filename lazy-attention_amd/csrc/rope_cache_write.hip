@@ -22,11 +22,12 @@ namespace {
 
 typedef __attribute__((ext_vector_type(2))) float f32x2_t;
 
-// value / scale -> e4m3, saturating (|x| <= 448), round to nearest even
-__device__ __forceinline__ uint8_t to_fp8_e4m3(float x, float inv_scale) {
+// value / scale -> fp8, saturating, round to nearest even; KIND 1: e4m3 (|x| <= 448), 2: e5m2 (|x| <= 57344)
+template <int KIND> __device__ __forceinline__ uint8_t to_fp8(float x, float inv_scale) {
     float y = x * inv_scale;
-    y = fminf(fmaxf(y, -448.f), 448.f);
-    const int w = __builtin_amdgcn_cvt_pk_fp8_f32(y, y, 0, false);
+    const float top = KIND == 2 ? 57344.f : 448.f;
+    y = fminf(fmaxf(y, -top), top);
+    const int w = KIND == 2 ? __builtin_amdgcn_cvt_pk_bf8_f32(y, y, 0, false) : __builtin_amdgcn_cvt_pk_fp8_f32(y, y, 0, false);
     return (uint8_t)(w & 0xff);
 }
 
@@ -39,7 +40,7 @@ __device__ __forceinline__ uint8_t to_fp8_e4m3(float x, float inv_scale) {
 // page in order (the usual case: a prefill chunk is written page by page; pages of 16, 32, ... slots) the
 // column is one 32-byte store, otherwise the item falls back to one store per token.
 constexpr int RUN = 16;
-template <typename T, typename TT, bool FP8>
+template <typename T, typename TT, int FP8>
 __global__ void __launch_bounds__(256)
 rope_cache_write_kernel(const lazyattn_rope_write_params p) {
     const int D = p.head_dim, R = p.rotary_dim, HALF = R / 2;
@@ -77,7 +78,7 @@ rope_cache_write_kernel(const lazyattn_rope_write_params p) {
             if (FP8) {
                 __attribute__((aligned(16))) uint8_t b[RUN];
 #pragma unroll
-                for (int i = 0; i < RUN; ++i) b[i] = to_fp8_e4m3(to_f32(src[i * p.v_stride[0]]), v_inv);
+                for (int i = 0; i < RUN; ++i) b[i] = to_fp8<FP8 ? FP8 : 1>(to_f32(src[i * p.v_stride[0]]), v_inv);
                 *reinterpret_cast<uint4 *>(dst) = *reinterpret_cast<const uint4 *>(b);
             } else {
                 __attribute__((aligned(16))) T col[RUN];
@@ -99,7 +100,7 @@ rope_cache_write_kernel(const lazyattn_rope_write_params p) {
             if (sl < 0) continue;
             const int64_t o0 = (sl / p.block_size) * p.vc_stride[0] + (int64_t)h * p.vc_stride[1] + (int64_t)d * p.vc_stride[2] +
                                (sl % p.block_size) * p.vc_stride[3];
-            if (FP8) ((uint8_t *)p.v_cache)[o0] = to_fp8_e4m3(to_f32(src[i * p.v_stride[0]]), v_inv);
+            if (FP8) ((uint8_t *)p.v_cache)[o0] = to_fp8<FP8 ? FP8 : 1>(to_f32(src[i * p.v_stride[0]]), v_inv);
             else ((T *)p.v_cache)[o0] = src[i * p.v_stride[0]];
         }
         return;
@@ -121,7 +122,7 @@ rope_cache_write_kernel(const lazyattn_rope_write_params p) {
         if (FP8) {
             uint8_t b[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) b[i] = to_fp8_e4m3(f[i], k_inv);
+            for (int i = 0; i < 8; ++i) b[i] = to_fp8<FP8 ? FP8 : 1>(f[i], k_inv);
             *reinterpret_cast<uint2 *>(dst) = *reinterpret_cast<const uint2 *>(b);
         } else if (p.x % 8 == 0) {
             raw.store(reinterpret_cast<T *>(dst));
@@ -198,9 +199,11 @@ rope_cache_write_kernel(const lazyattn_rope_write_params p) {
 template <typename T, typename TT>
 int launch_rw_cache(const lazyattn_rope_write_params &p, dim3 grid, hipStream_t stream) {
     if (p.cache_dtype == LAZYATTN_FP8_E4M3)
-        hipLaunchKernelGGL((rope_cache_write_kernel<T, TT, true>), grid, dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((rope_cache_write_kernel<T, TT, 1>), grid, dim3(256), 0, stream, p);
+    else if (p.cache_dtype == LAZYATTN_FP8_E5M2)
+        hipLaunchKernelGGL((rope_cache_write_kernel<T, TT, 2>), grid, dim3(256), 0, stream, p);
     else
-        hipLaunchKernelGGL((rope_cache_write_kernel<T, TT, false>), grid, dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((rope_cache_write_kernel<T, TT, 0>), grid, dim3(256), 0, stream, p);
     return hipGetLastError() == hipSuccess ? LAZYATTN_OK : LAZYATTN_E_LAUNCH;
 }
 

@@ -19,6 +19,8 @@ from ... import _ffi
 def _cache_code(kv_cache_dtype: str, dtype: torch.dtype) -> int:
     if kv_cache_dtype in ("fp8", "fp8_e4m3"):
         return _ffi.FP8_E4M3
+    if kv_cache_dtype == "fp8_e5m2":
+        return _ffi.FP8_E5M2
     if kv_cache_dtype == "auto":
         return _ffi.dtype_code(dtype)
     raise NotImplementedError(f"kv_cache_dtype {kv_cache_dtype!r} is not supported by the cache write")
@@ -83,7 +85,7 @@ def rotate_and_write(positions: Optional[torch.Tensor], query: Optional[torch.Te
         p.slot_mapping = slot_mapping.data_ptr()
         p.slot_bits = 64 if slot_mapping.dtype == torch.int64 else 32
         p.cache_dtype = code
-        if code == _ffi.FP8_E4M3:
+        if code in (_ffi.FP8_E4M3, _ffi.FP8_E5M2):
             ks = torch.as_tensor(k_scale, dtype=torch.float32, device=dev).reshape(1)
             vs = torch.as_tensor(v_scale, dtype=torch.float32, device=dev).reshape(1)
             keep += [ks, vs]

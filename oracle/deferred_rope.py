@@ -361,13 +361,15 @@ def rotary_new_tokens(positions, query, key, table, *, q_only: bool, compute_dty
 def paged_cache_write(key, value, k_cache, v_cache, slot_mapping, kv_cache_dtype="auto", k_scale=1.0, v_scale=1.0):
     """In place: token t -> slot_mapping[t] = block*BS + offset (negative: skipped);
     K[block, h, d // x, offset, d % x] = key[t, h, d]; V[block, h, d, offset] = value[t, h, d];
-    fp8 caches (uint8 storage) hold (value / scale) saturated to +-448 as e4m3."""
+    fp8 caches (uint8 storage) hold (value / scale) saturated to +-448 as e4m3, or to +-57344 as e5m2."""
     nb, hkv, dx, bs, x = k_cache.shape
     fp8 = "fp8" in kv_cache_dtype
 
     def enc(t, scale):
         if not fp8:
             return t.to(k_cache.dtype)
+        if kv_cache_dtype == "fp8_e5m2":
+            return (t.float() / float(scale)).clamp(-57344.0, 57344.0).to(torch.float8_e5m2).view(torch.uint8)
         return (t.float() / float(scale)).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8)
     for t in range(key.shape[0]):
         slot = int(slot_mapping[t])

@@ -71,21 +71,22 @@ def test_reference_call_sites_separately():
     assert torch.equal(kcg.cpu(), kc_ref) and torch.equal(vcg.cpu(), vc_ref)
 
 
-def test_fp8_quantise_on_write():
-    print("case: fp8 cache write", flush=True)
+@pytest.mark.parametrize("kv,top,f8", [("fp8", 448.0, torch.float8_e4m3fn), ("fp8_e5m2", 57344.0, torch.float8_e5m2)])
+def test_fp8_quantise_on_write(kv, top, f8):
+    print(f"case: {kv} cache write", flush=True)
     dtype, d = torch.bfloat16, 128
     table, q, k, v, pos, slots, kc, vc = _case(dtype, d, 8, 2, 64, fp8=True, seed=9)
     k = k * 3.0
-    ks, vs = float(k.abs().max() / 200.0), float(v.abs().max() / 448.0)      # K saturates on purpose
+    ks, vs = float(k.abs().max() / (top * 2.0)), float(v.abs().max() / top)       # K saturates on purpose
     kc_ref, vc_ref = kc.clone(), vc.clone()
-    orc.paged_cache_write(k, v, kc_ref, vc_ref, slots, "fp8", ks, vs)
+    orc.paged_cache_write(k, v, kc_ref, vc_ref, slots, kv, ks, vs)
     kg, vg, kcg, vcg = (a.to(DEV) for a in (k, v, kc, vc))
-    rope.write_to_paged_cache(kg, vg, kcg, vcg, slots.to(DEV), "fp8", ks, vs)
-    a = kcg.cpu().view(torch.float8_e4m3fn).float(); b = kc_ref.view(torch.float8_e4m3fn).float()
-    assert not torch.isnan(a).any()
-    # same e4m3 code except where value/scale sits on a rounding boundary of the division
-    assert (a != b).float().mean() < 1e-3 and (a - b).abs().max() <= 32.0
-    a = vcg.cpu().view(torch.float8_e4m3fn).float(); b = vc_ref.view(torch.float8_e4m3fn).float()
+    rope.write_to_paged_cache(kg, vg, kcg, vcg, slots.to(DEV), kv, ks, vs)
+    a = kcg.cpu().view(f8).float(); b = kc_ref.view(f8).float()
+    assert torch.isfinite(a).all() and a.abs().max() == top
+    # same code except where value/scale sits on a rounding boundary of the division: one step at most
+    assert (a != b).float().mean() < 1e-3 and ((a - b).abs() <= 0.26 * b.abs()).all()
+    a = vcg.cpu().view(f8).float(); b = vc_ref.view(f8).float()
     assert (a != b).float().mean() < 1e-3
 
 
