@@ -393,6 +393,21 @@ def test_paged_cache_write_is_inverse_of_gather_and_matches_layout_formula():
     assert torch.equal(kb, k) and torch.equal(vb, v)
 
 
+@pytest.mark.parametrize("kv,top,step_at_1", [("fp8", 448.0, 0.125), ("fp8_e5m2", 57344.0, 0.25)])
+def test_paged_cache_write_fp8_codes(kv, top, step_at_1):
+    """value / scale saturated to the format's largest finite number, nearest-even: exact values, a tie, the
+    saturation and the byte codes of 1.0 (0x38 in e4m3, 0x3C in e5m2) fixed by the formats themselves."""
+    f8 = torch.float8_e4m3fn if kv == "fp8" else torch.float8_e5m2
+    vals = torch.tensor([1.0, -2.0, 1.0 + step_at_1 / 2, 1e9, -1e9, 0.0, 3.0, 0.5])
+    k = (vals * 0.5).view(8, 1, 1).expand(8, 1, 16).contiguous()       # scale 0.5: stored value = vals
+    kc = torch.zeros(1, 1, 1, 8, 16, dtype=torch.uint8); vc = torch.zeros(1, 1, 16, 8, dtype=torch.uint8)
+    orc.paged_cache_write(k, k, kc, vc, torch.arange(8), kv, 0.5, 0.5)
+    got = kc.view(f8).float()[0, 0, 0, :, 0]
+    assert got.tolist() == [1.0, -2.0, 1.0, top, -top, 0.0, 3.0, 0.5]     # the tie goes to the even code
+    assert int(kc[0, 0, 0, 0, 0]) == (0x38 if kv == "fp8" else 0x3C)
+    assert torch.equal(vc.view(f8).float()[0, 0, 0, :], got)
+
+
 def test_rotary_new_tokens_q_only_leaves_key_and_preserves_norm():
     g = torch.Generator().manual_seed(2)
     table = orc.build_cos_sin_table(512, 32, 10000.0)
