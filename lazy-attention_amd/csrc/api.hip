@@ -129,6 +129,8 @@ extern "C" int lazyattn_rope_and_cache_write(const lazyattn_rope_write_params *p
         if (p->block_size <= 0 || p->x <= 0 || p->head_dim % p->x) return LAZYATTN_E_SHAPE;
         if (p->v_stride[0] % vec || p->v_stride[1] % vec || ((uintptr_t)p->v & 15)) return LAZYATTN_E_UNSUPPORTED;
         if (p->kc_stride[4] != 1) return LAZYATTN_E_UNSUPPORTED;
+        // an fp8 K chunk is written as one 8-byte store: the innermost cache axis must hold whole chunks
+        if (fp8 && p->x % 8) return LAZYATTN_E_UNSUPPORTED;
         // a K chunk of 8 elements is one store when x is a multiple of 8 (16-byte aligned for 2-byte types,
         // 8-byte aligned for fp8); x = 4 (fp32 caches) is written element-wise
         if (p->x % 8 == 0 &&

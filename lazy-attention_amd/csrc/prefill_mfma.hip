@@ -893,12 +893,13 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
 // The few fields the merge needs, not the whole parameter block: a launch with ~450 bytes of kernel
 // arguments costs about a microsecond more than one with 64 on this part.
 struct MergeArgs {
-    const void *workspace, *b_start_loc;
+    const void *workspace, *b_start_loc, *b_seq_len;
     void *o;
     int64_t o_stride[2];
     int32_t num_tokens, num_q_heads, index_bits, skip_decode;
     int32_t batch, token_grid;      // token_grid: rows are numbered over all tokens instead of per request
     int32_t head_dim;               // elements of an output row (below HD when the partial rows are padded)
+    int32_t group, unit_cap;        // q-heads per kv-head; 32-row units per (request, kv-head) the main grid covers
 };
 // NB = splits taken per batch of loads: 2, 4 or 8, the smallest that covers nsplit (more only when nsplit > 8)
 template <typename T, int HD, int NB>
@@ -908,27 +909,33 @@ prefill_combine_kernel(const MergeArgs p, const int nsplit) {
     constexpr int D = HD, LPR = HD / 8;                       // lanes per row (8 elements = one 16-byte load each)
     const int64_t r = (int64_t)blockIdx.x * (256 / LPR) + threadIdx.x / LPR;
     int64_t tok;
+    int b;
     if (p.token_grid) {
         // Rows over all tokens of the call: no workgroup is launched for rows a request does not have (a grid
         // of batch x longest request is mostly empty when one long request sits among one-token requests).
-        // Only the skipping of one-token requests needs the row's request: a binary search of the offsets.
+        // The row's request is found by a binary search of the offsets.
         tok = r / p.num_q_heads;
         if (tok >= load_index(p.b_start_loc, p.batch, p.index_bits)) return;
-        if (p.skip_decode) {
-            int lo = 0, hi = p.batch;                         // offsets[lo] <= tok < offsets[hi]
-            while (hi - lo > 1) {
-                const int mid = (lo + hi) >> 1;
-                if (load_index(p.b_start_loc, mid, p.index_bits) <= tok) lo = mid; else hi = mid;
-            }
-            if (load_index(p.b_start_loc, lo + 1, p.index_bits) - load_index(p.b_start_loc, lo, p.index_bits) == 1) return;
+        int lo = 0, hi = p.batch;                             // offsets[lo] <= tok < offsets[hi]
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (load_index(p.b_start_loc, mid, p.index_bits) <= tok) lo = mid; else hi = mid;
         }
+        b = lo;
     } else {
-        const int b = blockIdx.y;
+        b = blockIdx.y;
+        tok = load_index(p.b_start_loc, b, p.index_bits) + r / p.num_q_heads;
+    }
+    // Exactly the rows the main kernel wrote partials for: anything else would merge whatever an earlier call
+    // left in the workspace.
+    {
         const int64_t qs = load_index(p.b_start_loc, b, p.index_bits);
         const int64_t q_len = load_index(p.b_start_loc, b + 1, p.index_bits) - qs;
+        const int64_t row = tok - qs;
         if (q_len <= 0 || (p.skip_decode && q_len == 1)) return;
-        if (r >= q_len * p.num_q_heads) return;
-        tok = qs + r / p.num_q_heads;
+        if (row >= q_len) return;
+        if ((row / UNIT) * p.group + (r % p.num_q_heads) % p.group >= p.unit_cap) return;   // past the grid sized by max_q_len
+        if (load_index(p.b_seq_len, b, p.index_bits) - q_len < 0) return;
     }
     const int h = (int)(r % p.num_q_heads);
     const int d = (threadIdx.x % LPR) * 8;
@@ -1136,8 +1143,9 @@ int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
         // rows per request x requests, or rows over all tokens when that is at most half as many
         const int token_grid = p.batch > 1 && 2 * (int64_t)p.num_tokens <= (int64_t)p.batch * p.max_q_len;
         const int64_t rows = (int64_t)(token_grid ? p.num_tokens : p.max_q_len) * p.num_q_heads;
-        const MergeArgs m{p.workspace, p.b_start_loc, p.o, {p.o_stride[0], p.o_stride[1]}, p.num_tokens, p.num_q_heads,
-                          p.index_bits, p.skip_decode, p.batch, token_grid, p.head_dim};
+        const MergeArgs m{p.workspace, p.b_start_loc, p.b_seq_len, p.o, {p.o_stride[0], p.o_stride[1]}, p.num_tokens, p.num_q_heads,
+                          p.index_bits, p.skip_decode, p.batch, token_grid, p.head_dim, p.num_q_heads / p.num_kv_heads,
+                          mt_total > 0 ? 0x7fffffff : n_mt * nw};
         const int rows_wg = 256 / (tile_dim(p) / 8);
         const dim3 grid((unsigned)((rows + rows_wg - 1) / rows_wg), token_grid ? 1 : p.batch);
         const bool f16 = p.dtype == LAZYATTN_F16;

@@ -22,11 +22,13 @@ namespace {
 
 typedef __attribute__((ext_vector_type(2))) float f32x2_t;
 
-// value / scale -> fp8, saturating, round to nearest even; KIND 1: e4m3 (|x| <= 448), 2: e5m2 (|x| <= 57344)
-template <int KIND> __device__ __forceinline__ uint8_t to_fp8(float x, float inv_scale) {
-    float y = x * inv_scale;
+// value / scale -> fp8, saturating, round to nearest even; KIND 1: e4m3 (|x| <= 448), 2: e5m2 (|x| <= 57344).
+// A true division (IEEE, as the writer it replaces does: a product with the reciprocal differs in the last
+// place for about one value in a thousand); the clamp is NaN-propagating, so a NaN stays a NaN code.
+template <int KIND> __device__ __forceinline__ uint8_t to_fp8(float x, float scale) {
+    float y = __fdiv_rn(x, scale);
     const float top = KIND == 2 ? 57344.f : 448.f;
-    y = fminf(fmaxf(y, -top), top);
+    y = __builtin_elementwise_minimum(__builtin_elementwise_maximum(y, -top), top);
     const int w = KIND == 2 ? __builtin_amdgcn_cvt_pk_bf8_f32(y, y, 0, false) : __builtin_amdgcn_cvt_pk_fp8_f32(y, y, 0, false);
     return (uint8_t)(w & 0xff);
 }
@@ -65,7 +67,7 @@ rope_cache_write_kernel(const lazyattn_rope_write_params p) {
         const int h = (int)(vi % per_run) / D, d = (int)(vi % per_run) % D;
         const int64_t t0 = run * RUN;
         const int n = p.num_tokens - t0 < RUN ? (int)(p.num_tokens - t0) : RUN;
-        const float v_inv = FP8 ? 1.f / *p.v_scale : 1.f;
+        const float v_div = FP8 ? *p.v_scale : 1.f;
         const T *src = (const T *)p.v + t0 * p.v_stride[0] + (int64_t)h * p.v_stride[1] + d;
         const int64_t s0 = slot_of(t0);
         bool page = n == RUN && p.block_size % RUN == 0 && s0 >= 0 && s0 % RUN == 0 && p.vc_stride[3] == 1 &&
@@ -78,7 +80,7 @@ rope_cache_write_kernel(const lazyattn_rope_write_params p) {
             if (FP8) {
                 __attribute__((aligned(16))) uint8_t b[RUN];
 #pragma unroll
-                for (int i = 0; i < RUN; ++i) b[i] = to_fp8<FP8 ? FP8 : 1>(to_f32(src[i * p.v_stride[0]]), v_inv);
+                for (int i = 0; i < RUN; ++i) b[i] = to_fp8<FP8 ? FP8 : 1>(to_f32(src[i * p.v_stride[0]]), v_div);
                 *reinterpret_cast<uint4 *>(dst) = *reinterpret_cast<const uint4 *>(b);
             } else {
                 __attribute__((aligned(16))) T col[RUN];
@@ -100,7 +102,7 @@ rope_cache_write_kernel(const lazyattn_rope_write_params p) {
             if (sl < 0) continue;
             const int64_t o0 = (sl / p.block_size) * p.vc_stride[0] + (int64_t)h * p.vc_stride[1] + (int64_t)d * p.vc_stride[2] +
                                (sl % p.block_size) * p.vc_stride[3];
-            if (FP8) ((uint8_t *)p.v_cache)[o0] = to_fp8<FP8 ? FP8 : 1>(to_f32(src[i * p.v_stride[0]]), v_inv);
+            if (FP8) ((uint8_t *)p.v_cache)[o0] = to_fp8<FP8 ? FP8 : 1>(to_f32(src[i * p.v_stride[0]]), v_div);
             else ((T *)p.v_cache)[o0] = src[i * p.v_stride[0]];
         }
         return;
@@ -112,7 +114,7 @@ rope_cache_write_kernel(const lazyattn_rope_write_params p) {
     const bool write = slot >= 0 && p.k_cache != nullptr;
     const int64_t blk = write ? slot / p.block_size : 0;
     const int off = write ? (int)(slot % p.block_size) : 0;
-    const float k_inv = FP8 ? 1.f / *p.k_scale : 1.f;
+    const float k_div = FP8 ? *p.k_scale : 1.f;
 
     // K chunk (8 consecutive d starting at d0) of head h -> [block, head, d / x, offset, d % x]
     auto put_k = [&](int h, int d0, const float *f, const Vec8<T> &raw) {
@@ -122,7 +124,7 @@ rope_cache_write_kernel(const lazyattn_rope_write_params p) {
         if (FP8) {
             uint8_t b[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) b[i] = to_fp8<FP8 ? FP8 : 1>(f[i], k_inv);
+            for (int i = 0; i < 8; ++i) b[i] = to_fp8<FP8 ? FP8 : 1>(f[i], k_div);
             *reinterpret_cast<uint2 *>(dst) = *reinterpret_cast<const uint2 *>(b);
         } else if (p.x % 8 == 0) {
             raw.store(reinterpret_cast<T *>(dst));

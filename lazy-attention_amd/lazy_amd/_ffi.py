@@ -7,6 +7,7 @@ from __future__ import annotations
 
 import ctypes as C
 import os
+from collections import OrderedDict
 from typing import Optional
 
 import torch
@@ -137,27 +138,42 @@ def workspace(device: torch.device, nbytes: int) -> Optional[torch.Tensor]:
     return buf
 
 
-_packed_tables: dict = {}
+_packed_tables: "OrderedDict" = OrderedDict()
+_PACKED_TABLES_MAX = 8
+
+
+def table_version(table: torch.Tensor) -> Optional[int]:
+    """torch's in-place edit counter of the table, or None for a tensor made under
+    ``torch.inference_mode()`` (those carry no counter and reading it raises)."""
+    return None if table.is_inference() else table._version
+
+
+def invalidate_packed_tables() -> None:
+    """Drop every re-laid-out copy.  Needed only after writing in place to a table that was created under
+    ``torch.inference_mode()``: such an edit cannot be seen from here (other tables are re-packed on their own)."""
+    _packed_tables.clear()
 
 
 def packed_cos_sin(table: torch.Tensor) -> Optional[torch.Tensor]:
     """The table in the gather-friendly layout, built once per table (and again if the
-    caller writes to it) by the library's pack kernel."""
+    caller writes to it) by the library's pack kernel.  The few most recently used tables are kept."""
     if table.dim() != 2 or table.shape[1] % 16 or table.stride(1) != 1:
         return None
     key = (table.data_ptr(), tuple(table.shape), table.stride(0), table.dtype, table.device)
+    version = table_version(table)
     hit = _packed_tables.get(key)
-    if hit is not None and hit[0] == table._version:
+    if hit is not None and hit[0] == version:
+        _packed_tables.move_to_end(key)
         return hit[1]
-    if len(_packed_tables) >= 4:
-        _packed_tables.clear()
+    while len(_packed_tables) >= _PACKED_TABLES_MAX:
+        _packed_tables.popitem(last=False)
     packed = torch.empty(table.shape[0] * table.shape[1], dtype=table.dtype, device=table.device)
     rc = lib().lazyattn_pack_cos_sin_cache(table.data_ptr(), packed.data_ptr(), dtype_code(table.dtype),
                                            table.stride(0), table.shape[0], table.shape[1],
                                            torch.cuda.current_stream(table.device).cuda_stream)
     check(rc, "lazyattn_pack_cos_sin_cache")
     # the entry holds the table too: while it is cached its address cannot be handed to another tensor
-    _packed_tables[key] = (table._version, packed, table)
+    _packed_tables[key] = (version, packed, table)
     return packed
 
 

@@ -297,8 +297,8 @@ def paged_decode(q, k_cache, v_cache, block_table, query_start_loc, seq_lens,
       (old_ops/chunked_prefill_paged_decode.py:68-280).
     pos_mode=POS_BLOCK_UNIFORM: the reference de-rotates Q by q_offset-1 once per distinct
       offset (ops/models/llama_v1.py:231-262); rotating the page's keys forward by the same
-      angle gives the same scores, which is how it is stated here.  Requests with
-      is_lazy[b]==0 are not rotated and ignore q_mask."""
+      angle gives the same scores, which is how it is stated here.  An offset of 0 keeps the
+      previous page's rotation.  Requests with is_lazy[b]==0 are not rotated and ignore q_mask."""
     cdt = compute_dtype
     hq, d = q.shape[1], q.shape[2]
     hkv = k_cache.shape[1]
@@ -329,7 +329,15 @@ def paged_decode(q, k_cache, v_cache, block_table, query_start_loc, seq_lens,
             if pos_mode == POS_NATURAL:
                 pos = n
             else:
-                qo = q_offset[b, :npages].long()[n // bs]
+                # A page whose offset is 0 keeps the rotation of the page before it (the kernel only acts
+                # when the value changes and does nothing for 0: `prev_rot_offset`, llama_v1.py:231-262);
+                # before the first non-zero entry there is no rotation.  1 is "rotation by 0".
+                carried = []
+                last = 0
+                for v in q_offset[b, :npages].tolist():
+                    last = v if v != 0 else last
+                    carried.append(last)
+                qo = torch.tensor(carried, dtype=torch.long)[n // bs]
                 pos = torch.where(qo != 0, qo - 1, torch.zeros_like(qo))
             rows = table[pos]
             kg = neox_rotate(kg, rows[:, None, :half], rows[:, None, half:])

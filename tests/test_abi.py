@@ -113,3 +113,15 @@ def test_unpack_block_table_layout():
     over = (6 << 32) | ((0xFFFF + 1) << 16)
     blk, off, _ = unpack_block_table(torch.tensor([[over]], dtype=torch.int64))
     assert blk.item() == 7 and off.item() == 0
+
+
+def test_table_version_of_inference_tensors():
+    """A table made under torch.inference_mode() has no edit counter (reading it raises): the cache of
+    re-laid-out tables keys such a table on its address and shape only."""
+    with torch.inference_mode():
+        t = torch.zeros(32, 16).to(torch.bfloat16)
+    assert t.is_inference() and _ffi.table_version(t) is None
+    u = torch.zeros(32, 16)
+    v0 = _ffi.table_version(u)
+    u.add_(1)
+    assert _ffi.table_version(u) == v0 + 1

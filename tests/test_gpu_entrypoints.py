@@ -117,3 +117,36 @@ def test_reference_kernel_test_grid(head_size, queries_per_kv, block_size):
                     cos_sin_cache=g.cos_sin_cache, q_mask=g.q_mask)
     err = (out.cpu().float() - both.float()).abs().max().item()
     assert err < 5e-3, err
+
+
+def test_tables_made_under_inference_mode():
+    """In serving the cos/sin table is an inference tensor (the model runner works under
+    torch.inference_mode() and converts the table there, rotary_embedding.py:79-82): such a tensor has no
+    edit counter.  Both entry points of the un-rotated-cache variant, which re-lay the table out once and
+    cache the copy, take it -- inside and outside inference mode, repeatedly."""
+    from lazy_amd.attention.old_ops.prefix_prefill import context_attention_fwd
+    print("case: inference-mode table", flush=True)
+    w = _mixed("offset", torch.bfloat16, 128, seed=43)
+    ref = _expected(w)
+    prefill_only = torch.full_like(w.q, 5.0)
+    orc.prefix_prefill(w.q, w.k, w.v, w.k_cache, w.v_cache, w.block_table, w.b_start_loc, w.b_seq_len,
+                       w.cos_sin_cache, w.q_offset, w.q_mask, pos_mode=w.pos_mode, rotate_new_k=w.rotate_new_k,
+                       out=prefill_only)
+    g = w.to(DEV)
+    with torch.inference_mode():
+        table = g.cos_sin_cache.float().to(torch.bfloat16)
+        assert table.is_inference()
+        for _ in range(2):
+            out = torch.full_like(g.q, 5.0)
+            context_attention_fwd(g.q, g.k, g.v, out, "auto", g.k_cache, g.v_cache, g.block_table, g.b_start_loc,
+                                  g.b_seq_len, g.max_seq_len, g.max_query_len, g.k_scale, g.v_scale, rotary_dim=128,
+                                  cos_sin_cache=table, q_mask=g.q_mask, q_offset=g.q_offset, is_mepic=False)
+            err = (out.cpu().float() - prefill_only.float()).abs().max().item()
+            assert err < 2e-2, err
+    out = torch.full_like(g.q, 5.0)
+    entry_unrotated(g.q, g.k, g.v, out, "auto", g.k_cache, g.v_cache, g.block_table, g.b_start_loc, g.b_seq_len,
+                    g.max_seq_len, g.max_query_len, g.k_scale, g.v_scale, sm_scale=128 ** -0.5, rotary_dim=128,
+                    cos_sin_cache=table, q_mask=g.q_mask, q_offset=g.q_offset, is_mepic=False)
+    # (the q_len==1 rows of this variant are rotated at their natural positions, old_ops/chunked...:204-213)
+    err = (out.cpu().float() - ref.float()).abs().max().item()
+    assert err < 2e-2, err

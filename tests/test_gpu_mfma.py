@@ -1,7 +1,7 @@
 """GPU parity of the bf16 MFMA kernel (and its split-KV merge) against the CPU oracle,
 through the Python operators / C ABI.  Max abs error on N(0,1) inputs: 2e-2 for a bf16
 cache, 5e-2 for an fp8 cache.  Full-size configurations are checked against the oracle
-where it finishes in seconds and through split-count invariance otherwise."""
+(configurations 2-5 at full size, in all three position modes) and through split-count invariance."""
 import pytest
 import torch
 
@@ -367,9 +367,38 @@ def test_mfma_small_group_uses_four_wave_kernel():
     assert e < 2e-2, e
 
 
-def test_config2_north_star_full_size():
-    print("case: config 2 full", flush=True)
-    w = wl.config(2)
+@pytest.mark.parametrize("nsplit", [1, 3])
+def test_rows_past_the_grid_stay_untouched_with_split_merge(nsplit):
+    """max_input_len sizes the grid (ops/prefix_prefill.py:681-682): rows of a request beyond it are not
+    computed and `o` keeps what it held there -- also when the key axis is split and a second kernel merges
+    the partials (it may only merge rows the main kernel wrote; the workspace still holds an earlier call)."""
+    import dataclasses
+    print(f"case: mfma rows past max_input_len, nsplit={nsplit}", flush=True)
+    w = _ragged("offset")
+    ref = run_oracle(w)
+    g = w.to(DEV)
+    run_op(g, kernel=_ffi.KERNEL_MFMA, num_splits=3)                       # leaves partials of every row behind
+    short = dataclasses.replace(g, max_query_len=64)
+    got = run_op(short, kernel=_ffi.KERNEL_MFMA, num_splits=nsplit, out=torch.full_like(g.q, 5.0)).cpu()
+    starts = w.b_start_loc.tolist()
+    for b in range(len(starts) - 1):
+        qs, qe = starts[b], starts[b + 1]
+        cut = min(qe, qs + 64)
+        if cut > qs:
+            e = _err(got[qs:cut], ref[qs:cut])
+            assert e < 2e-2, (b, e)
+        assert torch.all(got[cut:qe] == 5.0), b
+
+
+VARIANTS = ["natural", "offset", "block_uniform"]
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_config2_north_star_full_size(variant):
+    """natural: key n rotated at n; offset: every page's position read from q_offset (the per-block offsets of
+    the un-rotated cache); block_uniform: cache rotated at document-local positions, one rotation per page."""
+    print(f"case: config 2 full {variant}", flush=True)
+    w = wl.config(2, variant=variant)
     assert w.q.shape == (128, 32, 128) and abs(w.flops / 1e9 - 10.873) < 1e-2
     ref = run_oracle(w)
     g = w.to(DEV)
@@ -379,23 +408,33 @@ def test_config2_north_star_full_size():
         assert e < 2e-2, (ns, e)
 
 
-def test_config3_batched_reuse_full_size():
-    print("case: config 3 full", flush=True)
-    w = wl.config(3)
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_config3_batched_reuse_full_size(variant):
+    print(f"case: config 3 full {variant}", flush=True)
+    w = wl.config(3, variant=variant)
     ref = run_oracle(w)
     got = run_op(w.to(DEV)).cpu()
     e = _err(got, ref)
     assert e < 2e-2, e
 
 
+@pytest.mark.parametrize("variant", VARIANTS)
 @pytest.mark.parametrize("idx,tol", [(4, 2e-2), (5, 5e-2)])
-def test_config4_config5_reduced_vs_oracle_and_full_size_split_invariance(idx, tol):
-    print(f"case: config {idx} reduced + full", flush=True)
-    w = wl.config(idx, shrink=8)
+def test_config4_config5_full_size_vs_oracle(idx, tol, variant):
+    """Long context (65 536 cached keys, 256 new tokens) and fp8 pages (8 requests x 16 384 keys) at full size
+    against the CPU oracle (about a second of host time each), in all three position modes."""
+    print(f"case: config {idx} full {variant}", flush=True)
+    w = wl.config(idx, variant=variant)
     ref = run_oracle(w)
     got = run_op(w.to(DEV)).cpu()
+    assert torch.isfinite(got.float()).all()
     e = _err(got, ref)
     assert e < tol, e
+
+
+@pytest.mark.parametrize("idx,tol", [(4, 2e-2), (5, 5e-2)])
+def test_config4_config5_split_invariance_and_generic_kernel(idx, tol):
+    print(f"case: config {idx} full, split invariance", flush=True)
     # full size: the result may not depend on how the key axis is split
     g = wl.config(idx).to(DEV)
     a = run_op(g, num_splits=1)
@@ -403,7 +442,7 @@ def test_config4_config5_reduced_vs_oracle_and_full_size_split_invariance(idx, t
     assert torch.isfinite(a.float()).all()
     e = _err(a, b)
     assert e < 1e-2, e
-    # and it agrees with the geometry-agnostic fp32 kernel on a slice of the queries
+    # and it agrees with the geometry-agnostic fp32 kernel
     c = run_op(g, kernel=_ffi.KERNEL_GENERIC)
     e = _err(a, c)
     assert e < tol, e

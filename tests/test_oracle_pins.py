@@ -366,6 +366,101 @@ def test_lazy_decode_rotating_keys_equals_derotating_query():
     assert (got[0].double() - ref).abs().max() < 1e-6
 
 
+def _token_into_cache(w, bs):
+    """Write every request's (single) new token where the attention backend leaves it (backends/triton_attn.py:100-109)."""
+    hkv, x = w.k_cache.shape[1], w.k_cache.shape[4]
+    for b in range(w.b_seq_len.numel()):
+        ctx = int(w.b_seq_len[b]) - 1
+        pb = int(w.block_table[b, ctx // bs]); o_ = ctx % bs
+        w.k_cache[pb, :, :, o_, :] = w.k[int(w.b_start_loc[b])].view(hkv, -1, x)
+        w.v_cache[pb, :, :, o_] = w.v[int(w.b_start_loc[b])]
+
+
+@pytest.mark.parametrize("window", [3, 6, 50])
+def test_decode_oracle_sliding_window_equals_prefill_oracle(window):
+    """paged_decode(sliding_window=w): the same rows through the prefill oracle, whose window branch is pinned by
+    the brute force above (old_ops/chunked_prefill_paged_decode.py:237-241 vs old_ops/prefix_prefill.py:270-284)."""
+    w = wl.make_workload("decw", dtype=torch.float32, hq=4, hkv=2, d=8, theta=10000.0, block_size=4,
+                         doc_lens=[8, 6, 5], requests=[[1, 0, 2], [0]], q_lens=[1, 1], variant="natural", seed=14)
+    pre = run_oracle(w, compute_dtype=torch.float64, sliding_window=window)
+    _token_into_cache(w, 4)
+    dec = orc.paged_decode(w.q, w.k_cache, w.v_cache, w.block_table, w.b_start_loc, w.b_seq_len,
+                           w.cos_sin_cache, w.q_mask, compute_dtype=torch.float64, sliding_window=window)
+    assert (dec - pre).abs().max() < 1e-6
+    if window < 8:
+        unwindowed = orc.paged_decode(w.q, w.k_cache, w.v_cache, w.block_table, w.b_start_loc, w.b_seq_len,
+                                      w.cos_sin_cache, w.q_mask, compute_dtype=torch.float64)
+        assert (dec - unwindowed).abs().max() > 1e-3                # the window does cut something
+
+
+def test_decode_oracle_unrotated_requests_equal_prefill_oracle():
+    """paged_decode(is_lazy[b] == 0) under the block-uniform mode (ops/models/llama_v1.py:290-434): no rotation, no
+    pad mask -- the same rows through the prefill oracle's un-rotated branch, which the brute force pins."""
+    w = wl.make_workload("decv", dtype=torch.float32, hq=4, hkv=2, d=8, theta=10000.0, block_size=4,
+                         doc_lens=[7, 6, 5], requests=[[1, 0, 2], [0], [2, 1]], q_lens=[1, 1, 1],
+                         variant="block_uniform", seed=15)
+    lazy = torch.tensor([False, True, False])
+    pre = run_oracle(w, compute_dtype=torch.float64, is_lazy=lazy)
+    _token_into_cache(w, 4)
+    dec = orc.paged_decode(w.q, w.k_cache, w.v_cache, w.block_table, w.b_start_loc, w.b_seq_len, w.cos_sin_cache,
+                           w.q_mask, q_offset=w.q_offset, is_lazy=lazy, pos_mode=orc.POS_BLOCK_UNIFORM,
+                           compute_dtype=torch.float64)
+    assert (dec - pre).abs().max() < 1e-6
+    all_lazy = orc.paged_decode(w.q, w.k_cache, w.v_cache, w.block_table, w.b_start_loc, w.b_seq_len, w.cos_sin_cache,
+                                w.q_mask, q_offset=w.q_offset, pos_mode=orc.POS_BLOCK_UNIFORM, compute_dtype=torch.float64)
+    assert (dec[0] - all_lazy[0]).abs().max() > 1e-3 and (dec[1] - all_lazy[1]).abs().max() < 1e-12
+
+
+def test_lazy_decode_zero_offset_keeps_the_previous_rotation():
+    """The page walk of ops/models/llama_v1.py:149-262 restated literally -- Q de-rotated when the page's offset
+    differs from the previous page's, 1 = the query as given, 0 = leave Q as it is -- on a table with zeros after
+    offsets above 1 (which the scheduler never emits, but the kernel defines)."""
+    w = wl.make_workload("carry", dtype=torch.float32, hq=4, hkv=2, d=8, theta=10000.0, block_size=4,
+                         doc_lens=[8, 8, 4], requests=[[1, 0, 2]], q_lens=[1], variant="block_uniform", seed=16)
+    _token_into_cache(w, 4)
+    seq = int(w.b_seq_len[0])
+    npages = (seq + 3) // 4
+    qo = w.q_offset.clone()
+    assert qo[0, :npages].tolist()[:5] == [1, 1, 9, 9, 17]
+    qo[0, 1] = 0          # after a 1: identity either way
+    qo[0, 3] = 0          # after a 9: keeps the rotation by 8
+    qo[0, 5] = 0          # the query page (was 1): keeps the rotation by 16 of page 4
+    got = orc.paged_decode(w.q, w.k_cache, w.v_cache, w.block_table, w.b_start_loc, w.b_seq_len, w.cos_sin_cache,
+                           w.q_mask, q_offset=qo, pos_mode=orc.POS_BLOCK_UNIFORM, compute_dtype=torch.float64)
+    tab = w.cos_sin_cache.double()
+    q_full = w.q[0].double()
+    q_rot = q_full
+    prev = -1
+    scores = torch.full((4, seq), float("-inf"), dtype=torch.float64)
+    vals = torch.zeros(seq, 2, 8, dtype=torch.float64)
+    for j in range(npages):
+        val = int(qo[0, j])
+        if val != prev:
+            if val == 1:
+                q_rot = q_full
+            elif val != 0:
+                rows = tab[val - 1]
+                q_rot = orc.neox_rotate(q_full, rows[:4], -rows[4:])
+            prev = val
+        blk = int(w.block_table[0, j])
+        for o_ in range(4):
+            n = j * 4 + o_
+            if n >= seq or o_ >= 4 - int(w.q_mask[0, j]):
+                continue
+            kvec = w.k_cache[blk, :, :, o_, :].reshape(2, 8).double()
+            vals[n] = w.v_cache[blk, :, :, o_].double()
+            for h in range(4):
+                scores[h, n] = (q_rot[h] * kvec[h // 2]).sum() / math.sqrt(8)
+    p = torch.softmax(scores, dim=-1)
+    ref = torch.stack([(p[h][:, None] * vals[:, h // 2]).sum(0) for h in range(4)])
+    assert (got[0].double() - ref).abs().max() < 1e-6
+    # and the carry matters: reading 0 as "no rotation" gives something else
+    naive = orc.paged_decode(w.q, w.k_cache, w.v_cache, w.block_table, w.b_start_loc, w.b_seq_len, w.cos_sin_cache,
+                             w.q_mask, q_offset=torch.where(qo == 0, torch.ones_like(qo), qo),
+                             pos_mode=orc.POS_BLOCK_UNIFORM, compute_dtype=torch.float64)
+    assert (got - naive).abs().max() > 1e-3
+
+
 def test_paged_cache_write_is_inverse_of_gather_and_matches_layout_formula():
     """K[block, h, d // x, off, d % x], V[block, h, d, off] (the third-party reshape_and_cache layout the
     reference's kernels index at old_ops/prefix_prefill.py:172-181,196-199): element-wise formula on a
