@@ -111,6 +111,16 @@ typedef struct lazyattn_prefill_params {
     int32_t num_tokens;         /* rows of `o` (>= b_start_loc[B]); sizes the split-KV workspace */
     int32_t max_seq_len;        /* upper bound of b_seq_len, 0 = unknown; only steers the split count */
     int32_t packed_rows;        /* rows of cos_sin_packed (0 when it is NULL) */
+    /* ---- read by lazyattn_paged_decode_rotary() only ---- */
+    const int64_t *packed_block_table; /* optional [B, NBmax]: [block:32 | q_offset:16 | q_mask:16] per entry, the table
+                                   the reference's q_len==1 kernel walks (ops/models/llama_v1.py:157-160,
+                                   ops/chunked_prefill_paged_decode.py:162-164).  When set it replaces block_table,
+                                   q_offset and q_mask (which may then be NULL): one 8-byte read per page. */
+    int64_t pbt_stride[2];
+    const float *rope_freqs;    /* optional [rotary_dim/2] float32 inverse frequencies, radians per position
+                                   (rope_freqs, model_executor/rope/cos_sin.py:24-59).  When set, cos/sin are computed
+                                   in the kernel (rope_cos_sin_from_freqs, :62-66; the reference's COMPUTE_COS_SIN
+                                   switch, ops/chunked_prefill_paged_decode.py:146-151) and cos_sin_cache is not read. */
 } lazyattn_prefill_params;
 
 /* Bytes of workspace lazyattn_prefix_prefill() may need for these sizes (0 when the
@@ -148,7 +158,8 @@ size_t lazyattn_paged_decode_workspace_bytes(const lazyattn_prefill_params *p);
  *   PagedAttention.write_to_paged_cache(key, value, key_cache, value_cache, slot_mapping,
  *     kv_cache_dtype, k_scale, v_scale)  (lazy_attn/lazy/attention/backends/triton_attn.py:100-109):
  *     token t -> slot_mapping[t] = block * block_size + offset (negative: not written);
- *     fp8 caches store value / scale, saturated to +-448, rounded to e4m3.
+ *     fp8 caches store value / scale (a true division), saturated to +-448 and rounded to e4m3, or to +-57344 and
+ *     e5m2; NaN stays NaN.  An fp8 K cache needs x % 8 == 0.
  * The key written to the cache is the key as it is left in `k` (rotated iff rotate_k). */
 typedef struct lazyattn_rope_write_params {
     void *q;                    /* [T, Hq, D], rotated in place when rotate_q; may be NULL when !rotate_q */
@@ -166,7 +177,7 @@ typedef struct lazyattn_rope_write_params {
     int64_t table_stride;
     int32_t num_tokens, num_q_heads, num_kv_heads, head_dim, rotary_dim, block_size, x;
     int32_t dtype;              /* q/k/v: LAZYATTN_F32 / BF16 / F16 */
-    int32_t cache_dtype;        /* = dtype, or LAZYATTN_FP8_E4M3 */
+    int32_t cache_dtype;        /* = dtype, or LAZYATTN_FP8_E4M3 / LAZYATTN_FP8_E5M2 */
     int32_t table_dtype;        /* = dtype, or LAZYATTN_F32 */
     int32_t rotate_q, rotate_k;
     int32_t pos_bits, slot_bits;

@@ -39,9 +39,11 @@ static int elem_bytes(int dt) {
 
 static int check_common(const lazyattn_prefill_params *p, bool decode) {
     if (!p) return LAZYATTN_E_NULL;
-    if (!p->q || !p->o || !p->k_cache || !p->v_cache || !p->block_table || !p->b_start_loc ||
-        !p->b_seq_len || !p->cos_sin_cache)
-        return LAZYATTN_E_NULL;
+    if (!p->q || !p->o || !p->k_cache || !p->v_cache || !p->b_start_loc || !p->b_seq_len) return LAZYATTN_E_NULL;
+    // the q_len == 1 entry takes the packed table in place of the three int32 tables, and frequencies in place of the table
+    const bool packed = decode && p->packed_block_table;
+    if (!p->block_table && !packed) return LAZYATTN_E_NULL;
+    if (!p->cos_sin_cache && !(decode && p->rope_freqs)) return LAZYATTN_E_NULL;
     if (!decode && (!p->k || !p->v)) return LAZYATTN_E_NULL;
     if (p->batch < 0 || p->num_q_heads <= 0 || p->num_kv_heads <= 0 || p->head_dim <= 0 ||
         p->block_size <= 0 || p->x <= 0)
@@ -58,7 +60,7 @@ static int check_common(const lazyattn_prefill_params *p, bool decode) {
     if (p->table_dtype != p->dtype && p->table_dtype != LAZYATTN_F32) return LAZYATTN_E_DTYPE;
     if (p->pos_mode < LAZYATTN_POS_NATURAL || p->pos_mode > LAZYATTN_POS_BLOCK_UNIFORM)
         return LAZYATTN_E_UNSUPPORTED;
-    if (p->pos_mode != LAZYATTN_POS_NATURAL && !p->q_offset) return LAZYATTN_E_NULL;
+    if (p->pos_mode != LAZYATTN_POS_NATURAL && !p->q_offset && !packed) return LAZYATTN_E_NULL;
     (void)elem_bytes;
     return LAZYATTN_OK;
 }
@@ -92,6 +94,8 @@ extern "C" int lazyattn_paged_decode_rotary(const lazyattn_prefill_params *p, vo
     if (p->pos_mode == LAZYATTN_POS_OFFSET) return LAZYATTN_E_UNSUPPORTED;
     if (p->batch == 0) return LAZYATTN_OK;
     if (p->kernel != LAZYATTN_KERNEL_GENERIC && decode_mfma_supports(*p)) return launch_decode_mfma(*p, (hipStream_t)stream);
+    // the packed table and computed cos/sin are read by the streaming kernel only
+    if (p->packed_block_table || p->rope_freqs) return LAZYATTN_E_UNSUPPORTED;
     if (p->kernel != LAZYATTN_KERNEL_AUTO && p->kernel != LAZYATTN_KERNEL_GENERIC) return LAZYATTN_E_UNSUPPORTED;
     return launch_prefill_generic(*p, 1, (hipStream_t)stream);
 }
@@ -219,4 +223,4 @@ extern "C" const char *lazyattn_error_string(int code) {
     }
 }
 
-extern "C" int lazyattn_abi_version(void) { return 1; }
+extern "C" int lazyattn_abi_version(void) { return 2; }

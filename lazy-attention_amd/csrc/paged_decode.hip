@@ -81,6 +81,7 @@ template <typename TT, int HD> struct KeyRegs {
     Tab8<TT> c[HD / 64], s[HD / 64];   // cos / sin for d = 32 j + 8 grp ..
     int lim;                    // valid slots
     int first;                  // first slot inside the sliding window (<= 0: all)
+    int tag;                    // computed cos/sin: what c and s currently hold (page or position), -1 = nothing
 };
 template <int HD> struct ValRegs {
     uint2 v[HD / 16];           // V[d = 16 blk + t][tokens 4 grp .. 4 grp + 3]
@@ -90,9 +91,12 @@ template <int HD> struct ValRegs {
 
 // PAD: the head size is a multiple of 16 below HD = 128; the lane's chunks, the query and the V rows are laid out as
 // for 128 with the two halves of the real head at (0 .., 64 ..) and zeros in between
-template <typename T, typename TT, int FP8, int HD, bool PAD>
+// COMPUTE: cos/sin come from the inverse frequencies (p.rope_freqs) instead of the table; they are kept as the table
+// would hold them, rounded to the element type (TT = T): half the registers of floats
+template <typename T, typename TT, int FP8, int HD, bool PAD, bool COMPUTE>
 __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2)))
 paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
+    static_assert(!COMPUTE || std::is_same<TT, T>::value, "computed cos/sin are kept in the element type");
     using E = Elem<T>;
     constexpr int D = HD, NM = HD / 32, NP = HD / 64, NBLK = HD / 16;
     constexpr int TSZ = sizeof(TT);
@@ -120,7 +124,10 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     const bool lazy_b = p.is_lazy ? p.is_lazy[b] != 0 : true;
     const bool vanilla = p.pos_mode == LAZYATTN_POS_BLOCK_UNIFORM && !lazy_b;
     const bool per_token = !vanilla && p.pos_mode == LAZYATTN_POS_NATURAL;
-    const bool use_qmask = !vanilla && p.q_mask != nullptr;
+    // the packed table [block:32 | q_offset:16 | q_mask:16] is read as pairs of 32-bit words: the block is the
+    // high word, offset and pad count share the low one
+    const bool packed = p.packed_block_table != nullptr;
+    const bool use_qmask = !vanilla && (packed || p.q_mask != nullptr);
     const bool use_qo = !vanilla && p.pos_mode == LAZYATTN_POS_BLOCK_UNIFORM;
     const int n_pages = seq_len > 0 ? (seq_len + BS - 1) / BS : 0;
     const int n_pairs = (n_pages + 1) / 2;
@@ -135,13 +142,16 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
 
     // page metadata through the scalar unit
     typedef const int32_t __attribute__((address_space(4))) *sptr_i32;
-    const sptr_i32 bt_row = (sptr_i32)(p.block_table + b * p.bt_stride[0]);
-    const sptr_i32 qo_row = use_qo ? (sptr_i32)(p.q_offset + b * p.qo_stride[0]) : bt_row;
-    const sptr_i32 qm_row = use_qmask ? (sptr_i32)(p.q_mask + b * p.qm_stride[0]) : bt_row;
-    const int64_t bt_s1 = p.bt_stride[1];
-    const int64_t qo_s1 = use_qo ? p.qo_stride[1] : p.bt_stride[1];
-    const int64_t qm_s1 = use_qmask ? p.qm_stride[1] : p.bt_stride[1];
-    const int qo_and = use_qo ? -1 : 0, qm_and = use_qmask ? -1 : 0;
+    const int32_t *pk_words = packed ? (const int32_t *)(p.packed_block_table + b * p.pbt_stride[0]) : nullptr;
+    const sptr_i32 pk_row = (sptr_i32)pk_words;                                      // low words
+    const sptr_i32 bt_row = packed ? pk_row + 1 : (sptr_i32)(p.block_table + b * p.bt_stride[0]);
+    const sptr_i32 qo_row = !use_qo ? bt_row : packed ? pk_row : (sptr_i32)(p.q_offset + b * p.qo_stride[0]);
+    const sptr_i32 qm_row = !use_qmask ? bt_row : packed ? pk_row : (sptr_i32)(p.q_mask + b * p.qm_stride[0]);
+    const int64_t bt_s1 = packed ? 2 * p.pbt_stride[1] : p.bt_stride[1];
+    const int64_t qo_s1 = !use_qo ? bt_s1 : packed ? 2 * p.pbt_stride[1] : p.qo_stride[1];
+    const int64_t qm_s1 = !use_qmask ? bt_s1 : packed ? 2 * p.pbt_stride[1] : p.qm_stride[1];
+    const int qo_shift = use_qo && packed ? 16 : 0;
+    const int qo_and = !use_qo ? 0 : packed ? 0xffff : -1, qm_and = !use_qmask ? 0 : packed ? 0xffff : -1;
 
     constexpr int CSZ = FP8 ? 1 : 2;                             // bytes per cache element
     const uint8_t *kc_base = (const uint8_t *)p.k_cache + (int64_t)g * p.kc_stride[1] * CSZ;
@@ -180,12 +190,41 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
         jc = jc < 0 ? 0 : jc;
         return bt_row[(jc >> pshift) * bt_s1];
     };
+    // Block-uniform rotation: a page whose offset is 0 keeps the rotation of the page before it (the reference acts
+    // only when the value changes and does nothing for 0, ops/models/llama_v1.py:207-262).  The pages of a slice
+    // are visited in order, so the last non-zero offset is carried along; a slice that does not start at page 0
+    // and whose first offset is 0 finds it by scanning backwards, 64 entries per step.
+    int carry = 0;
+    if (use_qo && pair_begin > 0 && pair_begin < pair_end) {
+        int pj = (2 * pair_begin) >> pshift;
+        if (((qo_row[pj * qo_s1] >> qo_shift) & qo_and) == 0) {
+            const int32_t *row = packed ? pk_words : p.q_offset + b * p.qo_stride[0];
+            for (int base = pj - 1; base >= 0 && carry == 0; base -= 64) {
+                const int idx = base - lane;
+                const int v = idx >= 0 ? (row[idx * qo_s1] >> qo_shift) & qo_and : 0;
+                const uint64_t hit = __builtin_amdgcn_ballot_w64(v != 0);
+                if (hit) carry = __builtin_amdgcn_readlane(v, __builtin_ctzll(hit));
+            }
+        }
+    }
+    // COMPUTE: this lane's inverse frequencies, in revolutions per position (d = 32 j + 8 grp + e)
+    float frev[COMPUTE ? NP * 8 : 1];
+    if constexpr (COMPUTE) {
+#pragma unroll
+        for (int j = 0; j < NP; ++j) {
+            const int e0 = PAD && 32 * j + 8 * grp >= HALFr ? 0 : 32 * j + 8 * grp;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) frev[j * 8 + e] = p.rope_freqs[e0 + e] * 0.15915494309189535f;
+        }
+    }
     auto load_keys = [&](int j, KeyRegs<TT, HD> &r) {
         int jc = j < n_pages ? j : n_pages - 1;
         jc = jc < 0 ? 0 : jc;
         const int pj = jc >> pshift, part = jc & pshift;
         const int bt = bt_row[pj * bt_s1];
-        const int qo = qo_row[pj * qo_s1] & qo_and;
+        int qo = (qo_row[pj * qo_s1] >> qo_shift) & qo_and;
+        carry = qo ? qo : carry;
+        qo = carry;
         const int qm = qm_row[pj * qm_s1] & qm_and;                                  // old_ops/chunked...:165-167 analogue
         const int ql = cache_bs - qm - (j & pshift) * BS;                            // valid slots of this part
         int l = seq_len - j * BS;
@@ -220,12 +259,38 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
             pos = pos < seq_len ? pos : seq_len - 1;     // slots past the end are masked; stay inside the table
             pos = pos < 0 ? 0 : pos;
         }
-        const uint8_t *row = tab + (int64_t)pos * row_bytes;
+        if constexpr (COMPUTE) {
+            // rope_cos_sin_from_freqs (model_executor/rope/cos_sin.py:62-66): cos / sin of position x frequency.  The
+            // product is formed exactly (rounded product + its fma remainder) and reduced to one revolution before the
+            // hardware sine and cosine, so the angle keeps float accuracy at positions in the tens of thousands.
+            // Block-uniform pages repeat their position for a whole document: recomputed only when it changes.
+            const int key = per_token ? j : pos;                                     // wave-uniform
+            if (key != r.tag) {
+                r.tag = key;
+                const float P = (float)pos;
 #pragma unroll
-        for (int j = 0; j < NP; ++j) {
-            const int e = PAD && 32 * j + 8 * grp >= HALFr ? 0 : 32 * j + 8 * grp;   // (a padded chunk is zero: any angle will do)
-            r.c[j].load(row, e);
-            r.s[j].load(row, HALFr + e);
+                for (int jj = 0; jj < NP; ++jj) {
+                    float cs[8], sn[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float f = frev[jj * 8 + e];
+                        const float hi = P * f, lo = fmaf(P, f, -hi);
+                        const float rev = __builtin_amdgcn_fractf(hi) + lo;
+                        cs[e] = __builtin_amdgcn_cosf(rev);
+                        sn[e] = __builtin_amdgcn_sinf(rev);
+                    }
+                    r.c[jj].v = make_uint4(E::pack(cs[0], cs[1]), E::pack(cs[2], cs[3]), E::pack(cs[4], cs[5]), E::pack(cs[6], cs[7]));
+                    r.s[jj].v = make_uint4(E::pack(sn[0], sn[1]), E::pack(sn[2], sn[3]), E::pack(sn[4], sn[5]), E::pack(sn[6], sn[7]));
+                }
+            }
+        } else {
+            const uint8_t *row = tab + (int64_t)pos * row_bytes;
+#pragma unroll
+            for (int j = 0; j < NP; ++j) {
+                const int e = PAD && 32 * j + 8 * grp >= HALFr ? 0 : 32 * j + 8 * grp;   // (a padded chunk is zero: any angle will do)
+                r.c[j].load(row, e);
+                r.s[j].load(row, HALFr + e);
+            }
         }
     };
     auto load_values = [&](int j, ValRegs<HD> &r) {
@@ -319,6 +384,7 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
     // registers it lands in, the value side of pair i at the top of its iteration: every load has
     // about half an iteration of other work between issue and use, at no extra registers.
     KeyRegs<TT, HD> KX, KY;
+    KX.tag = KY.tag = -1;
     if (pair_begin < pair_end) {
         load_keys(2 * pair_begin, KX);
         load_keys(2 * pair_begin + 1, KY);
@@ -464,12 +530,13 @@ bool decode_mfma_supports(const lazyattn_prefill_params &p) {
     if (p.kc_stride[4] != 1 || p.kc_stride[3] != p.x || p.kc_stride[2] != (int64_t)p.block_size * p.x) return false;
     if (p.vc_stride[3] != 1 || p.vc_stride[2] != p.block_size) return false;
     const int64_t al[] = {p.q_stride[0], p.q_stride[1], p.o_stride[0], p.o_stride[1], p.kc_stride[0], p.kc_stride[1],
-                          p.vc_stride[0], p.vc_stride[1], p.table_stride};
+                          p.vc_stride[0], p.vc_stride[1], p.rope_freqs ? 0 : p.table_stride};
     for (int64_t s : al)
         if (s % 16) return false;                      // 16-byte rows whatever the element size
     const void *ptrs[] = {p.q, p.o, p.k_cache, p.v_cache, p.cos_sin_cache};
     for (const void *q : ptrs)
         if (((uintptr_t)q) & 15) return false;
+    if (((uintptr_t)p.packed_block_table & 7) || ((uintptr_t)p.rope_freqs & 3)) return false;
     return true;
 }
 
@@ -511,12 +578,17 @@ int launch_decode_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
             using T = decltype(elem);
             constexpr int HD = decltype(hd)::value;
             constexpr bool PAD = decltype(pad)::value;
-            if (fp8 == 1 && t32) hipLaunchKernelGGL((paged_decode_kernel<T, float, 1, HD, PAD>), grid, block, 0, stream, p, nsplit);
-            else if (fp8 == 1) hipLaunchKernelGGL((paged_decode_kernel<T, T, 1, HD, PAD>), grid, block, 0, stream, p, nsplit);
-            else if (fp8 == 2 && t32) hipLaunchKernelGGL((paged_decode_kernel<T, float, 2, HD, PAD>), grid, block, 0, stream, p, nsplit);
-            else if (fp8 == 2) hipLaunchKernelGGL((paged_decode_kernel<T, T, 2, HD, PAD>), grid, block, 0, stream, p, nsplit);
-            else if (t32) hipLaunchKernelGGL((paged_decode_kernel<T, float, 0, HD, PAD>), grid, block, 0, stream, p, nsplit);
-            else hipLaunchKernelGGL((paged_decode_kernel<T, T, 0, HD, PAD>), grid, block, 0, stream, p, nsplit);
+            if (p.rope_freqs) {
+                if (fp8 == 1) hipLaunchKernelGGL((paged_decode_kernel<T, T, 1, HD, PAD, true>), grid, block, 0, stream, p, nsplit);
+                else if (fp8 == 2) hipLaunchKernelGGL((paged_decode_kernel<T, T, 2, HD, PAD, true>), grid, block, 0, stream, p, nsplit);
+                else hipLaunchKernelGGL((paged_decode_kernel<T, T, 0, HD, PAD, true>), grid, block, 0, stream, p, nsplit);
+            }
+            else if (fp8 == 1 && t32) hipLaunchKernelGGL((paged_decode_kernel<T, float, 1, HD, PAD, false>), grid, block, 0, stream, p, nsplit);
+            else if (fp8 == 1) hipLaunchKernelGGL((paged_decode_kernel<T, T, 1, HD, PAD, false>), grid, block, 0, stream, p, nsplit);
+            else if (fp8 == 2 && t32) hipLaunchKernelGGL((paged_decode_kernel<T, float, 2, HD, PAD, false>), grid, block, 0, stream, p, nsplit);
+            else if (fp8 == 2) hipLaunchKernelGGL((paged_decode_kernel<T, T, 2, HD, PAD, false>), grid, block, 0, stream, p, nsplit);
+            else if (t32) hipLaunchKernelGGL((paged_decode_kernel<T, float, 0, HD, PAD, false>), grid, block, 0, stream, p, nsplit);
+            else hipLaunchKernelGGL((paged_decode_kernel<T, T, 0, HD, PAD, false>), grid, block, 0, stream, p, nsplit);
         };
         using hd128 = std::integral_constant<int, 128>;
         using hd64 = std::integral_constant<int, 64>;

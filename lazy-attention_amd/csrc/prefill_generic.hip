@@ -150,7 +150,10 @@ prefill_generic_kernel(const lazyattn_prefill_params p, const int decode) {
                     if (pos_mode == LAZYATTN_POS_NATURAL) {
                         pos = n;
                     } else {
-                        const int qo = p.q_offset ? p.q_offset[b * p.qo_stride[0] + j * p.qo_stride[1]] : 0;
+                        int qo = p.q_offset ? p.q_offset[b * p.qo_stride[0] + j * p.qo_stride[1]] : 0;
+                        // q_len == 1 rows: an offset of 0 keeps the previous page's rotation (ops/models/llama_v1.py:207-262)
+                        if (decode && pos_mode == LAZYATTN_POS_BLOCK_UNIFORM && p.q_offset)
+                            for (int64_t jj = j; qo == 0 && jj > 0;) qo = p.q_offset[b * p.qo_stride[0] + (--jj) * p.qo_stride[1]];
                         if (pos_mode == LAZYATTN_POS_OFFSET) pos = qo != 0 ? (int64_t)qo - 1 + o : n;
                         else pos = qo != 0 ? (int64_t)qo - 1 : 0;
                     }

@@ -46,7 +46,8 @@ class PrefillParams(C.Structure):
                                     "rotate_new_k", "skip_decode", "fp32_rotary", "kernel",
                                     "num_splits", "phases")]
         + [("sm_scale", C.c_float), ("num_tokens", C.c_int32), ("max_seq_len", C.c_int32),
-           ("packed_rows", C.c_int32)])
+           ("packed_rows", C.c_int32),
+           ("packed_block_table", C.c_void_p), ("pbt_stride", C.c_int64 * 2), ("rope_freqs", C.c_void_p)])
 
 
 class RopeWriteParams(C.Structure):
@@ -186,7 +187,7 @@ def fill_params(*, q, k, v, o, k_cache, v_cache, block_table, b_start_loc, b_seq
                 max_q_len: int, rotary_dim: int, sliding_window: int, sm_scale: float,
                 pos_mode: int, rotate_new_k: bool, skip_decode: bool, fp32_rotary: bool = False,
                 kernel: int = KERNEL_AUTO, num_splits: int = 0, phases: int = PHASE_ALL,
-                max_seq_len: int = 0, packed_table=None) -> PrefillParams:
+                max_seq_len: int = 0, packed_table=None, packed_block_table=None, rope_freqs=None) -> PrefillParams:
     p = PrefillParams()
     p.q, p.k, p.v, p.o = _ptr(q), _ptr(k), _ptr(v), _ptr(o)
     p.k_cache, p.v_cache = _ptr(k_cache), _ptr(v_cache)
@@ -205,7 +206,11 @@ def fill_params(*, q, k, v, o, k_cache, v_cache, block_table, b_start_loc, b_seq
     p.bt_stride[:] = block_table.stride()
     p.qo_stride[:] = q_offset.stride() if q_offset is not None else (0, 0)
     p.qm_stride[:] = q_mask.stride() if q_mask is not None else (0, 0)
-    p.table_stride = cos_sin_cache.stride(0)
+    p.table_stride = cos_sin_cache.stride(0) if cos_sin_cache is not None else 0
+    if packed_block_table is not None:
+        p.packed_block_table = packed_block_table.data_ptr()
+        p.pbt_stride[:] = packed_block_table.stride()
+    p.rope_freqs = _ptr(rope_freqs)
     p.batch = b_seq_len.shape[0]
     p.num_q_heads, p.head_dim = q.shape[1], q.shape[2]
     p.num_kv_heads = k_cache.shape[1]
@@ -215,7 +220,7 @@ def fill_params(*, q, k, v, o, k_cache, v_cache, block_table, b_start_loc, b_seq
     p.sliding_window = int(sliding_window)
     p.dtype = dtype_code(q.dtype)
     p.cache_dtype = cache_code
-    p.table_dtype = dtype_code(cos_sin_cache.dtype)
+    p.table_dtype = dtype_code(cos_sin_cache.dtype) if cos_sin_cache is not None else p.dtype
     p.index_bits = 64 if b_start_loc.dtype == torch.int64 else 32
     p.pos_mode = pos_mode
     p.rotate_new_k = int(rotate_new_k)

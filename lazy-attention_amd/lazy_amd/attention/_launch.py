@@ -49,7 +49,8 @@ def launch_prefill(*, q, k, v, o, kv_cache_dtype, k_cache, v_cache, b_loc, b_sta
                    skip_decode, cos_sin_cache, rotary_dim, is_neox_style, is_lazy, q_offset, q_mask,
                    pos_mode: int, rotate_new_k: bool, fp32_rotary: bool = False,
                    kernel: int = _ffi.KERNEL_AUTO, num_splits: int = 0,
-                   phases: int = _ffi.PHASE_ALL, decode: bool = False, _return_plan: bool = False):
+                   phases: int = _ffi.PHASE_ALL, decode: bool = False, packed_block_table=None, rope_freqs=None,
+                   _return_plan: bool = False):
     lib = _ffi.lib()
     cache_code = _cache_code(kv_cache_dtype, k_cache, v_cache, q.dtype)
     if not decode:
@@ -68,11 +69,17 @@ def launch_prefill(*, q, k, v, o, kv_cache_dtype, k_cache, v_cache, b_loc, b_sta
     if not is_neox_style:
         raise NotImplementedError("only NeoX-style rotary embedding is supported")
     dev = _require_gpu(q, k, v, o, k_cache, v_cache, b_loc, b_start_loc, b_seq_len,
-                       cos_sin_cache, q_offset, q_mask, is_lazy)
+                       cos_sin_cache, q_offset, q_mask, is_lazy, packed_block_table, rope_freqs)
     if rotary_dim is None:
         rotary_dim = cos_sin_cache.shape[-1] if cos_sin_cache is not None else Lq
-    if cos_sin_cache is None:
+    if rope_freqs is not None:
+        # q_len == 1 rows with cos/sin computed from the inverse frequencies: the table is not read
+        assert decode and rope_freqs.dtype == torch.float32 and rope_freqs.is_contiguous()
+        assert rope_freqs.numel() * 2 == rotary_dim
+    elif cos_sin_cache is None:
         raise ValueError("cos_sin_cache is required")
+    if packed_block_table is not None:
+        assert decode and packed_block_table.dtype == torch.int64
     if b_start_loc.dtype != b_seq_len.dtype:
         b_seq_len = b_seq_len.to(b_start_loc.dtype)
     if b_start_loc.dtype not in (torch.int32, torch.int64):
@@ -97,9 +104,11 @@ def launch_prefill(*, q, k, v, o, kv_cache_dtype, k_cache, v_cache, b_loc, b_sta
         is_lazy=is_lazy, cache_code=cache_code, max_q_len=max_input_len, rotary_dim=rotary_dim,
         sliding_window=sliding_window, sm_scale=sm_scale, pos_mode=pos_mode,
         rotate_new_k=rotate_new_k, skip_decode=skip_decode, fp32_rotary=fp32_rotary,
-        kernel=kernel, num_splits=num_splits, phases=phases, max_seq_len=max_seq_len, packed_table=packed)
+        kernel=kernel, num_splits=num_splits, phases=phases, max_seq_len=max_seq_len, packed_table=packed,
+        packed_block_table=packed_block_table, rope_freqs=rope_freqs)
     plan = PrefillPlan(p, dev, decode, keep=(q, k, v, o, k_cache, v_cache, b_loc, b_start_loc, b_seq_len,
-                                            cos_sin_cache, q_offset, q_mask, is_lazy, k_scale, v_scale, packed))
+                                            cos_sin_cache, q_offset, q_mask, is_lazy, k_scale, v_scale, packed,
+                                            packed_block_table, rope_freqs))
     if _return_plan:
         return plan
     plan.run()

@@ -2,11 +2,14 @@
 
 Drop-in for ``lazy_attn/lazy/attention/ops/chunked_prefill_paged_decode.py:36-234``:
 ``context_attention_fwd`` for requests with more than one new token (``:79-106``), then
-the q_len==1 kernel for the rest (``:162-221``).  The reference's q_len==1 kernel reads a
-packed int64 table ``[block:32 | q_offset:16 | q_mask:16]``; here the un-packed
-``block_table`` / ``q_offset`` / ``q_mask`` the caller also passes are used, and a packed
-table is unpacked only when they are absent.  The ``NO_LAZY`` switch (``:66-67``) is the
-``NO_LAZY`` environment variable, read per call like the reference does.
+the q_len==1 kernel for the rest (``:162-221``).  Like the reference's, the q_len==1 kernel
+walks the packed int64 table ``[block:32 | q_offset:16 | q_mask:16]`` when one is passed
+(``:162-164``); the prefill kernel reads the un-packed ``q_offset`` / ``q_mask``
+(``ops/prefix_prefill.py:180-182``), which are unpacked from it only if the caller did not
+pass them.  Switches, read per call like the reference does (``utils/variants.py``):
+``NO_LAZY`` (``:66-67``) and ``LAZY_DECODE_COMPUTE_COS_SIN`` (``:146-151``: cos/sin of the
+q_len==1 kernel computed from the inverse frequencies -- ``freqs`` if given, else formed
+from ``rope_meta`` -- instead of read from ``cos_sin_cache``).
 """
 from __future__ import annotations
 
@@ -16,7 +19,20 @@ import torch
 
 from .. import _launch
 from ... import _ffi
+from ...model_executor.rope import cos_sin as _rope
 from .prefix_prefill import context_attention_fwd
+
+
+def _env_flag(name: str) -> bool:
+    return os.environ.get(name, "0") not in ("", "0")
+
+
+def _streaming_decode_covers(query, value_cache) -> bool:
+    """What the kernel that reads the packed table / computes cos and sin takes: 16-bit operands, head sizes
+    that are multiples of 16 up to 128, pages of 16 or 32 slots.  Anything else runs the generic kernel on the
+    un-packed tables and the cos/sin table."""
+    return (query.dtype in (torch.bfloat16, torch.float16) and query.shape[2] % 16 == 0 and query.shape[2] <= 128
+            and value_cache.shape[3] in (16, 32))
 
 
 def unpack_block_table(packed: torch.Tensor):
@@ -34,28 +50,39 @@ def chunked_prefill_paged_decode(query, key, value, output, kv_cache_dtype, key_
                                  sm_scale=None, rotary_dim=None, freqs=None, cos_sin_cache=None,
                                  rope_meta=None, is_neox_style=True, is_lazy=None, lazy_variant=None,
                                  q_offset=None, q_mask=None, packed_block_table=None):
-    if os.environ.get("NO_LAZY", "0") not in ("", "0") and is_lazy is not None:
+    if _env_flag("NO_LAZY") and is_lazy is not None:
         is_lazy.fill_(False)                             # ops/chunked...:66-67
     if sm_scale is None:
         sm_scale = 1.0 / (query.shape[1] ** 0.5)         # sic: ops/chunked...:71-72
     if sliding_window is None or sliding_window <= 0:
         sliding_window = 0
-    if (q_offset is None or q_mask is None) and packed_block_table is not None:
-        _, off, msk = unpack_block_table(packed_block_table)
-        q_offset = off if q_offset is None else q_offset
-        q_mask = msk if q_mask is None else q_mask
     if max_query_len > 1:
+        pq_offset, pq_mask = q_offset, q_mask
+        if (q_offset is None or q_mask is None) and packed_block_table is not None:
+            _, off, msk = unpack_block_table(packed_block_table)
+            pq_offset = off if q_offset is None else q_offset
+            pq_mask = msk if q_mask is None else q_mask
         context_attention_fwd(
             q=query, k=key, v=value, o=output, kv_cache_dtype=kv_cache_dtype, k_cache=key_cache,
             v_cache=value_cache, b_loc=block_table, b_start_loc=query_start_loc, b_seq_len=seq_lens,
             max_seq_len=max_seq_len, max_input_len=max_query_len, k_scale=k_scale, v_scale=v_scale,
             alibi_slopes=alibi_slopes, sliding_window=sliding_window, sm_scale=sm_scale,
             skip_decode=True, rotary_dim=rotary_dim, cos_sin_cache=cos_sin_cache,
-            is_neox_style=is_neox_style, is_lazy=is_lazy, q_offset=q_offset, q_mask=q_mask)
+            is_neox_style=is_neox_style, is_lazy=is_lazy, q_offset=pq_offset, q_mask=pq_mask)
     if is_lazy is None:
         is_lazy = torch.zeros(seq_lens.shape[0], dtype=torch.bool, device=query.device)
-    if q_offset is None:
-        q_offset = torch.zeros_like(block_table, dtype=torch.int32)
+    streaming = _streaming_decode_covers(query, value_cache)
+    packed = packed_block_table if streaming else None
+    if packed is None:
+        if (q_offset is None or q_mask is None) and packed_block_table is not None:
+            _, off, msk = unpack_block_table(packed_block_table)
+            q_offset = off if q_offset is None else q_offset
+            q_mask = msk if q_mask is None else q_mask
+        if q_offset is None:
+            q_offset = torch.zeros_like(block_table, dtype=torch.int32)
+    rope_freqs = None
+    if streaming and _env_flag("LAZY_DECODE_COMPUTE_COS_SIN"):           # ops/chunked...:146-151
+        rope_freqs = freqs if freqs is not None else _rope.rope_freqs(rope_meta, query.shape[2], query.device)
     _launch.launch_prefill(
         q=query, k=key, v=value, o=output, kv_cache_dtype=kv_cache_dtype, k_cache=key_cache,
         v_cache=value_cache, b_loc=block_table, b_start_loc=query_start_loc, b_seq_len=seq_lens,
@@ -63,4 +90,4 @@ def chunked_prefill_paged_decode(query, key, value, output, kv_cache_dtype, key_
         sliding_window=sliding_window, sm_scale=sm_scale, skip_decode=False,
         cos_sin_cache=cos_sin_cache, rotary_dim=rotary_dim, is_neox_style=is_neox_style,
         is_lazy=is_lazy, q_offset=q_offset, q_mask=q_mask, pos_mode=_ffi.POS_BLOCK_UNIFORM,
-        rotate_new_k=False, decode=True)
+        rotate_new_k=False, decode=True, packed_block_table=packed, rope_freqs=rope_freqs)

@@ -53,3 +53,36 @@ def build_cos_sin_cache(max_position: int, rotary_dim: int, rope_meta: dict | No
         torch.cuda.current_stream(device).cuda_stream)
     _ffi.check(rc, "lazyattn_build_cos_sin_cache")
     return out
+
+
+_freq_cache: dict = {}
+
+
+def rope_freqs(rope_meta: dict | None, head_size: int, device="cuda") -> torch.Tensor:
+    """``[head_size/2]`` float32 inverse frequencies (radians per position) on ``device``: what the
+    reference's ``rope_freqs`` evaluates inside its kernel (``cos_sin.py:24-59``), formed once on the
+    host in float64 and kept per (parameters, device).  ``inv[i] = BASE^(-2i/D)``; Llama-3: unchanged
+    where the wavelength is below ``orig/high``, divided by the factor above ``orig/low``, blended in
+    between."""
+    meta = dict(ROPE_TYPE=ROPE_DEFAULT, BASE=10000.0, SCALING_FACTOR=1.0, LOW_FACTOR=1.0,
+                HIGH_FACTOR=1.0, ORIG_MAX_POSITION=8192)
+    if rope_meta:
+        meta.update(rope_meta)
+    device = torch.device(device)
+    key = (int(meta["ROPE_TYPE"]), float(meta["BASE"]), float(meta["SCALING_FACTOR"]), float(meta["LOW_FACTOR"]),
+           float(meta["HIGH_FACTOR"]), int(meta["ORIG_MAX_POSITION"]), int(head_size), device)
+    hit = _freq_cache.get(key)
+    if hit is not None:
+        return hit
+    i = torch.arange(head_size // 2, dtype=torch.float64)
+    inv = float(meta["BASE"]) ** (-2.0 * i / head_size)
+    if int(meta["ROPE_TYPE"]) == ROPE_LLAMA3:
+        orig, low, high = float(meta["ORIG_MAX_POSITION"]), float(meta["LOW_FACTOR"]), float(meta["HIGH_FACTOR"])
+        factor = float(meta["SCALING_FACTOR"])
+        wavelen = 2.0 * math.pi / inv
+        smooth = (orig / wavelen - low) / (high - low)
+        blended = (1.0 - smooth) * inv / factor + smooth * inv
+        inv = torch.where(wavelen < orig / high, inv, torch.where(wavelen > orig / low, inv / factor, blended))
+    out = inv.to(torch.float32).to(device)
+    _freq_cache[key] = out
+    return out

@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol():
     assert set(names) == set(_ffi.EXPORTS)
     for n in names:
         assert getattr(lib, n) is not None
-    assert lib.lazyattn_abi_version() == 1
+    assert lib.lazyattn_abi_version() == 2
     assert lib.lazyattn_error_string(-4).decode().startswith("request not supported")
 
 

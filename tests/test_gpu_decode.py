@@ -52,11 +52,23 @@ def _oracle(w, lazy=None, sliding_window=0):
     return ref
 
 
-def _run(w, *, lazy=None, num_splits=0, kernel=_ffi.KERNEL_AUTO, sliding_window=0):
-    """The q_len==1 launch the entry points make, with the slicing and kernel choice exposed."""
+def _run(w, *, lazy=None, num_splits=0, kernel=_ffi.KERNEL_AUTO, sliding_window=0, packed=False, freqs=None):
+    """The q_len==1 launch the entry points make, with the slicing and kernel choice exposed.  packed: the
+    kernel is given the int64 table [block:32 | q_offset:16 | q_mask:16] and none of the three int32 tables'
+    contents (they are overwritten with junk); freqs: cos/sin computed in the kernel, no table."""
     g = w.to(DEV)
     out = torch.full_like(g.q, 5.0)
     bu = w.pos_mode == orc.POS_BLOCK_UNIFORM
+    pk = None
+    if packed:
+        pk = (g.block_table.long() << 32) | (g.q_offset.long() << 16) | g.q_mask.long()
+        g.block_table = torch.full_like(g.block_table, 1 << 20)
+        g.q_offset = torch.full_like(g.q_offset, 12345)
+        g.q_mask = torch.full_like(g.q_mask, 15)
+    fr = None
+    if freqs is not None:
+        fr = freqs.to(DEV)
+        g.cos_sin_cache = None
     _launch.launch_prefill(
         q=g.q, k=g.k, v=g.v, o=out, kv_cache_dtype=w.kv_cache_dtype, k_cache=g.k_cache, v_cache=g.v_cache,
         b_loc=g.block_table, b_start_loc=g.b_start_loc, b_seq_len=g.b_seq_len, max_input_len=1,
@@ -65,7 +77,7 @@ def _run(w, *, lazy=None, num_splits=0, kernel=_ffi.KERNEL_AUTO, sliding_window=
         is_neox_style=True, is_lazy=None if lazy is None else lazy.to(DEV),
         q_offset=g.q_offset if bu else None, q_mask=g.q_mask,
         pos_mode=_ffi.POS_BLOCK_UNIFORM if bu else _ffi.POS_NATURAL, rotate_new_k=not bu, decode=True,
-        kernel=kernel, num_splits=num_splits)
+        kernel=kernel, num_splits=num_splits, packed_block_table=pk, rope_freqs=fr)
     return out.cpu()
 
 
@@ -267,3 +279,104 @@ def test_decode_entry_points_long_context():
                   g.max_seq_len, 1, g.k_scale, g.v_scale, sm_scale=128 ** -0.5, rotary_dim=128,
                   cos_sin_cache=g.cos_sin_cache, is_lazy=g.is_lazy, q_offset=g.q_offset, q_mask=g.q_mask)
         assert _err(out.cpu(), ref) < 2e-2, (variant, _err(out.cpu(), ref))
+
+
+def _with_zero_offsets(w):
+    """Entries of the offset table set to 0 where the reference's page walk then keeps the previous page's rotation:
+    the second and later pages of documents (rotated like their first page)."""
+    qo = w.q_offset.clone()
+    for b in range(qo.shape[0]):
+        row = qo[b].tolist()
+        for j in range(1, len(row)):
+            if row[j] == row[j - 1] and row[j] > 1 and j % 3:
+                qo[b, j] = 0
+        # (row[] keeps the original values, so runs longer than two pages get several zeros)
+    assert (qo != w.q_offset).any()
+    return qo
+
+
+@pytest.mark.parametrize("nsplit", [1, 5])
+@pytest.mark.parametrize("kernel,dtype,d", [(_ffi.KERNEL_AUTO, torch.bfloat16, 128), (_ffi.KERNEL_GENERIC, torch.float32, 64)])
+def test_decode_zero_offset_keeps_previous_rotation(kernel, dtype, d, nsplit):
+    """ops/models/llama_v1.py:207-262: the query is re-rotated only when a page's offset differs from the previous
+    page's, and an offset of 0 does nothing -- such a page is rotated like the one before it.  With the page axis
+    cut into slices a slice may start on such a page and has to look back for the offset in force."""
+    print(f"case: decode offset-0 carry kernel={kernel} {dtype} nsplit={nsplit}", flush=True)
+    w = _decode_batch("block_uniform", dtype=dtype, d=d)
+    same = _oracle(w)
+    w.q_offset = _with_zero_offsets(w)
+    ref = _oracle(w)
+    assert _err(ref, same) < 1e-6                      # zeros inside a document change nothing ...
+    got = _run(w, num_splits=nsplit, kernel=kernel)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    assert _err(got, ref) < tol, _err(got, ref)
+    w.q_offset[:, 0] = 0                              # ... and before the first non-zero entry there is no rotation
+    ref0 = _oracle(w)
+    assert _err(ref0, ref) > 1e-3
+    got = _run(w, num_splits=nsplit, kernel=kernel)
+    assert _err(got, ref0) < tol, _err(got, ref0)
+
+
+@pytest.mark.parametrize("variant", ["natural", "block_uniform"])
+@pytest.mark.parametrize("bs", [16, 32])
+def test_decode_reads_the_packed_table(variant, bs):
+    """The int64 table of ops/models/llama_v1.py:157-160 read in place (one 8-byte entry per page): same result as
+    with the three int32 tables, which hold junk here."""
+    print(f"case: decode packed table {variant} page={bs}", flush=True)
+    w = _decode_batch(variant, bs=bs)
+    if variant == "block_uniform":
+        w.q_offset = _with_zero_offsets(w)
+    ref = _oracle(w)
+    for nsplit in (1, 4):
+        got = _run(w, num_splits=nsplit, packed=True)
+        assert _err(got, ref) < 2e-2, (nsplit, _err(got, ref))
+
+
+@pytest.mark.parametrize("variant", ["natural", "block_uniform"])
+@pytest.mark.parametrize("llama3", [False, True])
+@pytest.mark.parametrize("dtype,d,kv", [(torch.bfloat16, 128, "auto"), (torch.float16, 64, "auto"), (torch.bfloat16, 96, "fp8")])
+def test_decode_computed_cos_sin(variant, llama3, dtype, d, kv):
+    """cos/sin computed in the kernel from the inverse frequencies (rope_freqs / rope_cos_sin_from_freqs,
+    model_executor/rope/cos_sin.py:24-66; the reference's COMPUTE_COS_SIN switch) against the oracle reading a
+    table built in float64: plain and Llama-3-smoothed frequencies."""
+    from lazy_amd.model_executor.rope import cos_sin as rope_cs
+    print(f"case: decode computed cos/sin {variant} llama3={llama3} {dtype} d={d} kv={kv}", flush=True)
+    l3 = dict(scaling_factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0, orig_max_position=8192) if llama3 else None
+    w = wl.make_workload("cdec", dtype=dtype, hq=8, hkv=2, d=d, theta=500000.0, block_size=16,
+                         doc_lens=[40, 16, 333, 700, 5, 128, 97], requests=[[3, 1, 0], [2], [0, 2, 3, 1, 5, 6, 4, 5, 6], [4, 0]],
+                         q_lens=[1, 1, 1, 1], variant=variant, seed=5, kv_cache_dtype=kv, llama3=l3)
+    x = w.k_cache.shape[4]
+    for b in range(4):
+        n = int(w.b_seq_len[b]) - 1
+        pb = int(w.block_table[b, n // 16]); qs = int(w.b_start_loc[b])
+        enc = (lambda t, sc: (t.float() / sc).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8)) if kv == "fp8" else (lambda t, sc: t)
+        w.k_cache[pb, :, :, n % 16, :] = enc(w.k[qs], w.k_scale).view(2, d // x, x)
+        w.v_cache[pb, :, :, n % 16] = enc(w.v[qs], w.v_scale)
+    ref = _oracle(w)
+    meta = dict(ROPE_TYPE=1, BASE=500000.0, SCALING_FACTOR=8.0, LOW_FACTOR=1.0, HIGH_FACTOR=4.0, ORIG_MAX_POSITION=8192) \
+        if llama3 else dict(ROPE_TYPE=0, BASE=500000.0)
+    freqs = rope_cs.rope_freqs(meta, d, DEV)
+    tol = 5e-2 if kv == "fp8" else (5e-3 if dtype == torch.float16 else 2e-2)
+    for nsplit in (1, 3):
+        got = _run(w, num_splits=nsplit, freqs=freqs)
+        assert _err(got, ref) < tol, (nsplit, _err(got, ref))
+
+
+def test_computed_cos_sin_at_long_positions():
+    """Positions in the tens of thousands (the long-context configuration reaches 65 791): the angle is reduced to one
+    revolution from an exact product, so the computed values agree with a float64 table to the table's own rounding."""
+    from lazy_amd.model_executor.rope import cos_sin as rope_cs
+    print("case: decode computed cos/sin, positions to 66K", flush=True)
+    w = wl.make_workload("cdecl", dtype=torch.bfloat16, hq=8, hkv=2, d=128, theta=500000.0, block_size=16,
+                         doc_lens=[16] * 8, requests=[[0, 1, 2, 3, 4, 5, 6, 7]], q_lens=[1], variant="block_uniform", seed=6)
+    n = int(w.b_seq_len[0]) - 1
+    pb = int(w.block_table[0, n // 16])
+    w.k_cache[pb, :, :, n % 16, :] = w.k[0].view(2, 16, 8)
+    w.v_cache[pb, :, :, n % 16] = w.v[0]
+    # the eight documents are moved far out: offsets 65 000 + 100 i (+1 for the bias), table to match
+    for i in range(8):
+        w.q_offset[0, i] = 65001 + 100 * i
+    w.cos_sin_cache = orc.build_cos_sin_table(66000, 128, 500000.0).to(torch.bfloat16)      # float64 angles
+    ref = _oracle(w)
+    got = _run(w, freqs=rope_cs.rope_freqs(dict(ROPE_TYPE=0, BASE=500000.0), 128, DEV))
+    assert _err(got, ref) < 2e-2, _err(got, ref)
