@@ -28,6 +28,7 @@
 // second kernel merges them.
 #include "common.hpp"
 #include "elem16.hpp"
+#include <atomic>
 
 namespace lazyattn {
 
@@ -1083,13 +1084,14 @@ static int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt,
     auto kern = prefill_mfma_kernel<NC, HD, FP8, WIN, PAD, T, TT>;
     constexpr int LDS_BYTES = lds_bytes<HD>(NC);
     // the attribute belongs to the device's copy of the kernel: once per device, on the caller's current device
-    static bool attr_set[64] = {};
+    // (any host thread may call: the flag is atomic, and setting the attribute twice is harmless)
+    static std::atomic<bool> attr_set[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return LAZYATTN_E_LAUNCH;
-    if (!attr_set[dev]) {
+    if (!attr_set[dev].load(std::memory_order_acquire)) {
         if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
             return LAZYATTN_E_LAUNCH;
-        attr_set[dev] = true;
+        attr_set[dev].store(true, std::memory_order_release);
     }
     const int64_t nb = (int64_t)p.num_kv_heads * nsplit * (mt_total > 0 ? (int64_t)mt_total : (int64_t)p.batch * n_mt);
     if (nb <= 0 || nb > 0x7fffffff) return LAZYATTN_E_SHAPE;
