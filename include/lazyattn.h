@@ -50,7 +50,8 @@ enum {
     LAZYATTN_E_DTYPE = -3,       /* unsupported type combination */
     LAZYATTN_E_UNSUPPORTED = -4, /* valid request the selected kernel cannot run */
     LAZYATTN_E_WORKSPACE = -5,   /* workspace missing or too small */
-    LAZYATTN_E_LAUNCH = -6       /* hipLaunchKernel failed */
+    LAZYATTN_E_LAUNCH = -6,      /* hipLaunchKernel failed */
+    LAZYATTN_E_SCRATCH_LIMIT = -7 /* lazyattn_prefix_prefill_static_scratch: the call needs more than the static buffer holds */
 };
 
 /* Arguments of one prefix-prefill call.  Replaces the Triton launch in
@@ -131,6 +132,17 @@ size_t lazyattn_prefill_workspace_bytes(const lazyattn_prefill_params *p);
 /* Deferred-RoPE prefix-prefill attention.  Replaces `_fwd_kernel[grid](...)`
  * (old_ops/prefix_prefill.py:493, ops/prefix_prefill.py:683). `stream` is a hipStream_t. */
 int lazyattn_prefix_prefill(const lazyattn_prefill_params *p, void *stream);
+
+/* lazyattn_prefix_prefill() for callers that cannot allocate device memory or hand over a workspace: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the
+ * reference.  Same arguments and results; `workspace` / `workspace_bytes` are ignored and the split-KV
+ * partials go to a buffer of lazyattn_static_scratch_bytes() (32 MiB) that the library holds statically in
+ * each GPU's memory until the process ends.  A call that would need more returns
+ * LAZYATTN_E_SCRATCH_LIMIT (lazyattn_prefill_workspace_bytes() tells beforehand).  Allocates nothing.  All
+ * calls on one GPU share that buffer: calls that overlap in time on one GPU (two streams) race; calls on one
+ * stream, or otherwise ordered, are safe -- every partial a call merges was written by that call. */
+int lazyattn_prefix_prefill_static_scratch(const lazyattn_prefill_params *p, void *stream);
+size_t lazyattn_static_scratch_bytes(void);
 
 /* q_len == 1 rows: every key (the new token included) comes from the paged cache.
  * pos_mode NATURAL: each key is rotated at its natural position; replaces

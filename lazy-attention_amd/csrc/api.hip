@@ -1,5 +1,6 @@
 // C ABI: argument checks and kernel selection.  Nothing here allocates or synchronises.
 #include "common.hpp"
+#include <mutex>
 
 namespace lazyattn {
 int launch_prefill_generic(const lazyattn_prefill_params &p, int decode, hipStream_t stream);
@@ -86,6 +87,51 @@ extern "C" int lazyattn_prefix_prefill(const lazyattn_prefill_params *p, void *s
     }
     if (kernel == LAZYATTN_KERNEL_GENERIC) return launch_prefill_generic(*p, 0, s);
     return LAZYATTN_E_UNSUPPORTED;
+}
+
+// ---- the prefill call for callers that may not allocate ----
+// Split-KV partials of lazyattn_prefix_prefill_static_scratch() live in this array instead of a caller-provided
+// workspace.  One copy per GPU the library runs on, held until the process ends.  In host code the array's name
+// is only a handle: its device address is asked for once per device (with that device current) and kept.
+namespace {
+constexpr size_t STATIC_SCRATCH_BYTES = 32u << 20;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+constexpr int MAX_DEVICES = 64;
+std::mutex scratch_mutex;
+void *scratch_ptr[MAX_DEVICES] = {};
+
+int static_scratch_address(void **out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return LAZYATTN_E_LAUNCH;
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (!scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return LAZYATTN_E_LAUNCH;
+        scratch_ptr[dev] = ptr;
+    }
+    *out = scratch_ptr[dev];
+    return LAZYATTN_OK;
+}
+}  // namespace
+
+extern "C" size_t lazyattn_static_scratch_bytes(void) { return STATIC_SCRATCH_BYTES; }
+
+extern "C" int lazyattn_prefix_prefill_static_scratch(const lazyattn_prefill_params *p, void *stream) {
+    int rc = check_common(p, false);
+    if (rc != LAZYATTN_OK) return rc;
+    const size_t need = lazyattn_prefill_workspace_bytes(p);
+    if (need > STATIC_SCRATCH_BYTES) return LAZYATTN_E_SCRATCH_LIMIT;
+    lazyattn_prefill_params q = *p;
+    q.workspace = nullptr;
+    q.workspace_bytes = 0;
+    if (need > 0) {
+        void *ptr = nullptr;
+        rc = static_scratch_address(&ptr);
+        if (rc != LAZYATTN_OK) return rc;
+        q.workspace = ptr;                      // the kernels take the address as they take a caller's workspace
+        q.workspace_bytes = (int64_t)STATIC_SCRATCH_BYTES;
+    }
+    return lazyattn_prefix_prefill(&q, stream);
 }
 
 extern "C" int lazyattn_paged_decode_rotary(const lazyattn_prefill_params *p, void *stream) {
@@ -219,6 +265,7 @@ extern "C" const char *lazyattn_error_string(int code) {
         case LAZYATTN_E_UNSUPPORTED: return "request not supported by the selected kernel";
         case LAZYATTN_E_WORKSPACE: return "workspace missing or too small";
         case LAZYATTN_E_LAUNCH: return "kernel launch failed";
+        case LAZYATTN_E_SCRATCH_LIMIT: return "the call needs more split-KV scratch than the library's static buffer holds";
         default: return "unknown error";
     }
 }

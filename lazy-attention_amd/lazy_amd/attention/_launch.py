@@ -137,3 +137,11 @@ class PrefillPlan:
                        "lazyattn_paged_decode_rotary")
         else:
             _ffi.check(self._lib.lazyattn_prefix_prefill(self.params, stream), "lazyattn_prefix_prefill")
+
+    def run_static_scratch(self) -> None:
+        """The same prefill call through the entry point that allocates nothing: the split-KV partials go to
+        the library's static per-GPU buffer instead of this plan's workspace."""
+        assert not self.decode
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        _ffi.check(self._lib.lazyattn_prefix_prefill_static_scratch(self.params, stream),
+                   "lazyattn_prefix_prefill_static_scratch")
