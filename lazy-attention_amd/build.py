@@ -14,7 +14,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT_DIR = os.path.join(HERE, "lazy_amd", "_lib")
 LIB = os.path.join(OUT_DIR, "liblazyattn.so")
-SOURCES = ["api.hip", "prefill_generic.hip", "prefill_mfma.hip", "paged_decode.hip", "rope_cache_write.hip", "rotation_metadata.hip", "block_reposition.hip", "rope_table.hip"]
+SOURCES = ["prefill_mfma_bf16.hip", "prefill_mfma_bf16_e4m3.hip", "prefill_mfma_bf16_e5m2.hip", "prefill_mfma_f16.hip",
+           "prefill_mfma_f16_e4m3.hip", "prefill_mfma_f16_e5m2.hip", "api.hip", "prefill_generic.hip", "prefill_mfma.hip", "paged_decode.hip", "rope_cache_write.hip", "rotation_metadata.hip", "block_reposition.hip", "rope_table.hip"]
 # packed-fp32 VALU forms are kept off on purpose: some have produced wrong results on
 # this hardware pool; scalar fp32 code is used throughout.
 # No -ffast-math: the fp32 kernel needs IEEE expf/division and every kernel relies on

@@ -1,894 +1,16 @@
-// Deferred-RoPE prefix-prefill attention on the gfx950 matrix cores (bf16 MFMA).
-//
-// Work decomposition.  The query rows that share one kv-head -- `group` q-heads x q_len
-// tokens -- are cut into units of 32 rows (one q-head, 32 consecutive tokens).  A
-// workgroup of NW waves owns NW consecutive units (unit = chunk * group + head_in_group,
-// so with group = 4 the four heads of one token chunk sit side by side) and a slice of
-// the key axis (split-KV).  Every 64-key tile of paged K is therefore gathered from HBM,
-// rotated and written to LDS ONCE for all NW*32 rows, instead of once per q-head as the
-// reference's grid (batch, q_head, m_tile) does (ops/prefix_prefill.py:681-682).
-//
-// Per 64-key tile:
-//   gather   4 pages of K ([D/x][16][x], one contiguous 4 KB run per page and kv-head for
-//            bf16) with 16-byte loads off a wave-uniform base, the matching cos/sin rows,
-//            and 4 pages of V ([D][16]);
-//   rotate   k1*c - k2*s, k1*s + k2*c in fp32 registers, one rounding to bf16
-//            (old_ops/prefix_prefill.py:248-257 with FORCE_FP32_ROTARY), write to LDS in
-//            the cache's own [page][D/8][slot][8] order, which is exactly the A-operand
-//            order of v_mfma_f32_32x32x16_bf16;
-//   S^T      = K . Q^T (keys x rows) in two 32-key halves, Q fragments re-read from LDS;
-//   softmax  per lane one query row; Q carries sm_scale*log2(e) and the accumulators start at
-//            minus a per-row reference, so P = exp2(S) directly; the row max (one
-//            v_permlane32_swap) only decides when that reference moves (old_ops:287-291);
-//   O^T     += V^T . P^T: the S^T accumulator registers ARE the B operand (the k index of
-//            the MFMA is permuted so that no shuffle is needed), V^T comes from LDS.
-// Tiles come in three kinds: full context tiles (no masking code at all), edge context
-// tiles (pad slots / end of context) and new-token tiles (old_ops:326-396, causal mask).
-// With more than one split every workgroup writes (O/l, log2-sum-exp) partials and a
-// second kernel merges them.
-#include "common.hpp"
-#include "elem16.hpp"
-#include <atomic>
+// Host side of the matrix-core prefill path: which workgroup shape and how many key-axis splits a call gets, the
+// merge of the split partials, and the launch.  The kernel itself is in prefill_mfma_kernel.hpp.
+#include "prefill_mfma_kernel.hpp"
 
 namespace lazyattn {
 
-namespace {
-
-
-constexpr int BS = 16;          // page size (tokens)
-constexpr int NT = 64;          // keys per tile
-constexpr int PAGES = NT / BS;  // pages per tile
-constexpr int UNIT = 32;        // query rows per wave
-// LDS tiles (bytes).  K: [page][d8 = 16][slot = 16][8 bf16].
-// V: [page][g = 2][d = 128][slots 4g..4g+3 | slots 8+4g..8+4g+3] -- the 16 bytes one lane
-// feeds to the PV MFMA as its A operand.
-// Sizes that follow from the head size HD (128 or 64); a K page is HD * 32 bytes, a V page as well.
-template <int HD> struct Geo {
-    static constexpr int K_PAGE = HD * 32, K_TILE = PAGES * K_PAGE;
-    static constexpr int V_G = HD * 16, V_PAGE = 2 * V_G, V_TILE = PAGES * V_PAGE;
-    static constexpr int KV_BYTES = 2 * K_TILE + 2 * V_TILE;      // K and V tiles, double-buffered: 64 KB at 128
-    static constexpr int Q_WAVE = HD * 64;                        // Q^T fragments of one computing wave
-    static constexpr int KS = HD / 16, DT = HD / 32;              // k-steps of K.Q^T, 32-row blocks of O^T
-    static constexpr int K_ITEMS = HD / 64, V_ITEMS = HD / 32;    // 16-byte items per gathering lane and page
-    static constexpr int PAIR = (HD / 16) * 256;                  // bytes from the chunk of d to the chunk of d + HD/2 (16-bit cache)
-    static constexpr int PAIR8 = (HD / 32) * 256;                 // ... in an fp8 page
-};
-
-enum { TILE_FULL = 0, TILE_EDGE = 1, TILE_NEW = 2 };
-
-// value of x in the partner lane (lane ^ 32) of the wave, via v_permlane32_swap
-// IEEE-754 maximum of three (v_maximum3_f32): NaN-propagating, so no canonicalising pre-pass
-__device__ __forceinline__ float max3(float a, float b, float c) {
-    return __builtin_elementwise_maximum(__builtin_elementwise_maximum(a, b), c);
-}
-__device__ __forceinline__ float partner32(float x, bool upper) {
-    uint32_t a = __float_as_uint(x), b = a;
-    asm volatile("" : "+v"(b));      // two distinct registers for the swap
-    auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
-    // r[0] = {a.lo, b.lo}, r[1] = {a.hi, b.hi}
-    return __uint_as_float(upper ? r[0] : r[1]);
-}
-__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
-
-__device__ __forceinline__ uint4 ldg16(const uint8_t *base, uint32_t off) {
-    return *reinterpret_cast<const uint4 *>(base + off);
-}
-__device__ __forceinline__ uint2 ldg8(const uint8_t *base, uint32_t off) {
-    return *reinterpret_cast<const uint2 *>(base + off);
-}
-
-// 8 consecutive cos (or sin) table entries
-template <typename TT> struct TabVec {                     // a 16-bit table
-    uint4 v;
-    __device__ __forceinline__ void load(const uint8_t *base, uint32_t off) { v = ldg16(base, off); }
-    __device__ __forceinline__ void fill(float w) { const uint32_t u = Elem<TT>::splat(w); v = make_uint4(u, u, u, u); }
-    __device__ __forceinline__ void get(float *f) const {
-        f[0] = Elem<TT>::lo(v.x); f[1] = Elem<TT>::hi(v.x); f[2] = Elem<TT>::lo(v.y); f[3] = Elem<TT>::hi(v.y);
-        f[4] = Elem<TT>::lo(v.z); f[5] = Elem<TT>::hi(v.z); f[6] = Elem<TT>::lo(v.w); f[7] = Elem<TT>::hi(v.w);
-    }
-};
-template <> struct TabVec<float> {
-    float4 a, b;
-    __device__ __forceinline__ void load(const uint8_t *base, uint32_t off) {
-        a = *reinterpret_cast<const float4 *>(base + off);
-        b = *reinterpret_cast<const float4 *>(base + off + 16);
-    }
-    __device__ __forceinline__ void fill(float w) { a = make_float4(w, w, w, w); b = a; }
-    __device__ __forceinline__ void get(float *f) const {
-        f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
-    }
-};
-
-template <typename T> __device__ __forceinline__ void unpack8(const uint4 &w, float *f) {
-    f[0] = Elem<T>::lo(w.x); f[1] = Elem<T>::hi(w.x); f[2] = Elem<T>::lo(w.y); f[3] = Elem<T>::hi(w.y);
-    f[4] = Elem<T>::lo(w.z); f[5] = Elem<T>::hi(w.z); f[6] = Elem<T>::lo(w.w); f[7] = Elem<T>::hi(w.w);
-}
-// two fp8 bytes (the low 16 bits of w) -> two floats; KIND 1: e4m3, 2: e5m2
-template <int KIND> __device__ __forceinline__ f32x2_t cvt_fp8x2(uint32_t w) {
-    if constexpr (KIND == 2) return __builtin_amdgcn_cvt_pk_f32_bf8(w, false);
-    else return __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
-}
-// 8 fp8 bytes -> (float * scale) rounded to the query type, as floats  (old_ops:239-241)
-template <typename T, int KIND> __device__ __forceinline__ void unpack8_fp8(uint32_t lo, uint32_t hi, float scale, float *f) {
-    const f32x2_t a = cvt_fp8x2<KIND>(lo), b = cvt_fp8x2<KIND>(lo >> 16);
-    const f32x2_t c = cvt_fp8x2<KIND>(hi), d = cvt_fp8x2<KIND>(hi >> 16);
-    const float t[8] = {a[0], a[1], b[0], b[1], c[0], c[1], d[0], d[1]};
-#pragma unroll
-    for (int i = 0; i < 8; ++i) f[i] = round_to<T>(t[i] * scale);
-}
-
-// one K item in flight: 8 (d, d+64) pairs of one key
-template <typename TT> struct KRegs {
-    uint4 k1, k2;
-    TabVec<TT> c, s;
-    uint32_t lds_off;
-};
-
-}  // namespace
-
-// Workgroup = 8 waves: waves 0-3 compute (32 query rows each), waves 4-7 gather.  The
-// hardware places wave w on SIMD w % 4, so every SIMD hosts one computing and one
-// gathering wave: the gather's address arithmetic, fp32 rotation and LDS writes run in
-// the shadow of the other wave's MFMAs, and neither role ever waits for the other's
-// memory latency -- they only meet at one barrier per tile.
-// NC = computing waves = 32-row units per workgroup: 8 (12 waves, three per SIMD) for long
-// key ranges, 4 (8 waves) when the call is small and more, lighter workgroups fill the chip
-// with fewer key-axis splits.
-template <int HD> constexpr int lds_bytes(int nc) { return Geo<HD>::KV_BYTES + nc * Geo<HD>::Q_WAVE + 2 * PAGES * 4; }   // + Q^T fragments (re-read every tile) + page limits
-
-// WIN: built with the sliding-window code (calls without a window run the instantiation without it)
-// PAD: the head size is a multiple of 16 below HD = 128: Q, K and V sit zero-padded in the 128-wide tiles, the two
-// halves of the real head at (0 .., 64 ..) so that the rotation pairs stay (d, 64 + d)
-template <int NC, int HD, int FP8, bool WIN, bool PAD, typename T, typename TT>
-__global__ void __launch_bounds__((NC + 4) * 64)
-prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int n_mt, const int mt_total) {
-    using G = Geo<HD>;
-    constexpr int D = HD, HALF = HD / 2;
-    const int Dr = PAD ? p.head_dim : D, HALFr = Dr / 2, CPr = Dr / 16;   // real head size, its half, its chunk pairs
-    constexpr int K_PAGE = G::K_PAGE, K_TILE = G::K_TILE, V_G = G::V_G, V_PAGE = G::V_PAGE, V_TILE = G::V_TILE;
-    constexpr int KV_BYTES = G::KV_BYTES, KS = G::KS, DT = G::DT;
-    constexpr int KI = G::K_ITEMS, VI = G::V_ITEMS;   // a page has HD K items (HD/16 chunk pairs x 16 slots) and 2 HD V items
-    constexpr int VI_CTX = FP8 ? VI / 2 : VI;        // an fp8 page row of 16 slots is one 16-byte item
-    constexpr uint32_t TSZ = sizeof(TT);
-    using E = Elem<T>;
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = uniform(tid >> 6);              // in an SGPR: everything derived from it stays scalar
-    const bool gatherer = wave >= NC;
-
-    // ---- work item: the m-tiles of one (request, kv-head, split) land on the same XCD ----
-    const int group = p.num_q_heads / p.num_kv_heads;
-    int mt, split, g, b;
-    if (mt_total > 0) {
-        // Compact list: the grid holds (kv head, split, I) for I below a host-side bound on the number of m-tiles
-        // of all requests together; I is resolved to (request, m-tile) here from the token offsets.  Used when
-        // most (request, m-tile) pairs of the plain mapping would be empty: requests with one new token next to
-        // a long one.  Workgroups of one kv head stay on one XCD.
-        const int L = blockIdx.x, hkv = p.num_kv_heads;
-        int q;
-        if ((hkv & 7) == 0) { g = (L & 7) + 8 * ((L >> 3) % (hkv >> 3)); q = (L >> 3) / (hkv >> 3); }
-        else { g = L % hkv; q = L / hkv; }
-        split = q % nsplit;
-        const int item = q / nsplit;
-        int base = 0;
-        b = -1; mt = 0;
-        // 256 requests per round, four per lane: their offsets are requested together (one memory round trip),
-        // the m-tile counts are summed per lane, scanned over the wave, and the hit is located inside its lane
-        for (int c = 0; c < p.batch; c += 256) {
-            const int r0 = c + lane * 4;
-            int64_t off[5];
-#pragma unroll
-            for (int j = 0; j < 5; ++j) {
-                const int rb = r0 + j;
-                off[j] = load_index(p.b_start_loc, rb < p.batch ? rb : p.batch, p.index_bits);
-            }
-            int cn[4], tot = 0;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int ql = r0 + j < p.batch ? (int)(off[j + 1] - off[j]) : 0;
-                cn[j] = (ql > 0 && !(p.skip_decode && ql == 1)) ? (((ql + UNIT - 1) / UNIT) * group + NC - 1) / NC : 0;
-                tot += cn[j];
-            }
-            int incl = tot;                                       // inclusive prefix sum over the wave
-#pragma unroll
-            for (int d = 1; d < 64; d <<= 1) {
-                const int up = __shfl_up(incl, d);
-                if (lane >= d) incl += up;
-            }
-            const uint64_t hit = __builtin_amdgcn_ballot_w64(base + incl > item);
-            if (hit) {
-                const int idx = __builtin_ctzll(hit);
-                int rem = item - (base + __builtin_amdgcn_readlane(incl - tot, idx));
-                const int c0 = __builtin_amdgcn_readlane(cn[0], idx), c1 = __builtin_amdgcn_readlane(cn[1], idx),
-                          c2 = __builtin_amdgcn_readlane(cn[2], idx);
-                int j = 0;
-                if (rem >= c0) { rem -= c0; j = 1; if (rem >= c1) { rem -= c1; j = 2; if (rem >= c2) { rem -= c2; j = 3; } } }
-                b = c + idx * 4 + j;
-                mt = rem;
-                break;
-            }
-            base += __builtin_amdgcn_readlane(incl, 63);
-        }
-        if (b < 0) return;
-        b = uniform(b); mt = uniform(mt);
-    } else {
-        const int n_groups = p.batch * p.num_kv_heads * nsplit;
-        int kvgrp;
-        const int L = blockIdx.x;
-        if (((p.batch * p.num_kv_heads) & 7) == 0) {
-            // every split and m-tile of one (request, kv-head) on one XCD: they share K/V through its L2
-            const int xcd = L & 7, q = L >> 3;
-            mt = q % n_mt;
-            const int r = q / n_mt;
-            kvgrp = ((r / nsplit) * 8 + xcd) * nsplit + r % nsplit;
-        } else if ((n_groups & 7) == 0) {
-            const int xcd = L & 7, q = L >> 3;
-            mt = q % n_mt;
-            kvgrp = (q / n_mt) * 8 + xcd;
-        } else {
-            mt = L % n_mt;
-            kvgrp = L / n_mt;
-        }
-        split = kvgrp % nsplit;
-        g = (kvgrp / nsplit) % p.num_kv_heads;
-        b = kvgrp / (nsplit * p.num_kv_heads);
-    }
-
-    const int64_t qs = load_index(p.b_start_loc, b, p.index_bits);
-    const int q_len = (int)(load_index(p.b_start_loc, b + 1, p.index_bits) - qs);
-    const int ctx_len = (int)(load_index(p.b_seq_len, b, p.index_bits) - q_len);
-    if (q_len <= 0 || ctx_len < 0) return;
-    if (p.skip_decode && q_len == 1) return;                     // old_ops:109-110
-    const int n_chunks = (q_len + UNIT - 1) / UNIT;
-    const int n_units = n_chunks * group;
-    if (mt * NC >= n_units) return;                              // block_mask, old_ops:322-328
-    const bool lazy_b = p.is_lazy ? p.is_lazy[b] != 0 : true;
-    const int pos_mode = p.pos_mode;
-    const bool vanilla = pos_mode == LAZYATTN_POS_BLOCK_UNIFORM && !lazy_b;   // ops:398
-    const bool use_qmask = !vanilla && p.q_mask != nullptr;
-    const int n_pages = (ctx_len + BS - 1) / BS;
-    int t_end;                                                   // new-token keys [0, t_end) are visible here
-    {
-        int last_unit = mt * NC + NC - 1;
-        if (last_unit > n_units - 1) last_unit = n_units - 1;
-        const int te = (last_unit / group + 1) * UNIT;
-        t_end = te < q_len ? te : q_len;
-    }
-    const int n_ctx_tiles = (n_pages + PAGES - 1) / PAGES;
-    const int n_new_tiles = (t_end + NT - 1) / NT;
-    // The key axis is cut into nsplit ranges of equal estimated cost.  A new-token tile costs about
-    // three context tiles (element-wise V scatter, per-row causal masks, branchy loads), and all of them
-    // sit at the end: with equal tile counts the last split was the tail of every launch.
-    constexpr int NEW_COST = 3;
-    // Sliding window (old_ops:270-284, 373-376): the row at sequence position P sees the keys at positions
-    // P - window + 1 .. P only.  Positions: context slot n -> n, new token m -> ctx_len + m.  The tiles that
-    // lie entirely before the window of the workgroup's first row are not visited at all.
-    const int window = WIN ? p.sliding_window : 0;
-    int skip_ctx = 0, skip_new = 0;                 // whole context / new-token tiles before every window
-    if (window) {
-        const int first_row = ((mt * NC) / group) * UNIT;
-        const int lo_min = ctx_len + first_row - window + 1;
-        if (lo_min > 0) {
-            skip_ctx = lo_min < ctx_len ? lo_min / NT : n_ctx_tiles;
-            if (lo_min >= ctx_len) skip_new = (lo_min - ctx_len) / NT;
-            if (skip_new > n_new_tiles) skip_new = n_new_tiles;
-        }
-    }
-    const int live_ctx = n_ctx_tiles - skip_ctx, live_new = n_new_tiles - skip_new;
-    const int64_t cost = live_ctx + (int64_t)NEW_COST * live_new;
-    auto tile_at = [&](int64_t c) -> int {         // first tile whose cost interval ends after c
-        return skip_ctx + skip_new + (c <= live_ctx ? (int)c : live_ctx + (int)((c - live_ctx) / NEW_COST));
-    };
-    const int tile_begin = tile_at(cost * split / nsplit);
-    const int tile_end = split + 1 == nsplit ? n_ctx_tiles + n_new_tiles : tile_at(cost * (split + 1) / nsplit);
-
-    // ---- page metadata, fetched ahead of its use ----
-    // Gathering wave w owns page w of every tile, so it needs one block-table entry, one
-    // q_offset and one q_mask per tile.  They are read through the scalar unit (constant address
-    // space): the values are wave-uniform, land in SGPRs, and waiting for them never drains the
-    // vector loads in flight.  Branch-free on purpose (a branch around a load makes the compiler
-    // drain every outstanding load at the join): pages past the context read entry n_pages-1
-    // and get limit 0; an absent q_offset / q_mask array is replaced by the block table, masked to 0.
-    struct PageMeta { int bt, qo, lim; };      // physical block, q_offset, number of valid slots
-    typedef const int32_t __attribute__((address_space(4))) *sptr_i32;
-    const bool use_qo = !vanilla && pos_mode != LAZYATTN_POS_NATURAL;
-    const sptr_i32 bt_row = (sptr_i32)(p.block_table + b * p.bt_stride[0]);
-    const sptr_i32 qo_row = use_qo ? (sptr_i32)(p.q_offset + b * p.qo_stride[0]) : bt_row;
-    const sptr_i32 qm_row = use_qmask ? (sptr_i32)(p.q_mask + b * p.qm_stride[0]) : bt_row;
-    const int64_t bt_s1 = p.bt_stride[1];
-    const int64_t qo_s1 = use_qo ? p.qo_stride[1] : p.bt_stride[1];
-    const int64_t qm_s1 = use_qmask ? p.qm_stride[1] : p.bt_stride[1];
-    const int qo_and = use_qo ? -1 : 0, qm_and = use_qmask ? -1 : 0;
-    // A cache page of 32 slots is handled as two parts of 16: "page" j below is the j-th run of 16 context
-    // slots, part j & 1 of cache page j >> 1.  Its valid slots follow from the page's pad count.
-    const int pshift = p.block_size == 2 * BS ? 1 : 0, part_mask = pshift;
-    const int cache_bs = BS << pshift;
-    auto load_page = [&](int j) -> PageMeta {
-        PageMeta m;
-        int jc = j < n_pages ? j : n_pages - 1;
-        jc = jc < 0 ? 0 : jc;
-        const int pj = jc >> pshift;
-        m.bt = bt_row[pj * bt_s1];
-        m.qo = qo_row[pj * qo_s1] & qo_and;
-        const int qm = qm_row[pj * qm_s1] & qm_and;                                  // old_ops:165-167
-        const int ql = cache_bs - qm - (j & part_mask) * BS;                         // valid slots of this part
-        int l = ctx_len - j * BS;
-        l = l < ql ? l : ql;
-        l = l > BS ? BS : l;
-        m.lim = l < 0 ? 0 : l;
-        return m;
-    };
-    // Valid-slot counts of the four pages of a context tile, one int per page and LDS buffer:
-    // written by the gathering waves with the tile, read by the computing waves for the masks.
-    int *page_lims = reinterpret_cast<int *>(lds + KV_BYTES + NC * G::Q_WAVE);
-
-    if (gatherer) {
-        // ====================================================================== gather
-        const int gw = wave - NC;                                // this wave's page of every tile
-        const int nat_step = (vanilla || pos_mode == LAZYATTN_POS_BLOCK_UNIFORM) ? 0 : BS;
-        const bool rot_new = p.rotate_new_k && !vanilla;
-        const float k_scale = FP8 ? *p.k_scale : 1.f;
-        const float v_scale = FP8 ? *p.v_scale : 1.f;
-        const uint8_t *kc_base = (const uint8_t *)p.k_cache + (int64_t)g * p.kc_stride[1] * (FP8 ? 1 : 2);
-        const uint8_t *vc_base = (const uint8_t *)p.v_cache + (int64_t)g * p.vc_stride[1] * (FP8 ? 1 : 2);
-        const int64_t kc_page_bytes = p.kc_stride[0] * (FP8 ? 1 : 2);
-        const int64_t vc_page_bytes = p.vc_stride[0] * (FP8 ? 1 : 2);
-        const uint8_t *tab_base = (const uint8_t *)p.cos_sin_cache;
-        const uint32_t row_bytes = (uint32_t)p.table_stride * TSZ;
-        // per-token rotation of context pages reads the packed table [2][D/16][rows][8]: the 16
-        // slots of a page are 16 consecutive 16-byte chunks there
-        const bool per_token = !vanilla && pos_mode != LAZYATTN_POS_BLOCK_UNIFORM;
-        const bool packed_tab = p.cos_sin_packed != nullptr && per_token;
-        const uint8_t *ctab_base = packed_tab ? (const uint8_t *)p.cos_sin_packed : tab_base;
-        const uint32_t pos_bytes = packed_tab ? 8 * TSZ : row_bytes;       // bytes per unit of position
-        const uint32_t sin_delta = packed_tab ? (uint32_t)(HALFr / 8) * (uint32_t)p.packed_rows * 8 * TSZ : HALFr * TSZ;
-        // this wave's part of its cache pages (pages of 32 slots: the tile's pages 0, 1 are the two parts of
-        // one cache page, 2, 3 of the next): first slot, and the position step that goes with it
-        const int slot0 = (gw & part_mask) * BS;
-        const int part_pos = nat_step ? slot0 : 0;               // block-uniform: one position for the whole page
-        // K items of a page: 128 = (8 chunks of 8 (d, d+64) pairs) x 16 slots, two per lane
-        uint32_t k_toff[KI];
-        // Cache offsets of a lane's items: item i = item 0 + i * (a wave-uniform stride), so one offset register
-        // serves all of them and the strides go into the scalar page base.
-        // K bf16: [D/8][slots][8] -> item (cp, o) at (cp*slots + o)*16 bytes, cp = lane/16 + 4 i
-        //   fp8 : [D/16][slots][16] -> 8 bytes at chunk cp/2, half cp&1
-        // V bf16: row d = lane/2 + 32 i of `slots` slots, 8 slots (16 bytes) per item; fp8: row d = lane + 64 i, 16 slots
-        const uint32_t k_goff = FP8 ? (uint32_t)(((lane >> 5) * cache_bs + slot0 + (lane & 15)) * 16 + ((lane >> 4) & 1) * 8)
-                                    : (uint32_t)(((lane >> 4) * cache_bs + slot0 + (lane & 15)) * 16);
-        const uint32_t k_item = (uint32_t)((FP8 ? 2 : 4) * cache_bs * 16);
-        const uint32_t v_goff = FP8 ? (uint32_t)(lane * cache_bs + slot0)
-                                    : (uint32_t)((lane >> 1) * cache_bs * 2 + slot0 * 2 + (lane & 1) * 16);
-        const uint32_t v_item = (uint32_t)(64 * cache_bs);
-        // bytes from the chunk of d to the chunk of d + HD/2 in the cache page
-        const uint32_t pair = (uint32_t)(FP8 ? G::PAIR8 : G::PAIR) << pshift;
-#pragma unroll
-        for (int i = 0; i < KI; ++i) {
-            const int idx = lane + i * 64;
-            const int o = idx & 15, cp = PAD && (idx >> 4) >= CPr ? 0 : idx >> 4;   // (a padded chunk reads chunk 0 and is zeroed)
-            // block-uniform rotation and un-rotated requests use one table row for the whole page
-            k_toff[i] = packed_tab ? ((uint32_t)cp * (uint32_t)p.packed_rows + (uint32_t)o) * 8 * TSZ
-                                   : (per_token ? (uint32_t)o * row_bytes : 0u) + (uint32_t)cp * 8 * TSZ;
-        }
-        // PAD: per-item cache offsets (the chunk of d + Dr/2 is not a fixed distance away in an fp8 page) and
-        // which of the lane's items exist
-        uint32_t pk1[PAD ? KI : 1], pk2[PAD ? KI : 1], pv[PAD ? VI_CTX : 1];
-        bool pk_ok[PAD ? KI : 1], pv_ok[PAD ? VI_CTX : 1];
-        if constexpr (PAD) {
-#pragma unroll
-            for (int i = 0; i < KI; ++i) {
-                const int idx = lane + i * 64, o = idx & 15;
-                pk_ok[i] = (idx >> 4) < CPr;
-                const int c1 = pk_ok[i] ? idx >> 4 : 0, c2 = CPr + c1;                  // 8-element chunks of d and d + Dr/2
-                pk1[i] = FP8 ? (uint32_t)(((c1 >> 1) * cache_bs + slot0 + o) * 16 + (c1 & 1) * 8) : (uint32_t)((c1 * cache_bs + slot0 + o) * 16);
-                pk2[i] = FP8 ? (uint32_t)(((c2 >> 1) * cache_bs + slot0 + o) * 16 + (c2 & 1) * 8) : (uint32_t)((c2 * cache_bs + slot0 + o) * 16);
-            }
-#pragma unroll
-            for (int i = 0; i < VI_CTX; ++i) {
-                const int idx = lane + i * 64;
-                const int d = FP8 ? idx : idx >> 1;
-                pv_ok[i] = d < Dr;
-                const int dc = pv_ok[i] ? d : 0;
-                pv[i] = FP8 ? (uint32_t)(dc * cache_bs + slot0) : (uint32_t)(dc * cache_bs * 2 + slot0 * 2 + (idx & 1) * 16);
-            }
-        }
-        KRegs<TT> kr[KI];
-        uint4 vr[VI];
-
-        // ---- loads of a context page: no branch, no zero fill ----
-        auto issue_loads_ctx = [&](int tile, const PageMeta &pm) {
-            const int j = tile * PAGES + gw;
-            const uint8_t *kb = kc_base + pm.bt * kc_page_bytes;
-            // Position of the page's first slot.  Natural: j*16 (old_ops:183-184); offset: q_offset-1 if
-            // set, else natural (old_ops:186-191); block-uniform: q_offset-1 if set, else 0 (ops:180-186);
-            // un-rotated requests read row 0 of the table (cos 1, sin 0): exact identity.  pm.qo is 0
-            // wherever q_offset is not consulted, nat_step is 0 wherever the fallback is row 0.
-            // A page past the context (its slots are all masked) takes the last page's position: the
-            // table only has to cover the positions of real keys.
-            const int jp = j < n_pages ? j : n_pages - 1;
-            const int pos0 = pm.qo ? pm.qo - 1 + part_pos : jp * nat_step;
-            const uint8_t *tb = ctab_base + (int64_t)pos0 * pos_bytes;
-#pragma unroll
-            for (int i = 0; i < KI; ++i) {
-                kr[i].lds_off = (uint32_t)(gw * K_PAGE + (lane + i * 64) * 16);
-                if constexpr (PAD) {
-                    uint4 k1, k2;
-                    if (FP8) {
-                        const uint2 a = ldg8(kb, pk1[i]), a2 = ldg8(kb, pk2[i]);
-                        k1 = make_uint4(a.x, a.y, 0, 0);
-                        k2 = make_uint4(a2.x, a2.y, 0, 0);
-                    } else {
-                        k1 = ldg16(kb, pk1[i]);
-                        k2 = ldg16(kb, pk2[i]);
-                    }
-                    const uint4 z = make_uint4(0, 0, 0, 0);
-                    kr[i].k1 = pk_ok[i] ? k1 : z;
-                    kr[i].k2 = pk_ok[i] ? k2 : z;
-                } else if (FP8) {
-                    const uint2 a = ldg8(kb + i * k_item, k_goff), a2 = ldg8(kb + i * k_item + pair, k_goff);
-                    kr[i].k1 = make_uint4(a.x, a.y, 0, 0);
-                    kr[i].k2 = make_uint4(a2.x, a2.y, 0, 0);
-                } else {
-                    kr[i].k1 = ldg16(kb + i * k_item, k_goff);
-                    kr[i].k2 = ldg16(kb + i * k_item + pair, k_goff);
-                }
-                kr[i].c.load(tb, k_toff[i]);
-                kr[i].s.load(tb, k_toff[i] + sin_delta);
-            }
-            const uint8_t *vb = vc_base + pm.bt * vc_page_bytes;
-#pragma unroll
-            for (int i = 0; i < VI_CTX; ++i) {
-                if constexpr (PAD) {
-                    const uint4 t = ldg16(vb, pv[i]);
-                    vr[i] = pv_ok[i] ? t : make_uint4(0, 0, 0, 0);
-                } else {
-                    vr[i] = ldg16(vb + i * v_item, v_goff);
-                }
-            }
-        };
-        // ---- loads of this wave's 16 keys of a new-token tile ----
-        auto issue_loads_new = [&](int tile) {
-            const int m0 = (tile - n_ctx_tiles) * NT + gw * BS;
-#pragma unroll
-            for (int i = 0; i < KI; ++i) {
-                const int idx = lane + i * 64;
-                const int cp = idx & (D / 16 - 1), kl = idx / (D / 16), m = m0 + kl;
-                kr[i].lds_off = (uint32_t)(gw * K_PAGE + cp * 256 + kl * 16);
-                uint4 k1 = make_uint4(0, 0, 0, 0), k2 = k1;
-                TabVec<TT> c, sn;
-                c.fill(1.f); sn.fill(0.f);
-                if (m < t_end && (!PAD || cp < CPr)) {
-                    const T *kn = (const T *)p.k + (qs + m) * p.k_stride[0] + (int64_t)g * p.k_stride[1] + cp * 8;
-                    k1 = *reinterpret_cast<const uint4 *>(kn);
-                    k2 = *reinterpret_cast<const uint4 *>(kn + HALFr);
-                    if (rot_new) {                                               // old_ops:342-343
-                        const uint8_t *tb = tab_base + (int64_t)(ctx_len + m) * row_bytes;
-                        c.load(tb, (uint32_t)cp * 8 * TSZ);
-                        sn.load(tb, (uint32_t)cp * 8 * TSZ + HALFr * TSZ);
-                    }
-                }
-                kr[i].k1 = k1; kr[i].k2 = k2; kr[i].c = c; kr[i].s = sn;
-            }
-#pragma unroll
-            for (int i = 0; i < VI; ++i) {
-                const int idx = lane + i * 64;
-                const int dc = idx & (D / 8 - 1), m = m0 + idx / (D / 8);
-                // (the value is chosen before the one store: a store under the branch lets the compiler merge
-                // the iterations' stores behind a pointer phi, and the array then stays in scratch memory)
-                uint4 t = make_uint4(0, 0, 0, 0);
-                if (m < t_end && (!PAD || dc * 8 < Dr))
-                    t = *reinterpret_cast<const uint4 *>((const T *)p.v + (qs + m) * p.v_stride[0] +
-                                                         (int64_t)g * p.v_stride[1] + dc * 8);
-                vr[i] = t;
-            }
-        };
-        // kind of this wave's part of a tile, and its loads
-        auto issue_loads = [&](int tile, const PageMeta &pm) -> int {
-            if (tile >= n_ctx_tiles) { issue_loads_new(tile); return TILE_NEW; }
-            issue_loads_ctx(tile, pm);                     // pages past the context re-read the last page: harmless
-            if (pm.lim == BS) return TILE_FULL;
-            if (tile * PAGES + gw >= n_pages) {
-#pragma unroll
-                for (int i = 0; i < KI; ++i) { kr[i].k1 = make_uint4(0, 0, 0, 0); kr[i].k2 = kr[i].k1; }
-            }
-            return TILE_EDGE;
-        };
-        // ---- rotate the K items in fp32 and write them to a K tile ----
-        auto store_k = [&](uint8_t *ktile, int kind) {
-#pragma unroll
-            for (int i = 0; i < KI; ++i) {
-                float a[8], bb[8], cs[8], sn[8];
-                if (FP8 && kind != TILE_NEW) {
-                    unpack8_fp8<T, FP8>(kr[i].k1.x, kr[i].k1.y, k_scale, a);
-                    unpack8_fp8<T, FP8>(kr[i].k2.x, kr[i].k2.y, k_scale, bb);
-                } else {
-                    unpack8<T>(kr[i].k1, a);
-                    unpack8<T>(kr[i].k2, bb);
-                }
-                kr[i].c.get(cs);
-                kr[i].s.get(sn);
-                float x[8], y[8];
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    x[e] = a[e] * cs[e] - bb[e] * sn[e];                             // old_ops:253
-                    y[e] = a[e] * sn[e] + bb[e] * cs[e];                             // old_ops:254
-                }
-                *reinterpret_cast<uint4 *>(ktile + kr[i].lds_off) = make_uint4(
-                    E::pack(x[0], x[1]), E::pack(x[2], x[3]), E::pack(x[4], x[5]), E::pack(x[6], x[7]));
-                *reinterpret_cast<uint4 *>(ktile + kr[i].lds_off + G::PAIR) = make_uint4(
-                    E::pack(y[0], y[1]), E::pack(y[2], y[3]), E::pack(y[4], y[5]), E::pack(y[6], y[7]));
-            }
-        };
-        // ---- write the V items to a V tile; lim = valid slots of the page ----
-        auto store_v = [&](uint8_t *vtile, int kind, int lim) {
-            if (kind == TILE_NEW) {
-                // item = 8 d of one new-token key: scatter 2-byte entries
-#pragma unroll
-                for (int i = 0; i < VI; ++i) {
-                    const int idx = lane + i * 64;
-                    const int dc = idx & (D / 8 - 1), slot = idx / (D / 8);
-                    uint8_t *dst = vtile + gw * V_PAGE + ((slot >> 2) & 1) * V_G + (dc * 8) * 16 + (slot >> 3) * 8 +
-                                   (slot & 3) * 2;
-                    const uint32_t w[4] = {vr[i].x, vr[i].y, vr[i].z, vr[i].w};
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        *reinterpret_cast<uint16_t *>(dst + (2 * e) * 16) = (uint16_t)(w[e] & 0xffffu);
-                        *reinterpret_cast<uint16_t *>(dst + (2 * e + 1) * 16) = (uint16_t)(w[e] >> 16);
-                    }
-                }
-                return;
-            }
-#pragma unroll
-            for (int i = 0; i < VI_CTX; ++i) {
-                const int idx = lane + i * 64;
-                if (FP8) {
-                    // 16 fp8 slots of one d: entry g=0 <- slots 0-3 | 8-11, entry g=1 <- slots 4-7 | 12-15
-                    const int d = idx;
-                    const uint32_t w[4] = {vr[i].x, vr[i].y, vr[i].z, vr[i].w};
-                    uint32_t o2[4][2];
-#pragma unroll
-                    for (int q4 = 0; q4 < 4; ++q4) {
-                        const f32x2_t lo = cvt_fp8x2<FP8>(w[q4]);
-                        const f32x2_t hi = cvt_fp8x2<FP8>(w[q4] >> 16);
-                        float f[4] = {lo[0] * v_scale, lo[1] * v_scale, hi[0] * v_scale, hi[1] * v_scale};
-                        if (kind == TILE_EDGE) {
-#pragma unroll
-                            for (int s = 0; s < 4; ++s)
-                                if (q4 * 4 + s >= lim) f[s] = 0.f;   // masked slots contribute nothing, whatever they hold
-                        }
-                        o2[q4][0] = E::pack(f[0], f[1]);
-                        o2[q4][1] = E::pack(f[2], f[3]);
-                    }
-                    uint8_t *dst = vtile + gw * V_PAGE + d * 16;
-                    *reinterpret_cast<uint4 *>(dst) = make_uint4(o2[0][0], o2[0][1], o2[2][0], o2[2][1]);
-                    *reinterpret_cast<uint4 *>(dst + V_G) = make_uint4(o2[1][0], o2[1][1], o2[3][0], o2[3][1]);
-                } else {
-                    // 8 bf16 slots (8*hf ..) of one d: slots +0..3 -> entry g=0, +4..7 -> entry g=1, half hf
-                    const int d = idx >> 1, hf = idx & 1;
-                    uint4 v = vr[i];
-                    if (kind == TILE_EDGE) {
-                        uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            if (hf * 8 + 2 * e >= lim) w[e] &= 0xffff0000u;
-                            if (hf * 8 + 2 * e + 1 >= lim) w[e] &= 0x0000ffffu;
-                        }
-                        v = make_uint4(w[0], w[1], w[2], w[3]);
-                    }
-                    uint8_t *dst = vtile + gw * V_PAGE + d * 16 + hf * 8;
-                    *reinterpret_cast<uint2 *>(dst) = make_uint2(v.x, v.y);
-                    *reinterpret_cast<uint2 *>(dst + V_G) = make_uint2(v.z, v.w);
-                }
-            }
-        };
-        // tile + its page limit -> LDS buffer `buf`
-        auto store_tile = [&](int buf, int kind, int lim) {
-            store_k(lds + buf * K_TILE, kind);
-            store_v(lds + 2 * K_TILE + buf * V_TILE, kind, lim);
-            if (lane == 0) page_lims[buf * PAGES + gw] = lim;
-        };
-
-        // At the top of iteration `tile` the raw K/V of tile+1 sit in registers (loaded during
-        // the previous iteration); they are rotated into the other LDS buffer while the
-        // computing waves work on `tile`, then the loads of tile+2 are issued.
-        int nxt_kind = TILE_FULL, nxt_lim = BS;
-        PageMeta pm_pend = load_page((tile_begin + 2) * PAGES + gw);
-        if (tile_begin < tile_end) {
-            const PageMeta pm0 = load_page(tile_begin * PAGES + gw);
-            const PageMeta pm1 = load_page((tile_begin + 1) * PAGES + gw);
-            const int k0 = issue_loads(tile_begin, pm0);
-            store_tile(0, k0, pm0.lim);
-            if (tile_begin + 1 < tile_end) {
-                nxt_kind = issue_loads(tile_begin + 1, pm1);
-                nxt_lim = pm1.lim;
-            }
-        }
-        __syncthreads();
-        int tile = tile_begin;
-        while (tile < tile_end) {
-            // steady state: this wave's pages of tile+1 (in registers) and tile+2 (to load) are full context pages
-            while (tile + 2 < n_ctx_tiles && tile + 2 < tile_end && nxt_kind == TILE_FULL && pm_pend.lim == BS) {
-                const int cur = (tile - tile_begin) & 1;
-                const PageMeta pm_new = load_page((tile + 3) * PAGES + gw);      // scalar loads, land during the rotation
-                store_tile(cur ^ 1, TILE_FULL, BS);
-                issue_loads_ctx(tile + 2, pm_pend);
-                pm_pend = pm_new;
-                ++tile;
-                __syncthreads();
-            }
-            if (tile >= tile_end) break;
-            const int cur = (tile - tile_begin) & 1;
-            if (tile + 1 < tile_end) store_tile(cur ^ 1, nxt_kind, nxt_lim);
-            int new_kind = TILE_FULL;
-            if (tile + 2 < tile_end) new_kind = issue_loads(tile + 2, pm_pend);
-            nxt_kind = new_kind;
-            nxt_lim = pm_pend.lim;
-            pm_pend = load_page((tile + 3) * PAGES + gw);
-            ++tile;
-            __syncthreads();
-        }
-        return;
-    }
-
-    // ========================================================================== compute
-    const int l32 = lane & 31, gh = lane >> 5;
-    const int unit = mt * NC + wave;
-    const bool active = unit < n_units;
-    const int chunk = active ? unit / group : 0;
-    const int h = g * group + (active ? unit % group : 0);
-    const int t0 = chunk * UNIT;
-    const int row = t0 + l32;                                    // token index of this lane's query row
-    const bool row_ok = active && row < q_len;
-
-    // Q^T fragments: B operand of S^T = K.Q^T, lane = (row l32, d = ks*16 + gh*8 .. +8).
-    // They live in this wave's own LDS slice (not in registers: three waves share a SIMD's
-    // register file) and are re-read for every tile.
-    // Q is multiplied by sm_scale * log2(e) here, once, and rounded to bf16 again: the MFMA then
-    // delivers the scores in log2 units and no per-score multiply is left in the tile loop (the
-    // reference scales the fp32 scores, old_ops:287; the extra rounding of Q is one more relative
-    // 2^-9 per element, like the one the rotated K already carries).
-    const float cs2 = p.sm_scale * 1.4426950408889634f;
-    uint8_t *qlds = lds + KV_BYTES + wave * G::Q_WAVE + lane * 16;
-    {
-        const T *qp = (const T *)p.q + (qs + row) * p.q_stride[0] + (int64_t)h * p.q_stride[1] + gh * 8;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if constexpr (PAD) {
-                // tile column c = ks*16 + gh*8: real element c (first half of the head) or Dr/2 + c - 64 (second)
-                const int c = ks * 16 + gh * 8, lo = c & 63;
-                if (row_ok && lo < HALFr) v = *reinterpret_cast<const uint4 *>(qp - gh * 8 + (c < 64 ? lo : HALFr + lo));
-            } else {
-                if (row_ok) v = *reinterpret_cast<const uint4 *>(qp + ks * 16);
-            }
-            float f[8];
-            unpack8<T>(v, f);
-            *reinterpret_cast<uint4 *>(qlds + ks * 1024) =
-                make_uint4(E::pack(f[0] * cs2, f[1] * cs2), E::pack(f[2] * cs2, f[3] * cs2),
-                           E::pack(f[4] * cs2, f[5] * cs2), E::pack(f[6] * cs2, f[7] * cs2));
-        }
-    }
-    // Online softmax against a reference m_ref per row that moves rarely.  The MFMA accumulators of S^T
-    // start at -m_ref, so the scores arrive already relative to it and P = exp2(S) needs no subtraction.
-    // m_ref is moved (and O, l rescaled, old_ops:287-291) only when a row's tile maximum exceeds it by more
-    // than REBASE, or when the row sees its first valid key; in between P may exceed 1 (by at most
-    // 2^REBASE), which fp32 accumulation and bf16's exponent range carry without loss.
-    constexpr float REBASE = E::REBASE;
-    float m_ref = 0.f, l_run = 0.f, l_alt = 0.f;                    // row sum kept as two chains
-    bool seen = false;                                              // the row has had a valid key
-    f32x16_t cinit;                                                 // -m_ref in every element
-#pragma unroll
-    for (int i = 0; i < 16; ++i) cinit[i] = 0.f;
-    f32x16_t acc[DT];
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[dt][i] = 0.f;
-
-    // ---- S^T = K . Q^T for one 64-key tile: two independent 32-key accumulation chains ----
-    auto qk_tile = [&](const uint8_t *ktile, f32x16_t &s0, f32x16_t &s1) {
-        const uint8_t *kp = ktile + (l32 >> 4) * K_PAGE + gh * 256 + (l32 & 15) * 16;
-        // A wave in a matrix phase goes first on its SIMD: its MFMAs are issued the moment the pipe is
-        // free and the vector work of the other waves fills the cycles in between (measured: -3 % on
-        // long key ranges against equal priorities).
-        __builtin_amdgcn_s_setprio(2);
-        // operands are requested two k-steps ahead of their MFMAs (a ring of three sets): one step ahead
-        // leaves the LDS latency exposed in every step
-        uint4 a0[3], a1[3], q[3];
-        auto fetch = [&](int ks) {
-            a0[ks % 3] = *reinterpret_cast<const uint4 *>(kp + ks * 512);
-            a1[ks % 3] = *reinterpret_cast<const uint4 *>(kp + 2 * K_PAGE + ks * 512);
-            q[ks % 3] = *reinterpret_cast<const uint4 *>(qlds + ks * 1024);
-        };
-        fetch(0);
-        fetch(1);
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            if (ks + 2 < KS) fetch(ks + 2);
-            s0 = E::mfma(a0[ks % 3], q[ks % 3], ks ? s0 : cinit);
-            s1 = E::mfma(a1[ks % 3], q[ks % 3], ks ? s1 : cinit);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        __builtin_amdgcn_s_setprio(0);
-    };
-    // ---- masks: register i of half `sub` holds key sub*32 + 8*(i/4) + 4*gh + i%4 ----
-    // key0 = sequence position of the tile's first key (only used under a sliding window)
-    auto mask_half = [&](f32x16_t &s, uint32_t vbits, int sub, int kind, int m0, int key0) {
-        const uint32_t w = vbits >> (4 * gh);
-        // causal: key m0 + kk <= row  <=>  8*(i/4) + i%4 <= row - m0 - sub*32 - 4*gh   (old_ops:371-372)
-        const int lim = kind == TILE_NEW ? row - m0 - sub * 32 - 4 * gh : 64;
-        // window: key0 + sub*32 + 4*gh + kb >= ctx_len + row - window + 1
-        const int lb = window ? ctx_len + row - window + 1 - key0 - sub * 32 - 4 * gh : -64;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int kb = 8 * (i >> 2) + (i & 3);
-            const bool ok = ((w >> kb) & 1u) && kb <= lim && (!WIN || kb >= lb);
-            s[i] = ok ? s[i] : -INFINITY;
-        }
-    };
-    // ---- tile maximum per row; move the reference if a row needs it (rare after its first tile) ----
-    auto rebase = [&](f32x16_t &s0, f32x16_t &s1) {
-        // v_maximum3_f32: no quieting pre-pass over the MFMA results, NaN scores stay NaN
-        float ma = max3(s0[0], s0[1], s0[2]), mb = max3(s1[0], s1[1], s1[2]);
-#pragma unroll
-        for (int i = 3; i < 15; i += 2) { ma = max3(ma, s0[i], s0[i + 1]); mb = max3(mb, s1[i], s1[i + 1]); }
-        float mx = max3(ma, mb, s0[15]);
-        mx = max3(mx, s1[15], s1[15]);
-        mx = max3(mx, partner32(mx, gh != 0), mx);                  // relative to m_ref; -inf: no valid key in this tile
-        const bool valid = mx > -INFINITY;                          // false for NaN too: NaN rows stay NaN below
-        const float delta = (valid && (!seen || mx > REBASE)) ? mx : 0.f;
-        if (__builtin_amdgcn_ballot_w64(delta != 0.f)) {
-            const float alpha = seen ? __builtin_amdgcn_exp2f(-delta) : 1.f;   // nothing accumulated before the first key
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) acc[dt] *= alpha;
-            l_run *= alpha;
-            l_alt *= alpha;
-            s0 -= delta;
-            s1 -= delta;
-            m_ref += delta;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) cinit[i] = -m_ref;
-        }
-        seen = seen || valid;
-    };
-    // ---- P = exp2(S) for 32 keys (S is relative to m_ref), packed as the two B operands of the PV steps ----
-    auto exp_half = [&](const f32x16_t &s, uint4 &p0, uint4 &p1) {
-        float pr[16];
-#pragma unroll
-        for (int i = 0; i < 16; ++i) pr[i] = __builtin_amdgcn_exp2f(s[i]);
-        uint32_t w[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) w[i] = E::pack(pr[2 * i], pr[2 * i + 1]);
-        // row sum of the rounded probabilities, two per instruction (old_ops:312 sums them unrounded)
-#pragma unroll
-        for (int i = 0; i < 8; i += 2) { l_run = E::dot2_ones(w[i], l_run); l_alt = E::dot2_ones(w[i + 1], l_alt); }
-        p0 = make_uint4(w[0], w[1], w[2], w[3]);
-        p1 = make_uint4(w[4], w[5], w[6], w[7]);
-    };
-    // ---- O^T += V^T . P^T for 32 keys (pages 2*sub, 2*sub+1 of the tile) ----
-    // k index j of a 16-key step <-> slot 4*gh + j (j < 4), 8 + 4*gh + j - 4 (j >= 4)
-    auto pv_half = [&](const uint8_t *vtile, int sub, const uint4 &p0, const uint4 &p1) {
-        const uint8_t *vp = vtile + (sub * 2) * V_PAGE + gh * V_G + l32 * 16;
-        // 2 DT MFMAs: the 32-row blocks of d for the first page of the half, then for the second;
-        // their V^T operands are requested two MFMAs ahead
-        uint4 a[3];
-        auto fetch = [&](int j) { a[j % 3] = *reinterpret_cast<const uint4 *>(vp + (j / DT) * V_PAGE + (j % DT) * 512); };
-        fetch(0);
-        fetch(1);
-#pragma unroll
-        for (int j = 0; j < 2 * DT; ++j) {
-            if (j + 2 < 2 * DT) fetch(j + 2);
-            acc[j % DT] = E::mfma(a[j % 3], j < DT ? p0 : p1, acc[j % DT]);
-        }
-    };
-    auto attend = [&](const uint8_t *vtile, f32x16_t &s0, f32x16_t &s1) {
-        rebase(s0, s1);
-        uint4 p0, p1, p2, p3;
-        exp_half(s0, p0, p1);
-        __builtin_amdgcn_s_setprio(2);
-        pv_half(vtile, 0, p0, p1);
-        exp_half(s1, p2, p3);
-        pv_half(vtile, 1, p2, p3);
-        __builtin_amdgcn_s_setprio(0);
-    };
-
-    // which of the tile's 64 keys exist: new-token tiles from the token count, context tiles from the
-    // page limits the gathering waves left beside the tile
-    struct Desc { int kind; uint32_t vlo, vhi; int m0, key0; };
-    auto describe = [&](int tile, int cur) -> Desc {
-        Desc td{TILE_FULL, ~0u, ~0u, 0, tile * NT};
-        if (tile >= n_ctx_tiles) {
-            td.kind = TILE_NEW;
-            td.m0 = (tile - n_ctx_tiles) * NT;
-            td.key0 = ctx_len + td.m0;
-            const int n = t_end - td.m0;
-            const uint64_t valid = n >= 64 ? ~0ull : (n <= 0 ? 0ull : ((1ull << n) - 1ull));
-            td.vlo = (uint32_t)valid; td.vhi = (uint32_t)(valid >> 32);
-        } else {
-            const int4 lims = *reinterpret_cast<const int4 *>(page_lims + cur * PAGES);
-            const int l0 = uniform(lims.x), l1 = uniform(lims.y), l2 = uniform(lims.z), l3 = uniform(lims.w);
-            if ((l0 & l1 & l2 & l3) != BS) {
-                td.kind = TILE_EDGE;
-                td.vlo = ((1u << l0) - 1u) | (((1u << l1) - 1u) << BS);
-                td.vhi = ((1u << l2) - 1u) | (((1u << l3) - 1u) << BS);
-            }
-        }
-        // a tile that starts before the window of this wave's last row needs the per-row lower bound
-        if (window && td.kind == TILE_FULL && td.key0 < ctx_len + t0 + UNIT - window) td.kind = TILE_EDGE;
-        return td;
-    };
-    __syncthreads();
-    for (int tile = tile_begin; tile < tile_end; ++tile) {
-        const int cur = (tile - tile_begin) & 1;
-        const uint8_t *ktile = lds + cur * K_TILE;
-        const uint8_t *vtile = lds + 2 * K_TILE + cur * V_TILE;
-        const Desc td = describe(tile, cur);
-        // One call site for the tile body: the accumulators keep their registers round the loop.
-        // Rows of an idle wave are all-zero queries (harmless, never stored); a new-token tile
-        // entirely in this wave's future contributes nothing (causal) and is skipped.
-        if (td.kind != TILE_NEW || td.m0 <= t0 + UNIT - 1) {
-            f32x16_t s0, s1;
-            qk_tile(ktile, s0, s1);
-            if (td.kind != TILE_FULL) {
-                mask_half(s0, td.vlo, 0, td.kind, td.m0, td.key0);
-                mask_half(s1, td.vhi, 1, td.kind, td.m0, td.key0);
-            }
-            attend(vtile, s0, s1);
-        }
-        __syncthreads();
-    }
-
-    // ---- epilogue ----
-    l_run += l_alt;
-    l_run += partner32(l_run, gh != 0);
-    if (!row_ok) return;
-    const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
-    if (nsplit == 1) {
-        T *op = (T *)p.o + (qs + row) * p.o_stride[0] + (int64_t)h * p.o_stride[1];
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int i4 = 0; i4 < 4; ++i4) {
-                const int d = dt * 32 + 8 * i4 + 4 * gh;
-                if (PAD && d >= Dr) continue;                                  // padding columns of the tile
-                *reinterpret_cast<uint2 *>(op + d) =
-                    make_uint2(E::pack(acc[dt][4 * i4] * inv, acc[dt][4 * i4 + 1] * inv),
-                               E::pack(acc[dt][4 * i4 + 2] * inv, acc[dt][4 * i4 + 3] * inv));
-            }
-    } else {
-        // Partial row = 128 halves sharing one power-of-two scale (the row's largest |O/l| lands in
-        // [0.5, 1)) + (log2-sum-exp, scale) as two floats: half the bytes of an fp32 row, written by every
-        // workgroup at the same moment and read back by the merge, for an error of at most 2^-12 of the
-        // row's largest element -- an eighth of the rounding of the bf16 output.
-        float am = 0.f;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int i = 0; i < 16; i += 2) am = max3(am, fabsf(acc[dt][i]), fabsf(acc[dt][i + 1]));
-        am = fmaxf(am, partner32(am, gh != 0)) * inv;
-        uint32_t eb = (__float_as_uint(am) >> 23) & 0xffu;           // biased exponent: am in [2^(eb-127), 2^(eb-126))
-        eb = eb > 252u ? 252u : eb;
-        const float down = __uint_as_float((253u - eb) << 23) * inv;   // 2^-(eb-126) / l
-        const float up = __uint_as_float((eb + 1u) << 23);            // 2^(eb-126)
-        const int64_t NTOK = p.num_tokens;
-        _Float16 *wo = (_Float16 *)p.workspace;
-        float2 *wl = reinterpret_cast<float2 *>(wo + (int64_t)nsplit * NTOK * p.num_q_heads * D);
-        const int64_t r_idx = ((int64_t)split * NTOK + (qs + row)) * p.num_q_heads + h;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int i4 = 0; i4 < 4; ++i4) {
-                const int d = dt * 32 + 8 * i4 + 4 * gh;
-                const f32x2_t lo = {acc[dt][4 * i4] * down, acc[dt][4 * i4 + 1] * down};
-                const f32x2_t hi = {acc[dt][4 * i4 + 2] * down, acc[dt][4 * i4 + 3] * down};
-                const f16x2_t hl = __builtin_convertvector(lo, f16x2_t), hh = __builtin_convertvector(hi, f16x2_t);   // RNE
-                *reinterpret_cast<uint2 *>(wo + r_idx * D + d) =
-                    make_uint2(*reinterpret_cast<const uint32_t *>(&hl), *reinterpret_cast<const uint32_t *>(&hh));
-            }
-        if (gh == 0)
-            wl[r_idx] = make_float2(l_run > 0.f ? m_ref + __builtin_amdgcn_logf(l_run) : -INFINITY, up);
-    }
-}
+// instantiated in prefill_mfma_<type>[_<fp8 kind>].hip
+extern template int launch_mfma_family<bf16_t, 0>(const lazyattn_prefill_params &, int, int, int, int, hipStream_t);
+extern template int launch_mfma_family<bf16_t, 1>(const lazyattn_prefill_params &, int, int, int, int, hipStream_t);
+extern template int launch_mfma_family<bf16_t, 2>(const lazyattn_prefill_params &, int, int, int, int, hipStream_t);
+extern template int launch_mfma_family<f16_t, 0>(const lazyattn_prefill_params &, int, int, int, int, hipStream_t);
+extern template int launch_mfma_family<f16_t, 1>(const lazyattn_prefill_params &, int, int, int, int, hipStream_t);
+extern template int launch_mfma_family<f16_t, 2>(const lazyattn_prefill_params &, int, int, int, int, hipStream_t);
 
 // ---- merge split-KV partials: one 16-lane group (head size 128) per (token, q-head) row ----
 // The few fields the merge needs, not the whole parameter block: a launch with ~450 bytes of kernel
@@ -1079,50 +201,6 @@ size_t mfma_workspace_bytes(const lazyattn_prefill_params &p) {
     return (size_t)ns * (size_t)p.num_tokens * p.num_q_heads * partial_row_bytes(p);
 }
 
-template <int NC, int HD, int FP8, bool WIN, bool PAD, typename T, typename TT>
-static int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt, int mt_total, hipStream_t stream) {
-    auto kern = prefill_mfma_kernel<NC, HD, FP8, WIN, PAD, T, TT>;
-    constexpr int LDS_BYTES = lds_bytes<HD>(NC);
-    // the attribute belongs to the device's copy of the kernel: once per device, on the caller's current device
-    // (any host thread may call: the flag is atomic, and setting the attribute twice is harmless)
-    static std::atomic<bool> attr_set[64];
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return LAZYATTN_E_LAUNCH;
-    if (!attr_set[dev].load(std::memory_order_acquire)) {
-        if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess)
-            return LAZYATTN_E_LAUNCH;
-        attr_set[dev].store(true, std::memory_order_release);
-    }
-    const int64_t nb = (int64_t)p.num_kv_heads * nsplit * (mt_total > 0 ? (int64_t)mt_total : (int64_t)p.batch * n_mt);
-    if (nb <= 0 || nb > 0x7fffffff) return LAZYATTN_E_SHAPE;
-    hipLaunchKernelGGL(kern, dim3((unsigned)nb), dim3((NC + 4) * 64), LDS_BYTES, stream, p, nsplit, n_mt, mt_total);
-    return hipGetLastError() == hipSuccess ? LAZYATTN_OK : LAZYATTN_E_LAUNCH;
-}
-
-template <int NC, int HD, bool WIN, bool PAD, typename T>
-static int launch_mfma_hd(const lazyattn_prefill_params &p, int nsplit, int n_mt, int mt_total, hipStream_t stream) {
-    const bool t32 = p.table_dtype == LAZYATTN_F32;
-    // cache pages: 0 the element type, 1 fp8 e4m3, 2 fp8 e5m2
-    if (p.cache_dtype == LAZYATTN_FP8_E4M3)
-        return t32 ? launch_mfma_t<NC, HD, 1, WIN, PAD, T, float>(p, nsplit, n_mt, mt_total, stream)
-                   : launch_mfma_t<NC, HD, 1, WIN, PAD, T, T>(p, nsplit, n_mt, mt_total, stream);
-    if (p.cache_dtype == LAZYATTN_FP8_E5M2)
-        return t32 ? launch_mfma_t<NC, HD, 2, WIN, PAD, T, float>(p, nsplit, n_mt, mt_total, stream)
-                   : launch_mfma_t<NC, HD, 2, WIN, PAD, T, T>(p, nsplit, n_mt, mt_total, stream);
-    return t32 ? launch_mfma_t<NC, HD, 0, WIN, PAD, T, float>(p, nsplit, n_mt, mt_total, stream)
-               : launch_mfma_t<NC, HD, 0, WIN, PAD, T, T>(p, nsplit, n_mt, mt_total, stream);
-}
-template <int NC, typename T>
-static int launch_mfma_nc(const lazyattn_prefill_params &p, int nsplit, int n_mt, int mt_total, hipStream_t stream) {
-    if (p.head_dim == 64)
-        return p.sliding_window > 0 ? launch_mfma_hd<NC, 64, true, false, T>(p, nsplit, n_mt, mt_total, stream)
-                                    : launch_mfma_hd<NC, 64, false, false, T>(p, nsplit, n_mt, mt_total, stream);
-    // other head sizes: the 128-wide kernel with padding (built with the window code, which a window of 0 switches off)
-    if (p.head_dim != 128) return launch_mfma_hd<NC, 128, true, true, T>(p, nsplit, n_mt, mt_total, stream);
-    if (p.sliding_window > 0) return launch_mfma_hd<NC, 128, true, false, T>(p, nsplit, n_mt, mt_total, stream);
-    return launch_mfma_hd<NC, 128, false, false, T>(p, nsplit, n_mt, mt_total, stream);
-}
-
 int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
     const int nw = mfma_waves(p);
     const int nsplit = mfma_splits(p, nw);
@@ -1137,8 +215,13 @@ int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
     }
     if (phases & LAZYATTN_PHASE_MAIN) {
         const bool f16 = p.dtype == LAZYATTN_F16;
-        const int rc = nw == 8 ? (f16 ? launch_mfma_nc<8, f16_t>(p, nsplit, n_mt, mt_total, stream) : launch_mfma_nc<8, bf16_t>(p, nsplit, n_mt, mt_total, stream))
-                               : (f16 ? launch_mfma_nc<4, f16_t>(p, nsplit, n_mt, mt_total, stream) : launch_mfma_nc<4, bf16_t>(p, nsplit, n_mt, mt_total, stream));
+        int rc;
+        if (p.cache_dtype == LAZYATTN_FP8_E4M3)
+            rc = f16 ? launch_mfma_family<f16_t, 1>(p, nw, nsplit, n_mt, mt_total, stream) : launch_mfma_family<bf16_t, 1>(p, nw, nsplit, n_mt, mt_total, stream);
+        else if (p.cache_dtype == LAZYATTN_FP8_E5M2)
+            rc = f16 ? launch_mfma_family<f16_t, 2>(p, nw, nsplit, n_mt, mt_total, stream) : launch_mfma_family<bf16_t, 2>(p, nw, nsplit, n_mt, mt_total, stream);
+        else
+            rc = f16 ? launch_mfma_family<f16_t, 0>(p, nw, nsplit, n_mt, mt_total, stream) : launch_mfma_family<bf16_t, 0>(p, nw, nsplit, n_mt, mt_total, stream);
         if (rc != LAZYATTN_OK) return rc;
     }
     if (nsplit > 1 && (phases & LAZYATTN_PHASE_COMBINE)) {
