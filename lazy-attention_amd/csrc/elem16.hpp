@@ -19,6 +19,9 @@ template <typename T> struct Elem;
 template <> struct Elem<bf16_t> {
     // largest P = 2^REBASE between two moves of the softmax reference: anything bf16's exponent carries
     static constexpr float REBASE = 16.f;
+    // a lane's sum of 16 probabilities above this means some P is far from 1: time to move the reference
+    // (2^40: decades below what bf16 and the fp32 sums hold)
+    static constexpr float SUM_LIMIT = 1099511627776.f;
     static __device__ __forceinline__ float lo(uint32_t w) { return __uint_as_float(w << 16); }
     static __device__ __forceinline__ float hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
     static __device__ __forceinline__ uint32_t pack(float a, float b) {
@@ -44,6 +47,7 @@ template <> struct Elem<bf16_t> {
 };
 template <> struct Elem<f16_t> {
     static constexpr float REBASE = 8.f;                      // P <= 256: far inside the half range
+    static constexpr float SUM_LIMIT = 4096.f;                // every P below 2^12 then, the half range ends at 65504
     static __device__ __forceinline__ float lo(uint32_t w) { return (float)(*reinterpret_cast<const f16x2_t *>(&w))[0]; }
     static __device__ __forceinline__ float hi(uint32_t w) { return (float)(*reinterpret_cast<const f16x2_t *>(&w))[1]; }
     static __device__ __forceinline__ uint32_t pack(float a, float b) {

@@ -12,6 +12,55 @@ extern template int launch_mfma_family<f16_t, 0>(const lazyattn_prefill_params &
 extern template int launch_mfma_family<f16_t, 1>(const lazyattn_prefill_params &, int, int, int, int, hipStream_t);
 extern template int launch_mfma_family<f16_t, 2>(const lazyattn_prefill_params &, int, int, int, int, hipStream_t);
 
+// One 16-byte piece (8 elements from column d) of an output row, merged from the row's nsplit partial rows
+// (row0 = token x q-heads + head; consecutive splits are split_rows rows apart).  Log-sum-exps and partial rows of
+// NB splits are requested together and before the first use: one memory round trip per batch; batches are chained
+// like the tiles of the main kernel, by a running maximum.
+template <typename T, int HD, int NB>
+__device__ __forceinline__ uint4 merge_piece(const _Float16 *wo, const float2 *wl, int64_t row0, int64_t split_rows, int nsplit, int d) {
+    using E = Elem<T>;
+    float mx = -INFINITY, wsum = 0.f;
+    float o[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = 0.f;
+    for (int s0 = 0; s0 < nsplit; s0 += NB) {
+        float2 e[NB];                                        // (log2-sum-exp, scale of the row's halves)
+        uint4 v[NB];
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+            const int64_t ri = (int64_t)(s0 + j < nsplit ? s0 + j : nsplit - 1) * split_rows + row0;
+            e[j] = wl[ri];
+            v[j] = *reinterpret_cast<const uint4 *>(wo + ri * HD + d);
+        }
+        float bm = e[0].x;
+#pragma unroll
+        for (int j = 1; j < NB; ++j) bm = fmaxf(bm, e[j].x);
+        const float m_new = fmaxf(mx, bm);
+        if (m_new == -INFINITY) continue;                    // nothing visible so far
+        const float keep = __builtin_amdgcn_exp2f(mx - m_new);   // mx = -inf -> 0
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] *= keep;
+        wsum *= keep;
+        mx = m_new;
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+            const float w = s0 + j < nsplit ? __builtin_amdgcn_exp2f(e[j].x - mx) : 0.f;
+            const float ws = w * e[j].y;
+            const uint32_t u[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const f16x2_t hh = *reinterpret_cast<const f16x2_t *>(&u[i]);
+                o[2 * i] = fmaf(ws, (float)hh[0], o[2 * i]);
+                o[2 * i + 1] = fmaf(ws, (float)hh[1], o[2 * i + 1]);
+            }
+            wsum += w;
+        }
+    }
+    const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
+    return make_uint4(E::pack(o[0] * inv, o[1] * inv), E::pack(o[2] * inv, o[3] * inv),
+                      E::pack(o[4] * inv, o[5] * inv), E::pack(o[6] * inv, o[7] * inv));
+}
+
 // ---- merge split-KV partials: one 16-lane group (head size 128) per (token, q-head) row ----
 // The few fields the merge needs, not the whole parameter block: a launch with ~450 bytes of kernel
 // arguments costs about a microsecond more than one with 64 on this part.
@@ -28,7 +77,6 @@ struct MergeArgs {
 template <typename T, int HD, int NB>
 __global__ void __launch_bounds__(256)
 prefill_combine_kernel(const MergeArgs p, const int nsplit) {
-    using E = Elem<T>;
     constexpr int D = HD, LPR = HD / 8;                       // lanes per row (8 elements = one 16-byte load each)
     const int64_t r = (int64_t)blockIdx.x * (256 / LPR) + threadIdx.x / LPR;
     int64_t tok;
@@ -66,51 +114,8 @@ prefill_combine_kernel(const MergeArgs p, const int nsplit) {
     const int64_t NTOK = p.num_tokens;
     const _Float16 *wo = (const _Float16 *)p.workspace;
     const float2 *wl = reinterpret_cast<const float2 *>(wo + (int64_t)nsplit * NTOK * p.num_q_heads * D);
-    // Log-sum-exps and partial rows of a batch of splits are requested together and before the first use:
-    // one memory round trip per batch.  Batches are chained like the tiles of the main kernel, by a running
-    // maximum.
-    const int64_t row0 = tok * p.num_q_heads + h, split_rows = NTOK * p.num_q_heads;
-    float mx = -INFINITY, wsum = 0.f;
-    float o[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) o[i] = 0.f;
-    for (int s0 = 0; s0 < nsplit; s0 += NB) {
-        float2 e[NB];                                        // (log2-sum-exp, scale of the row's halves)
-        uint4 v[NB];
-#pragma unroll
-        for (int j = 0; j < NB; ++j) {
-            const int64_t ri = (int64_t)(s0 + j < nsplit ? s0 + j : nsplit - 1) * split_rows + row0;
-            e[j] = wl[ri];
-            v[j] = *reinterpret_cast<const uint4 *>(wo + ri * D + d);
-        }
-        float bm = e[0].x;
-#pragma unroll
-        for (int j = 1; j < NB; ++j) bm = fmaxf(bm, e[j].x);
-        const float m_new = fmaxf(mx, bm);
-        if (m_new == -INFINITY) continue;                    // nothing visible so far
-        const float keep = __builtin_amdgcn_exp2f(mx - m_new);   // mx = -inf -> 0
-#pragma unroll
-        for (int i = 0; i < 8; ++i) o[i] *= keep;
-        wsum *= keep;
-        mx = m_new;
-#pragma unroll
-        for (int j = 0; j < NB; ++j) {
-            const float w = s0 + j < nsplit ? __builtin_amdgcn_exp2f(e[j].x - mx) : 0.f;
-            const float ws = w * e[j].y;
-            const uint32_t u[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const f16x2_t hh = *reinterpret_cast<const f16x2_t *>(&u[i]);
-                o[2 * i] = fmaf(ws, (float)hh[0], o[2 * i]);
-                o[2 * i + 1] = fmaf(ws, (float)hh[1], o[2 * i + 1]);
-            }
-            wsum += w;
-        }
-    }
-    const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
-    T *op = (T *)p.o + tok * p.o_stride[0] + (int64_t)h * p.o_stride[1] + d;
-    *reinterpret_cast<uint4 *>(op) = make_uint4(E::pack(o[0] * inv, o[1] * inv), E::pack(o[2] * inv, o[3] * inv),
-                                                E::pack(o[4] * inv, o[5] * inv), E::pack(o[6] * inv, o[7] * inv));
+    const uint4 v = merge_piece<T, HD, NB>(wo, wl, tok * p.num_q_heads + h, NTOK * p.num_q_heads, nsplit, d);
+    *reinterpret_cast<uint4 *>((T *)p.o + tok * p.o_stride[0] + (int64_t)h * p.o_stride[1] + d) = v;
 }
 
 // ------------------------------------------------------------------ host side

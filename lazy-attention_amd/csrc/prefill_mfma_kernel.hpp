@@ -33,6 +33,7 @@
 #pragma once
 #include "common.hpp"
 #include "elem16.hpp"
+#include "fastdiv.hpp"
 #include <atomic>
 
 namespace lazyattn {
@@ -74,6 +75,10 @@ __device__ __forceinline__ float partner32(float x, bool upper) {
     return __uint_as_float(upper ? r[0] : r[1]);
 }
 __device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
+
+// the divisors of the kernel's prologue
+struct MfmaDivs { FastDiv n_mt, nsplit, kv_heads, group; };
+
 
 __device__ __forceinline__ uint4 ldg16(const uint8_t *base, uint32_t off) {
     return *reinterpret_cast<const uint4 *>(base + off);
@@ -139,14 +144,19 @@ template <typename TT> struct KRegs {
 // NC = computing waves = 32-row units per workgroup: 8 (12 waves, three per SIMD) for long
 // key ranges, 4 (8 waves) when the call is small and more, lighter workgroups fill the chip
 // with fewer key-axis splits.
-template <int HD> constexpr int lds_bytes(int nc) { return Geo<HD>::KV_BYTES + nc * Geo<HD>::Q_WAVE + 2 * PAGES * 4; }   // + Q^T fragments (re-read every tile) + page limits
+// With four computing waves two waves share a SIMD's registers and the Q^T fragments stay in registers; with eight
+// (three waves per SIMD) they live in LDS and are re-read every tile.
+constexpr bool q_in_registers(int nc) { return nc == 4; }
+template <int HD> constexpr int lds_bytes(int nc) {      // K and V tiles + Q^T fragments (if in LDS) + page limits
+    return Geo<HD>::KV_BYTES + (q_in_registers(nc) ? 0 : nc * Geo<HD>::Q_WAVE) + 2 * PAGES * 4;
+}
 
 // WIN: built with the sliding-window code (calls without a window run the instantiation without it)
 // PAD: the head size is a multiple of 16 below HD = 128: Q, K and V sit zero-padded in the 128-wide tiles, the two
 // halves of the real head at (0 .., 64 ..) so that the rotation pairs stay (d, 64 + d)
 template <int NC, int HD, int FP8, bool WIN, bool PAD, typename T, typename TT>
 __global__ void __launch_bounds__((NC + 4) * 64)
-prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int n_mt, const int mt_total) {
+prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int n_mt, const int mt_total, const MfmaDivs dv) {
     using G = Geo<HD>;
     constexpr int D = HD, HALF = HD / 2;
     const int Dr = PAD ? p.head_dim : D, HALFr = Dr / 2, CPr = Dr / 16;   // real head size, its half, its chunk pairs
@@ -224,20 +234,23 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         if (((p.batch * p.num_kv_heads) & 7) == 0) {
             // every split and m-tile of one (request, kv-head) on one XCD: they share K/V through its L2
             const int xcd = L & 7, q = L >> 3;
-            mt = q % n_mt;
-            const int r = q / n_mt;
-            kvgrp = ((r / nsplit) * 8 + xcd) * nsplit + r % nsplit;
+            const int r = (int)dv.n_mt.quot(q);
+            mt = (int)dv.n_mt.rem(q, r);
+            const int rs = (int)dv.nsplit.quot(r);
+            kvgrp = (rs * 8 + xcd) * nsplit + (int)dv.nsplit.rem(r, rs);
         } else if ((n_groups & 7) == 0) {
             const int xcd = L & 7, q = L >> 3;
-            mt = q % n_mt;
-            kvgrp = (q / n_mt) * 8 + xcd;
+            const int r = (int)dv.n_mt.quot(q);
+            mt = (int)dv.n_mt.rem(q, r);
+            kvgrp = r * 8 + xcd;
         } else {
-            mt = L % n_mt;
-            kvgrp = L / n_mt;
+            kvgrp = (int)dv.n_mt.quot(L);
+            mt = (int)dv.n_mt.rem(L, kvgrp);
         }
-        split = kvgrp % nsplit;
-        g = (kvgrp / nsplit) % p.num_kv_heads;
-        b = kvgrp / (nsplit * p.num_kv_heads);
+        const int bg = (int)dv.nsplit.quot(kvgrp);               // (request, kv head)
+        split = (int)dv.nsplit.rem(kvgrp, bg);
+        b = (int)dv.kv_heads.quot(bg);
+        g = (int)dv.kv_heads.rem(bg, b);
     }
 
     const int64_t qs = load_index(p.b_start_loc, b, p.index_bits);
@@ -257,7 +270,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     {
         int last_unit = mt * NC + NC - 1;
         if (last_unit > n_units - 1) last_unit = n_units - 1;
-        const int te = (last_unit / group + 1) * UNIT;
+        const int te = ((int)dv.group.quot(last_unit) + 1) * UNIT;
         t_end = te < q_len ? te : q_len;
     }
     const int n_ctx_tiles = (n_pages + PAGES - 1) / PAGES;
@@ -272,7 +285,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     const int window = WIN ? p.sliding_window : 0;
     int skip_ctx = 0, skip_new = 0;                 // whole context / new-token tiles before every window
     if (window) {
-        const int first_row = ((mt * NC) / group) * UNIT;
+        const int first_row = (int)dv.group.quot(mt * NC) * UNIT;
         const int lo_min = ctx_len + first_row - window + 1;
         if (lo_min > 0) {
             skip_ctx = lo_min < ctx_len ? lo_min / NT : n_ctx_tiles;
@@ -281,12 +294,12 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         }
     }
     const int live_ctx = n_ctx_tiles - skip_ctx, live_new = n_new_tiles - skip_new;
-    const int64_t cost = live_ctx + (int64_t)NEW_COST * live_new;
-    auto tile_at = [&](int64_t c) -> int {         // first tile whose cost interval ends after c
-        return skip_ctx + skip_new + (c <= live_ctx ? (int)c : live_ctx + (int)((c - live_ctx) / NEW_COST));
+    const uint32_t cost = (uint32_t)live_ctx + (uint32_t)NEW_COST * (uint32_t)live_new;   // (tiles: far below 2^25; splits <= 64)
+    auto tile_at = [&](uint32_t c) -> int {        // first tile whose cost interval ends after c
+        return skip_ctx + skip_new + (c <= (uint32_t)live_ctx ? (int)c : live_ctx + (int)((c - (uint32_t)live_ctx) / NEW_COST));
     };
-    const int tile_begin = tile_at(cost * split / nsplit);
-    const int tile_end = split + 1 == nsplit ? n_ctx_tiles + n_new_tiles : tile_at(cost * (split + 1) / nsplit);
+    const int tile_begin = tile_at(dv.nsplit.quot(cost * (uint32_t)split));
+    const int tile_end = split + 1 == nsplit ? n_ctx_tiles + n_new_tiles : tile_at(dv.nsplit.quot(cost * (uint32_t)(split + 1)));
 
     // ---- page metadata, fetched ahead of its use ----
     // Gathering wave w owns page w of every tile, so it needs one block-table entry, one
@@ -326,7 +339,9 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     };
     // Valid-slot counts of the four pages of a context tile, one int per page and LDS buffer:
     // written by the gathering waves with the tile, read by the computing waves for the masks.
-    int *page_lims = reinterpret_cast<int *>(lds + KV_BYTES + NC * G::Q_WAVE);
+    constexpr bool QREG = q_in_registers(NC);
+    constexpr int Q_BYTES = QREG ? 0 : NC * G::Q_WAVE;
+    int *page_lims = reinterpret_cast<int *>(lds + KV_BYTES + Q_BYTES);
 
     if (gatherer) {
         // ====================================================================== gather
@@ -401,55 +416,60 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         uint4 vr[VI];
 
         // ---- loads of a context page: no branch, no zero fill ----
-        auto issue_loads_ctx = [&](int tile, const PageMeta &pm) {
+        // Position of the page's first slot.  Natural: j*16 (old_ops:183-184); offset: q_offset-1 if
+        // set, else natural (old_ops:186-191); block-uniform: q_offset-1 if set, else 0 (ops:180-186);
+        // un-rotated requests read row 0 of the table (cos 1, sin 0): exact identity.  pm.qo is 0
+        // wherever q_offset is not consulted, nat_step is 0 wherever the fallback is row 0.
+        // A page past the context (its slots are all masked) takes the last page's position: the
+        // table only has to cover the positions of real keys.
+        struct PageBase { const uint8_t *kb, *tb, *vb; };
+        auto page_base = [&](int tile, const PageMeta &pm) -> PageBase {
             const int j = tile * PAGES + gw;
-            const uint8_t *kb = kc_base + pm.bt * kc_page_bytes;
-            // Position of the page's first slot.  Natural: j*16 (old_ops:183-184); offset: q_offset-1 if
-            // set, else natural (old_ops:186-191); block-uniform: q_offset-1 if set, else 0 (ops:180-186);
-            // un-rotated requests read row 0 of the table (cos 1, sin 0): exact identity.  pm.qo is 0
-            // wherever q_offset is not consulted, nat_step is 0 wherever the fallback is row 0.
-            // A page past the context (its slots are all masked) takes the last page's position: the
-            // table only has to cover the positions of real keys.
             const int jp = j < n_pages ? j : n_pages - 1;
             const int pos0 = pm.qo ? pm.qo - 1 + part_pos : jp * nat_step;
-            const uint8_t *tb = ctab_base + (int64_t)pos0 * pos_bytes;
-#pragma unroll
-            for (int i = 0; i < KI; ++i) {
-                kr[i].lds_off = (uint32_t)(gw * K_PAGE + (lane + i * 64) * 16);
-                if constexpr (PAD) {
-                    uint4 k1, k2;
-                    if (FP8) {
-                        const uint2 a = ldg8(kb, pk1[i]), a2 = ldg8(kb, pk2[i]);
-                        k1 = make_uint4(a.x, a.y, 0, 0);
-                        k2 = make_uint4(a2.x, a2.y, 0, 0);
-                    } else {
-                        k1 = ldg16(kb, pk1[i]);
-                        k2 = ldg16(kb, pk2[i]);
-                    }
-                    const uint4 z = make_uint4(0, 0, 0, 0);
-                    kr[i].k1 = pk_ok[i] ? k1 : z;
-                    kr[i].k2 = pk_ok[i] ? k2 : z;
-                } else if (FP8) {
-                    const uint2 a = ldg8(kb + i * k_item, k_goff), a2 = ldg8(kb + i * k_item + pair, k_goff);
-                    kr[i].k1 = make_uint4(a.x, a.y, 0, 0);
-                    kr[i].k2 = make_uint4(a2.x, a2.y, 0, 0);
+            return PageBase{kc_base + pm.bt * kc_page_bytes, ctab_base + (int64_t)pos0 * pos_bytes, vc_base + pm.bt * vc_page_bytes};
+        };
+        auto load_k_item = [&](int i, const PageBase &pb) {
+            const uint8_t *kb = pb.kb;
+            kr[i].lds_off = (uint32_t)(gw * K_PAGE + (lane + i * 64) * 16);
+            if constexpr (PAD) {
+                uint4 k1, k2;
+                if (FP8) {
+                    const uint2 a = ldg8(kb, pk1[i]), a2 = ldg8(kb, pk2[i]);
+                    k1 = make_uint4(a.x, a.y, 0, 0);
+                    k2 = make_uint4(a2.x, a2.y, 0, 0);
                 } else {
-                    kr[i].k1 = ldg16(kb + i * k_item, k_goff);
-                    kr[i].k2 = ldg16(kb + i * k_item + pair, k_goff);
+                    k1 = ldg16(kb, pk1[i]);
+                    k2 = ldg16(kb, pk2[i]);
                 }
-                kr[i].c.load(tb, k_toff[i]);
-                kr[i].s.load(tb, k_toff[i] + sin_delta);
+                const uint4 z = make_uint4(0, 0, 0, 0);
+                kr[i].k1 = pk_ok[i] ? k1 : z;
+                kr[i].k2 = pk_ok[i] ? k2 : z;
+            } else if (FP8) {
+                const uint2 a = ldg8(kb + i * k_item, k_goff), a2 = ldg8(kb + i * k_item + pair, k_goff);
+                kr[i].k1 = make_uint4(a.x, a.y, 0, 0);
+                kr[i].k2 = make_uint4(a2.x, a2.y, 0, 0);
+            } else {
+                kr[i].k1 = ldg16(kb + i * k_item, k_goff);
+                kr[i].k2 = ldg16(kb + i * k_item + pair, k_goff);
             }
-            const uint8_t *vb = vc_base + pm.bt * vc_page_bytes;
+            kr[i].c.load(pb.tb, k_toff[i]);
+            kr[i].s.load(pb.tb, k_toff[i] + sin_delta);
+        };
+        auto load_v_item = [&](int i, const PageBase &pb) {
+            if constexpr (PAD) {
+                const uint4 t = ldg16(pb.vb, pv[i]);
+                vr[i] = pv_ok[i] ? t : make_uint4(0, 0, 0, 0);
+            } else {
+                vr[i] = ldg16(pb.vb + i * v_item, v_goff);
+            }
+        };
+        auto issue_loads_ctx = [&](int tile, const PageMeta &pm) {
+            const PageBase pb = page_base(tile, pm);
 #pragma unroll
-            for (int i = 0; i < VI_CTX; ++i) {
-                if constexpr (PAD) {
-                    const uint4 t = ldg16(vb, pv[i]);
-                    vr[i] = pv_ok[i] ? t : make_uint4(0, 0, 0, 0);
-                } else {
-                    vr[i] = ldg16(vb + i * v_item, v_goff);
-                }
-            }
+            for (int i = 0; i < KI; ++i) load_k_item(i, pb);
+#pragma unroll
+            for (int i = 0; i < VI_CTX; ++i) load_v_item(i, pb);
         };
         // ---- loads of this wave's 16 keys of a new-token tile ----
         auto issue_loads_new = [&](int tile) {
@@ -499,29 +519,72 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             return TILE_EDGE;
         };
         // ---- rotate the K items in fp32 and write them to a K tile ----
+        auto store_k_item = [&](int i, uint8_t *ktile, int kind) {
+            float a[8], bb[8], cs[8], sn[8];
+            if (FP8 && kind != TILE_NEW) {
+                unpack8_fp8<T, FP8>(kr[i].k1.x, kr[i].k1.y, k_scale, a);
+                unpack8_fp8<T, FP8>(kr[i].k2.x, kr[i].k2.y, k_scale, bb);
+            } else {
+                unpack8<T>(kr[i].k1, a);
+                unpack8<T>(kr[i].k2, bb);
+            }
+            kr[i].c.get(cs);
+            kr[i].s.get(sn);
+            float x[8], y[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                x[e] = a[e] * cs[e] - bb[e] * sn[e];                             // old_ops:253
+                y[e] = a[e] * sn[e] + bb[e] * cs[e];                             // old_ops:254
+            }
+            *reinterpret_cast<uint4 *>(ktile + kr[i].lds_off) = make_uint4(
+                E::pack(x[0], x[1]), E::pack(x[2], x[3]), E::pack(x[4], x[5]), E::pack(x[6], x[7]));
+            *reinterpret_cast<uint4 *>(ktile + kr[i].lds_off + G::PAIR) = make_uint4(
+                E::pack(y[0], y[1]), E::pack(y[2], y[3]), E::pack(y[4], y[5]), E::pack(y[6], y[7]));
+        };
         auto store_k = [&](uint8_t *ktile, int kind) {
 #pragma unroll
-            for (int i = 0; i < KI; ++i) {
-                float a[8], bb[8], cs[8], sn[8];
-                if (FP8 && kind != TILE_NEW) {
-                    unpack8_fp8<T, FP8>(kr[i].k1.x, kr[i].k1.y, k_scale, a);
-                    unpack8_fp8<T, FP8>(kr[i].k2.x, kr[i].k2.y, k_scale, bb);
-                } else {
-                    unpack8<T>(kr[i].k1, a);
-                    unpack8<T>(kr[i].k2, bb);
-                }
-                kr[i].c.get(cs);
-                kr[i].s.get(sn);
-                float x[8], y[8];
+            for (int i = 0; i < KI; ++i) store_k_item(i, ktile, kind);
+        };
+        // one V item of a context page (16 bytes of one row of d) -> its two 8-byte LDS entries
+        auto store_v_item = [&](int i, uint8_t *vtile, int kind, int lim) {
+            const int idx = lane + i * 64;
+            if (FP8) {
+                // 16 fp8 slots of one d: entry g=0 <- slots 0-3 | 8-11, entry g=1 <- slots 4-7 | 12-15
+                const int d = idx;
+                const uint32_t w[4] = {vr[i].x, vr[i].y, vr[i].z, vr[i].w};
+                uint32_t o2[4][2];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    x[e] = a[e] * cs[e] - bb[e] * sn[e];                             // old_ops:253
-                    y[e] = a[e] * sn[e] + bb[e] * cs[e];                             // old_ops:254
+                for (int q4 = 0; q4 < 4; ++q4) {
+                    const f32x2_t lo = cvt_fp8x2<FP8>(w[q4]);
+                    const f32x2_t hi = cvt_fp8x2<FP8>(w[q4] >> 16);
+                    float f[4] = {lo[0] * v_scale, lo[1] * v_scale, hi[0] * v_scale, hi[1] * v_scale};
+                    if (kind == TILE_EDGE) {
+#pragma unroll
+                        for (int s = 0; s < 4; ++s)
+                            if (q4 * 4 + s >= lim) f[s] = 0.f;   // masked slots contribute nothing, whatever they hold
+                    }
+                    o2[q4][0] = E::pack(f[0], f[1]);
+                    o2[q4][1] = E::pack(f[2], f[3]);
                 }
-                *reinterpret_cast<uint4 *>(ktile + kr[i].lds_off) = make_uint4(
-                    E::pack(x[0], x[1]), E::pack(x[2], x[3]), E::pack(x[4], x[5]), E::pack(x[6], x[7]));
-                *reinterpret_cast<uint4 *>(ktile + kr[i].lds_off + G::PAIR) = make_uint4(
-                    E::pack(y[0], y[1]), E::pack(y[2], y[3]), E::pack(y[4], y[5]), E::pack(y[6], y[7]));
+                uint8_t *dst = vtile + gw * V_PAGE + d * 16;
+                *reinterpret_cast<uint4 *>(dst) = make_uint4(o2[0][0], o2[0][1], o2[2][0], o2[2][1]);
+                *reinterpret_cast<uint4 *>(dst + V_G) = make_uint4(o2[1][0], o2[1][1], o2[3][0], o2[3][1]);
+            } else {
+                // 8 bf16 slots (8*hf ..) of one d: slots +0..3 -> entry g=0, +4..7 -> entry g=1, half hf
+                const int d = idx >> 1, hf = idx & 1;
+                uint4 v = vr[i];
+                if (kind == TILE_EDGE) {
+                    uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (hf * 8 + 2 * e >= lim) w[e] &= 0xffff0000u;
+                        if (hf * 8 + 2 * e + 1 >= lim) w[e] &= 0x0000ffffu;
+                    }
+                    v = make_uint4(w[0], w[1], w[2], w[3]);
+                }
+                uint8_t *dst = vtile + gw * V_PAGE + d * 16 + hf * 8;
+                *reinterpret_cast<uint2 *>(dst) = make_uint2(v.x, v.y);
+                *reinterpret_cast<uint2 *>(dst + V_G) = make_uint2(v.z, v.w);
             }
         };
         // ---- write the V items to a V tile; lim = valid slots of the page ----
@@ -544,47 +607,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                 return;
             }
 #pragma unroll
-            for (int i = 0; i < VI_CTX; ++i) {
-                const int idx = lane + i * 64;
-                if (FP8) {
-                    // 16 fp8 slots of one d: entry g=0 <- slots 0-3 | 8-11, entry g=1 <- slots 4-7 | 12-15
-                    const int d = idx;
-                    const uint32_t w[4] = {vr[i].x, vr[i].y, vr[i].z, vr[i].w};
-                    uint32_t o2[4][2];
-#pragma unroll
-                    for (int q4 = 0; q4 < 4; ++q4) {
-                        const f32x2_t lo = cvt_fp8x2<FP8>(w[q4]);
-                        const f32x2_t hi = cvt_fp8x2<FP8>(w[q4] >> 16);
-                        float f[4] = {lo[0] * v_scale, lo[1] * v_scale, hi[0] * v_scale, hi[1] * v_scale};
-                        if (kind == TILE_EDGE) {
-#pragma unroll
-                            for (int s = 0; s < 4; ++s)
-                                if (q4 * 4 + s >= lim) f[s] = 0.f;   // masked slots contribute nothing, whatever they hold
-                        }
-                        o2[q4][0] = E::pack(f[0], f[1]);
-                        o2[q4][1] = E::pack(f[2], f[3]);
-                    }
-                    uint8_t *dst = vtile + gw * V_PAGE + d * 16;
-                    *reinterpret_cast<uint4 *>(dst) = make_uint4(o2[0][0], o2[0][1], o2[2][0], o2[2][1]);
-                    *reinterpret_cast<uint4 *>(dst + V_G) = make_uint4(o2[1][0], o2[1][1], o2[3][0], o2[3][1]);
-                } else {
-                    // 8 bf16 slots (8*hf ..) of one d: slots +0..3 -> entry g=0, +4..7 -> entry g=1, half hf
-                    const int d = idx >> 1, hf = idx & 1;
-                    uint4 v = vr[i];
-                    if (kind == TILE_EDGE) {
-                        uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            if (hf * 8 + 2 * e >= lim) w[e] &= 0xffff0000u;
-                            if (hf * 8 + 2 * e + 1 >= lim) w[e] &= 0x0000ffffu;
-                        }
-                        v = make_uint4(w[0], w[1], w[2], w[3]);
-                    }
-                    uint8_t *dst = vtile + gw * V_PAGE + d * 16 + hf * 8;
-                    *reinterpret_cast<uint2 *>(dst) = make_uint2(v.x, v.y);
-                    *reinterpret_cast<uint2 *>(dst + V_G) = make_uint2(v.z, v.w);
-                }
-            }
+            for (int i = 0; i < VI_CTX; ++i) store_v_item(i, vtile, kind, lim);
         };
         // tile + its page limit -> LDS buffer `buf`
         auto store_tile = [&](int buf, int kind, int lim) {
@@ -615,8 +638,25 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             while (tile + 2 < n_ctx_tiles && tile + 2 < tile_end && nxt_kind == TILE_FULL && pm_pend.lim == BS) {
                 const int cur = (tile - tile_begin) & 1;
                 const PageMeta pm_new = load_page((tile + 3) * PAGES + gw);      // scalar loads, land during the rotation
-                store_tile(cur ^ 1, TILE_FULL, BS);
-                issue_loads_ctx(tile + 2, pm_pend);
+                // Item by item: as soon as an item of tile+1 has left its registers for LDS, the same item of
+                // tile+2 is requested into them.  The four gathering waves' loads then reach the CU's memory
+                // pipeline spread over the tile instead of in one burst at its end (in a burst each of the twelve
+                // loads of a wave waited tens of cycles to be accepted, all of it on this wave's critical path).
+                const PageBase pb = page_base(tile + 2, pm_pend);
+                uint8_t *kt = lds + (cur ^ 1) * K_TILE, *vt = lds + 2 * K_TILE + (cur ^ 1) * V_TILE;
+#pragma unroll
+                for (int i = 0; i < KI; ++i) {
+                    store_k_item(i, kt, TILE_FULL);
+                    load_k_item(i, pb);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int i = 0; i < VI_CTX; ++i) {
+                    store_v_item(i, vt, TILE_FULL, BS);
+                    load_v_item(i, pb);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if (lane == 0) page_lims[(cur ^ 1) * PAGES + gw] = BS;
                 pm_pend = pm_new;
                 ++tile;
                 __syncthreads();
@@ -639,21 +679,22 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     const int l32 = lane & 31, gh = lane >> 5;
     const int unit = mt * NC + wave;
     const bool active = unit < n_units;
-    const int chunk = active ? unit / group : 0;
-    const int h = g * group + (active ? unit % group : 0);
+    const int chunk = active ? (int)dv.group.quot(unit) : 0;
+    const int h = g * group + (active ? unit - chunk * group : 0);
     const int t0 = chunk * UNIT;
     const int row = t0 + l32;                                    // token index of this lane's query row
     const bool row_ok = active && row < q_len;
 
     // Q^T fragments: B operand of S^T = K.Q^T, lane = (row l32, d = ks*16 + gh*8 .. +8).
-    // They live in this wave's own LDS slice (not in registers: three waves share a SIMD's
-    // register file) and are re-read for every tile.
+    // Eight computing waves: they live in this wave's own LDS slice (three waves share a SIMD's register
+    // file) and are re-read for every tile.  Four: 32 registers per lane, no LDS traffic for Q at all.
     // Q is multiplied by sm_scale * log2(e) here, once, and rounded to bf16 again: the MFMA then
     // delivers the scores in log2 units and no per-score multiply is left in the tile loop (the
     // reference scales the fp32 scores, old_ops:287; the extra rounding of Q is one more relative
     // 2^-9 per element, like the one the rotated K already carries).
     const float cs2 = p.sm_scale * 1.4426950408889634f;
-    uint8_t *qlds = lds + KV_BYTES + wave * G::Q_WAVE + lane * 16;
+    uint8_t *qlds = lds + KV_BYTES + (QREG ? 0 : wave * G::Q_WAVE) + lane * 16;
+    uint4 qreg[QREG ? KS : 1];
     {
         const T *qp = (const T *)p.q + (qs + row) * p.q_stride[0] + (int64_t)h * p.q_stride[1] + gh * 8;
 #pragma unroll
@@ -668,9 +709,10 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             }
             float f[8];
             unpack8<T>(v, f);
-            *reinterpret_cast<uint4 *>(qlds + ks * 1024) =
-                make_uint4(E::pack(f[0] * cs2, f[1] * cs2), E::pack(f[2] * cs2, f[3] * cs2),
-                           E::pack(f[4] * cs2, f[5] * cs2), E::pack(f[6] * cs2, f[7] * cs2));
+            const uint4 qs4 = make_uint4(E::pack(f[0] * cs2, f[1] * cs2), E::pack(f[2] * cs2, f[3] * cs2),
+                                         E::pack(f[4] * cs2, f[5] * cs2), E::pack(f[6] * cs2, f[7] * cs2));
+            if constexpr (QREG) qreg[ks] = qs4;
+            else *reinterpret_cast<uint4 *>(qlds + ks * 1024) = qs4;
         }
     }
     // Online softmax against a reference m_ref per row that moves rarely.  The MFMA accumulators of S^T
@@ -678,8 +720,12 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     // m_ref is moved (and O, l rescaled, old_ops:287-291) only when a row's tile maximum exceeds it by more
     // than REBASE, or when the row sees its first valid key; in between P may exceed 1 (by at most
     // 2^REBASE), which fp32 accumulation and bf16's exponent range carry without loss.
-    constexpr float REBASE = E::REBASE;
-    float m_ref = 0.f, l_run = 0.f, l_alt = 0.f;                    // row sum kept as two chains
+    // Once every row of the wave has seen a key, full tiles do not compute the row maximum at all: P = exp2(S)
+    // is formed at once and the rows' sums of P -- needed anyway -- tell whether any P left the range the
+    // element type and the fp32 accumulators carry comfortably (SUM_LIMIT); only then is the maximum taken
+    // and the reference moved, before the P.V step that would use those P.
+    constexpr float REBASE = E::REBASE, SUM_LIMIT = E::SUM_LIMIT;
+    float m_ref = 0.f, l_run = 0.f;
     bool seen = false;                                              // the row has had a valid key
     f32x16_t cinit;                                                 // -m_ref in every element
 #pragma unroll
@@ -690,31 +736,28 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[dt][i] = 0.f;
 
-    // ---- S^T = K . Q^T for one 64-key tile: two independent 32-key accumulation chains ----
-    auto qk_tile = [&](const uint8_t *ktile, f32x16_t &s0, f32x16_t &s1) {
-        const uint8_t *kp = ktile + (l32 >> 4) * K_PAGE + gh * 256 + (l32 & 15) * 16;
-        // A wave in a matrix phase goes first on its SIMD: its MFMAs are issued the moment the pipe is
-        // free and the vector work of the other waves fills the cycles in between (measured: -3 % on
-        // long key ranges against equal priorities).
-        __builtin_amdgcn_s_setprio(2);
-        // operands are requested two k-steps ahead of their MFMAs (a ring of three sets): one step ahead
-        // leaves the LDS latency exposed in every step
-        uint4 a0[3], a1[3], q[3];
+    // ---- S^T = K . Q^T for 32 keys of a tile (pages 2*sub, 2*sub+1) ----
+    // Operands are requested two k-steps ahead of their MFMAs (a ring of three sets): one step ahead leaves the
+    // LDS latency exposed in every step.  `between(ks)` is vector work of this wave placed behind the MFMA of
+    // step ks in the instruction stream: the wave runs it while the matrix pipe works (the exponentials of the
+    // other half, see the tile loop).
+    auto qk_half = [&](const uint8_t *ktile, int sub, f32x16_t &s, auto between) {
+        const uint8_t *kp = ktile + (sub * 2 + (l32 >> 4)) * K_PAGE + gh * 256 + (l32 & 15) * 16;
+        uint4 a[3], q[QREG ? 1 : 3];
         auto fetch = [&](int ks) {
-            a0[ks % 3] = *reinterpret_cast<const uint4 *>(kp + ks * 512);
-            a1[ks % 3] = *reinterpret_cast<const uint4 *>(kp + 2 * K_PAGE + ks * 512);
-            q[ks % 3] = *reinterpret_cast<const uint4 *>(qlds + ks * 1024);
+            a[ks % 3] = *reinterpret_cast<const uint4 *>(kp + ks * 512);
+            if constexpr (!QREG) q[ks % 3] = *reinterpret_cast<const uint4 *>(qlds + ks * 1024);
         };
         fetch(0);
         fetch(1);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             if (ks + 2 < KS) fetch(ks + 2);
-            s0 = E::mfma(a0[ks % 3], q[ks % 3], ks ? s0 : cinit);
-            s1 = E::mfma(a1[ks % 3], q[ks % 3], ks ? s1 : cinit);
+            const uint4 &qf = QREG ? qreg[QREG ? ks : 0] : q[QREG ? 0 : ks % 3];
+            s = E::mfma(a[ks % 3], qf, ks ? s : cinit);
+            between(ks);
             __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_s_setprio(0);
     };
     // ---- masks: register i of half `sub` holds key sub*32 + 8*(i/4) + 4*gh + i%4 ----
     // key0 = sequence position of the tile's first key (only used under a sliding window)
@@ -747,7 +790,6 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) acc[dt] *= alpha;
             l_run *= alpha;
-            l_alt *= alpha;
             s0 -= delta;
             s1 -= delta;
             m_ref += delta;
@@ -756,24 +798,46 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         }
         seen = seen || valid;
     };
+    // ---- the rare step of the lazy path: the P of `sa` left the comfortable range; move the reference to the
+    // maximum of those 32 keys.  `sb`: scores still to be used that were formed against the old reference;
+    // `hsum`: row sum of a half already added to O under the old reference ----
+    auto bump = [&](f32x16_t &sa, f32x16_t *sb, float *hsum) {
+        float mx = max3(sa[0], sa[1], sa[2]);
+#pragma unroll
+        for (int i = 3; i < 15; i += 2) mx = max3(mx, sa[i], sa[i + 1]);
+        mx = max3(mx, sa[15], sa[15]);
+        mx = max3(mx, partner32(mx, gh != 0), mx);
+        const float delta = mx > 0.f ? mx : 0.f;                    // (NaN: 0, the row stays NaN)
+        const float alpha = __builtin_amdgcn_exp2f(-delta);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) acc[dt] *= alpha;
+        l_run *= alpha;
+        if (hsum) *hsum *= alpha;
+        sa -= delta;
+        if (sb) *sb -= delta;
+        m_ref += delta;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) cinit[i] = -m_ref;
+    };
     // ---- P = exp2(S) for 32 keys (S is relative to m_ref), packed as the two B operands of the PV steps ----
-    auto exp_half = [&](const f32x16_t &s, uint4 &p0, uint4 &p1) {
-        float pr[16];
+    // One eighth of a half at a time (two exponentials, one pack, one partial row sum), so that the pieces can be
+    // placed between MFMAs: w[] collects the packed probabilities, ta / tb the two chains of the lane's row sum
+    // (of the rounded probabilities, two per instruction; old_ops:312 sums them unrounded).
+    struct HalfP { uint32_t w[8]; float ta, tb; };
+    auto exp_piece = [&](const f32x16_t &s, HalfP &h, int i) {
+        h.w[i] = E::pack(__builtin_amdgcn_exp2f(s[2 * i]), __builtin_amdgcn_exp2f(s[2 * i + 1]));
+        if (i & 1) h.tb = E::dot2_ones(h.w[i], i == 1 ? 0.f : h.tb);
+        else h.ta = E::dot2_ones(h.w[i], i == 0 ? 0.f : h.ta);
+    };
+    auto exp_half = [&](const f32x16_t &s, HalfP &h) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) pr[i] = __builtin_amdgcn_exp2f(s[i]);
-        uint32_t w[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) w[i] = E::pack(pr[2 * i], pr[2 * i + 1]);
-        // row sum of the rounded probabilities, two per instruction (old_ops:312 sums them unrounded)
-#pragma unroll
-        for (int i = 0; i < 8; i += 2) { l_run = E::dot2_ones(w[i], l_run); l_alt = E::dot2_ones(w[i + 1], l_alt); }
-        p0 = make_uint4(w[0], w[1], w[2], w[3]);
-        p1 = make_uint4(w[4], w[5], w[6], w[7]);
+        for (int i = 0; i < 8; ++i) exp_piece(s, h, i);
     };
     // ---- O^T += V^T . P^T for 32 keys (pages 2*sub, 2*sub+1 of the tile) ----
     // k index j of a 16-key step <-> slot 4*gh + j (j < 4), 8 + 4*gh + j - 4 (j >= 4)
-    auto pv_half = [&](const uint8_t *vtile, int sub, const uint4 &p0, const uint4 &p1) {
+    auto pv_half = [&](const uint8_t *vtile, int sub, const HalfP &h, auto between) {
         const uint8_t *vp = vtile + (sub * 2) * V_PAGE + gh * V_G + l32 * 16;
+        const uint4 p0 = make_uint4(h.w[0], h.w[1], h.w[2], h.w[3]), p1 = make_uint4(h.w[4], h.w[5], h.w[6], h.w[7]);
         // 2 DT MFMAs: the 32-row blocks of d for the first page of the half, then for the second;
         // their V^T operands are requested two MFMAs ahead
         uint4 a[3];
@@ -784,23 +848,15 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         for (int j = 0; j < 2 * DT; ++j) {
             if (j + 2 < 2 * DT) fetch(j + 2);
             acc[j % DT] = E::mfma(a[j % 3], j < DT ? p0 : p1, acc[j % DT]);
+            between(j);
+            __builtin_amdgcn_sched_barrier(0);
         }
-    };
-    auto attend = [&](const uint8_t *vtile, f32x16_t &s0, f32x16_t &s1) {
-        rebase(s0, s1);
-        uint4 p0, p1, p2, p3;
-        exp_half(s0, p0, p1);
-        __builtin_amdgcn_s_setprio(2);
-        pv_half(vtile, 0, p0, p1);
-        exp_half(s1, p2, p3);
-        pv_half(vtile, 1, p2, p3);
-        __builtin_amdgcn_s_setprio(0);
     };
 
     // which of the tile's 64 keys exist: new-token tiles from the token count, context tiles from the
     // page limits the gathering waves left beside the tile
     struct Desc { int kind; uint32_t vlo, vhi; int m0, key0; };
-    auto describe = [&](int tile, int cur) -> Desc {
+    auto describe = [&](int tile, const int4 &lims) -> Desc {
         Desc td{TILE_FULL, ~0u, ~0u, 0, tile * NT};
         if (tile >= n_ctx_tiles) {
             td.kind = TILE_NEW;
@@ -810,7 +866,6 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             const uint64_t valid = n >= 64 ? ~0ull : (n <= 0 ? 0ull : ((1ull << n) - 1ull));
             td.vlo = (uint32_t)valid; td.vhi = (uint32_t)(valid >> 32);
         } else {
-            const int4 lims = *reinterpret_cast<const int4 *>(page_lims + cur * PAGES);
             const int l0 = uniform(lims.x), l1 = uniform(lims.y), l2 = uniform(lims.z), l3 = uniform(lims.w);
             if ((l0 & l1 & l2 & l3) != BS) {
                 td.kind = TILE_EDGE;
@@ -822,29 +877,80 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         if (window && td.kind == TILE_FULL && td.key0 < ctx_len + t0 + UNIT - window) td.kind = TILE_EDGE;
         return td;
     };
+    // The tile body, in the order the instructions are issued.  A wave's own vector work sits behind its own
+    // MFMAs wherever the data allow it, so that a single wave keeps the matrix pipe busy through the whole tile
+    // and the waves of a SIMD need not be out of step with each other to fill it:
+    //   A  S0 = K0.Q^T                       8 MFMAs
+    //   B  S1 = K1.Q^T                       8 MFMAs, behind each: two exponentials of S0, pack, row sum
+    //      (head size 64: four MFMAs per phase, twice the vector work behind each)
+    //   C  O += V0^T.P0^T                    8 MFMAs, behind each: the same for S1
+    //   D  O += V1^T.P1^T                    8 MFMAs
+    // That is the path of a full tile whose rows have all seen a key (no masks, no row maximum).  Any other
+    // tile computes S1 first, masks, takes the maximum over both halves (the reference may move), and then forms
+    // P0 in one go; from C on the two paths are the same instructions.
     __syncthreads();
     for (int tile = tile_begin; tile < tile_end; ++tile) {
         const int cur = (tile - tile_begin) & 1;
         const uint8_t *ktile = lds + cur * K_TILE;
         const uint8_t *vtile = lds + 2 * K_TILE + cur * V_TILE;
-        const Desc td = describe(tile, cur);
-        // One call site for the tile body: the accumulators keep their registers round the loop.
+        const bool is_new = tile >= n_ctx_tiles;
         // Rows of an idle wave are all-zero queries (harmless, never stored); a new-token tile
         // entirely in this wave's future contributes nothing (causal) and is skipped.
-        if (td.kind != TILE_NEW || td.m0 <= t0 + UNIT - 1) {
+        if (!is_new || (tile - n_ctx_tiles) * NT <= t0 + UNIT - 1) {
+            // valid-slot counts of the tile's pages: requested now, looked at after phase A
+            const int4 lims = *reinterpret_cast<const int4 *>(page_lims + cur * PAGES);
             f32x16_t s0, s1;
-            qk_tile(ktile, s0, s1);
-            if (td.kind != TILE_FULL) {
-                mask_half(s0, td.vlo, 0, td.kind, td.m0, td.key0);
-                mask_half(s1, td.vhi, 1, td.kind, td.m0, td.key0);
+            HalfP h0, h1;
+            __builtin_amdgcn_s_setprio(2);
+            qk_half(ktile, 0, s0, [](int) {});
+            const Desc td = describe(tile, lims);
+            const bool lazy = td.kind == TILE_FULL && __builtin_amdgcn_ballot_w64(!seen) == 0;
+            // (the exponentials of S0 are formed behind these MFMAs on every tile: a tile that is not lazy forms
+            // them again after its masks and maximum, and the first set, possibly garbage, is dropped)
+            qk_half(ktile, 1, s1, [&](int ks) {
+#pragma unroll
+                for (int i = 0; i < 8 / KS; ++i) exp_piece(s0, h0, ks * (8 / KS) + i);
+            });
+            // The maximum is needed when the tile is not lazy, or when a lazy tile's row sums say that some P of
+            // the first half left the comfortable range: one path for both (then P0 is formed again).
+            bool slow = !lazy;
+            if (lazy) slow = __builtin_amdgcn_ballot_w64(!(h0.ta + h0.tb <= SUM_LIMIT)) != 0;
+            if (slow) {
+                // (the first set of P0 counts as used here too: otherwise the compiler moves its exponentials
+                // out from behind the MFMAs into the branch that keeps them)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) asm volatile("" ::"v"(h0.w[i]));
+                __builtin_amdgcn_s_setprio(0);
+                if (td.kind != TILE_FULL) {
+                    mask_half(s0, td.vlo, 0, td.kind, td.m0, td.key0);
+                    mask_half(s1, td.vhi, 1, td.kind, td.m0, td.key0);
+                }
+                rebase(s0, s1);
+                exp_half(s0, h0);
+                __builtin_amdgcn_s_setprio(2);
             }
-            attend(vtile, s0, s1);
+            float sum0 = h0.ta + h0.tb;
+            pv_half(vtile, 0, h0, [&](int j) {
+#pragma unroll
+                for (int i = 0; i < 8 / (2 * DT); ++i) exp_piece(s1, h1, j * (8 / (2 * DT)) + i);
+            });
+            if (lazy && __builtin_amdgcn_ballot_w64(!(h1.ta + h1.tb <= SUM_LIMIT))) {
+                bump(s1, nullptr, &sum0);
+                exp_half(s1, h1);
+            }
+            pv_half(vtile, 1, h1, [](int) {});
+            __builtin_amdgcn_s_setprio(0);
+            l_run += sum0 + (h1.ta + h1.tb);
         }
         __syncthreads();
     }
 
     // ---- epilogue ----
-    l_run += l_alt;
+    // (Measured and dropped, twice each way: staging the rows through LDS so that they leave as whole 256-byte rows
+    // -- this once-per-wave code runs from a cold instruction cache and the staging cost what the better store
+    // pattern gained; and merging the splits here, by the last workgroup of a set to arrive -- device-scope stores
+    // and loads for the partial rows plus one release/acquire ticket per workgroup made the call 1 us shorter at
+    // 5 K keys and 5 % longer at 65 K, where every finishing workgroup's cache invalidation hits the others.)
     l_run += partner32(l_run, gh != 0);
     if (!row_ok) return;
     const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
@@ -911,7 +1017,9 @@ int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt, int mt
     }
     const int64_t nb = (int64_t)p.num_kv_heads * nsplit * (mt_total > 0 ? (int64_t)mt_total : (int64_t)p.batch * n_mt);
     if (nb <= 0 || nb > 0x7fffffff) return LAZYATTN_E_SHAPE;
-    hipLaunchKernelGGL(kern, dim3((unsigned)nb), dim3((NC + 4) * 64), LDS_BYTES, stream, p, nsplit, n_mt, mt_total);
+    const MfmaDivs dv{FastDiv((uint32_t)n_mt), FastDiv((uint32_t)nsplit), FastDiv((uint32_t)p.num_kv_heads),
+                      FastDiv((uint32_t)(p.num_q_heads / p.num_kv_heads))};
+    hipLaunchKernelGGL(kern, dim3((unsigned)nb), dim3((NC + 4) * 64), LDS_BYTES, stream, p, nsplit, n_mt, mt_total, dv);
     return hipGetLastError() == hipSuccess ? LAZYATTN_OK : LAZYATTN_E_LAUNCH;
 }
 

@@ -130,11 +130,11 @@ def dtype_code(dt: torch.dtype) -> int:
 _workspaces: dict = {}
 
 
-def workspace(device: torch.device, nbytes: int) -> Optional[torch.Tensor]:
-    """Per-device scratch for split-KV partials, grown on demand and kept."""
+def workspace(device: torch.device, nbytes: int, kind: str = "prefill") -> Optional[torch.Tensor]:
+    """Per-device scratch for split-KV partials, grown on demand and kept; one per kind of call."""
     if nbytes <= 0:
         return None
-    key = (device.type, device.index)
+    key = (device.type, device.index, kind)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
         buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)

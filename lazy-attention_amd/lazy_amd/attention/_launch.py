@@ -125,7 +125,7 @@ class PrefillPlan:
         self._ws = None
         nbytes = (self._lib.lazyattn_paged_decode_workspace_bytes(params) if decode
                   else self._lib.lazyattn_prefill_workspace_bytes(params))
-        self._ws = _ffi.workspace(device, nbytes)
+        self._ws = _ffi.workspace(device, nbytes, "decode" if decode else "prefill")
         if self._ws is not None:
             params.workspace = self._ws.data_ptr()
             params.workspace_bytes = self._ws.numel()

@@ -125,3 +125,35 @@ def test_table_version_of_inference_tensors():
     v0 = _ffi.table_version(u)
     u.add_(1)
     assert _ffi.table_version(u) == v0 + 1
+
+
+def test_fast_division_is_exact(tmp_path):
+    """csrc/fastdiv.hpp (the kernel prologue's divisions by launch-time constants): the multiply-high form equals
+    n / d for divisors from 1 to 2^32 - 1 and numerators over the whole 32-bit range, edges included."""
+    import subprocess
+    src = tmp_path / "fd.cpp"
+    src.write_text('''
+#include "fastdiv.hpp"
+#include <cstdio>
+int main() {
+    using lazyattn::FastDiv;
+    unsigned long long bad = 0;
+    const uint32_t ds[] = {1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 12, 16, 17, 31, 32, 33, 63, 64, 65, 100, 127, 128, 1000, 4096,
+                           65535, 65536, 65537, 1000003, 0x7fffffffu, 0x80000000u, 0xfffffffeu, 0xffffffffu};
+    for (uint32_t d : ds) {
+        const FastDiv f(d);
+        for (uint64_t i = 0; i < 400000; ++i) {
+            uint32_t n = (uint32_t)(i * 2654435761ull + i * i);
+            if (i < 100000) n = (uint32_t)i;
+            if (i > 300000) n = 0xffffffffu - (uint32_t)(i - 300000);
+            const uint32_t q = f.quot(n);
+            if (q != n / d || f.rem(n, q) != n % d) ++bad;
+        }
+    }
+    printf("%llu\\n", bad);
+    return bad != 0;
+}
+''')
+    exe = tmp_path / "fd"
+    subprocess.check_call(["g++", "-O2", "-std=c++17", "-I", os.path.join(ROOT, "lazy-attention_amd", "csrc"), str(src), "-o", str(exe)])
+    assert subprocess.check_output([str(exe)]).split()[0] == b"0"

@@ -307,13 +307,20 @@ def test_mfma_split_partials_keep_their_precision_at_any_magnitude(scale):
 
 
 @pytest.mark.parametrize("nsplit", [1, 2])
-def test_mfma_softmax_reference_moves_down_then_far_up(nsplit):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("hot_page,boost", [(9, 1.0), (11, 1.0), (10, 0.75), (8, 0.3)])
+def test_mfma_softmax_reference_moves_down_then_far_up(nsplit, dtype, hot_page, boost):
     """Un-rotated requests, so the scores are under control: every query row is 3u, the first 64 cached keys
     of every request are -3u (scores of about -150 in log2 units, the first tile's maximum), a later page
-    is +u (about +50, far above everything before).  The kernel's softmax reference first settles on the
-    very negative first tile, then jumps by ~150 and again by ~50; the early keys end with weight ~0."""
-    print(f"case: mfma softmax reference jumps nsplit={nsplit}", flush=True)
-    w = _ragged("block_uniform")
+    is +boost*u (about +50 * boost, far above everything before; the other keys are random, within +-15).  The
+    kernel's softmax reference first settles on the very negative first tile, moves up by ~150 on the second,
+    and on the third tile meets the hot page -- in its first or second half (pages 8, 9 / 10, 11), by an amount
+    that does (boost 1: P would be 2^40 and more) or does not (0.75, 0.3: P of 2^10 - 2^30 is carried; float16
+    moves at 2^12) make it move again.  The early keys end with weight ~0."""
+    print(f"case: mfma softmax reference jumps nsplit={nsplit} {dtype} page {hot_page} boost {boost}", flush=True)
+    w = wl.make_workload("ragged", dtype=dtype, **GEOM, doc_lens=[100, 16, 333, 70, 5, 250],
+                         requests=[[3, 1, 0], [2], [0, 2, 3, 1, 5], [4], []], q_lens=[70, 1, 9, 33, 130],
+                         variant="block_uniform", seed=31)
     lazy = torch.zeros(5, dtype=torch.bool)
     u = torch.ones(128)
     w.q[:] = (3.0 * u).to(w.q.dtype)
@@ -322,13 +329,13 @@ def test_mfma_softmax_reference_moves_down_then_far_up(nsplit):
         n_ctx = int(w.b_seq_len[b]) - int(w.b_start_loc[b + 1] - w.b_start_loc[b])
         for j in range(min(4, n_ctx // 16)):
             w.k_cache[int(w.block_table[b, j])] = (-3.0 * u).view(128 // x, 1, x).expand(hkv, 128 // x, 16, x).to(w.k_cache.dtype)
-        if n_ctx // 16 > 9:
-            w.k_cache[int(w.block_table[b, 9])] = u.view(128 // x, 1, x).expand(hkv, 128 // x, 16, x).to(w.k_cache.dtype)
+        if n_ctx // 16 > hot_page:
+            w.k_cache[int(w.block_table[b, hot_page])] = (boost * u).view(128 // x, 1, x).expand(hkv, 128 // x, 16, x).to(w.k_cache.dtype)
     ref = run_oracle(w, is_lazy=lazy)
     got = run_op(w.to(DEV), kernel=_ffi.KERNEL_MFMA, num_splits=nsplit, is_lazy=lazy.to(DEV)).cpu()
     assert torch.isfinite(got.float()).all()
     e = _err(got, ref)
-    assert e < 2e-2, e
+    assert e < (2e-2 if dtype == torch.bfloat16 else 5e-3), e
 
 
 @pytest.mark.parametrize("table_f32", [False, True])
