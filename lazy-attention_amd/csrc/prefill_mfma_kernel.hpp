@@ -346,6 +346,12 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     if (gatherer) {
         // ====================================================================== gather
         const int gw = wave - NC;                                // this wave's page of every tile
+        // The block-table entries of the first three tiles are requested before anything else is set up: the
+        // scalar loads are a memory round trip, the per-lane set-up below a few hundred instructions from a
+        // cold instruction cache -- the two run side by side.
+        const PageMeta pm0 = load_page(tile_begin * PAGES + gw);
+        const PageMeta pm1 = load_page((tile_begin + 1) * PAGES + gw);
+        PageMeta pm_pend = load_page((tile_begin + 2) * PAGES + gw);
         const int nat_step = (vanilla || pos_mode == LAZYATTN_POS_BLOCK_UNIFORM) ? 0 : BS;
         const bool rot_new = p.rotate_new_k && !vanilla;
         const float k_scale = FP8 ? *p.k_scale : 1.f;
@@ -620,10 +626,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         // the previous iteration); they are rotated into the other LDS buffer while the
         // computing waves work on `tile`, then the loads of tile+2 are issued.
         int nxt_kind = TILE_FULL, nxt_lim = BS;
-        PageMeta pm_pend = load_page((tile_begin + 2) * PAGES + gw);
         if (tile_begin < tile_end) {
-            const PageMeta pm0 = load_page(tile_begin * PAGES + gw);
-            const PageMeta pm1 = load_page((tile_begin + 1) * PAGES + gw);
             const int k0 = issue_loads(tile_begin, pm0);
             store_tile(0, k0, pm0.lim);
             if (tile_begin + 1 < tile_end) {
