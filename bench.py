@@ -49,6 +49,43 @@ def make_plan(g, num_splits, phases):
     return plan, o
 
 
+def host_us_per_call(g, calls=1000, chunk=100):
+    """Host time of one call of the backend's entry point (``chunked_prefill_paged_decode``: the prefill launch,
+    its merge and the q_len==1 launch) on fixed buffers, in microseconds: ``calls`` calls in chunks the GPU is
+    drained between, so no enqueue ever waits for queue space.  Returns (entry point, its launches alone)."""
+    import torch
+    from lazy_amd import _ffi
+    from lazy_amd.attention import _launch
+    from lazy_amd.attention.old_ops.chunked_prefill_paged_decode import chunked_prefill_paged_decode as unrotated
+    from lazy_amd.attention.ops.chunked_prefill_paged_decode import chunked_prefill_paged_decode as block_uniform
+    o = torch.zeros_like(g.q)
+    args = (g.q, g.k, g.v, o, g.kv_cache_dtype, g.k_cache, g.v_cache, g.block_table, g.b_start_loc,
+            g.b_seq_len, g.max_seq_len, g.max_query_len, g.k_scale, g.v_scale)
+    kw = dict(cos_sin_cache=g.cos_sin_cache, rotary_dim=g.q.shape[-1], q_mask=g.q_mask, q_offset=g.q_offset)
+    if g.pos_mode == _ffi.POS_BLOCK_UNIFORM:
+        call = lambda: block_uniform(*args, is_lazy=g.is_lazy, **kw)
+    else:
+        call = lambda: unrotated(*args, is_mepic=g.pos_mode == _ffi.POS_NATURAL, **kw)
+    call()
+    plans = next(reversed(_launch._calls.values()))[1]       # the launches that call was reduced to
+    stream = torch.cuda.current_stream().cuda_stream
+    raw = lambda: [p._entry(p.params, stream) for p in plans]
+    res = []
+    for fn in (call, raw):
+        for _ in range(chunk):
+            fn()
+        spent = 0.0
+        for _ in range(calls // chunk):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(chunk):
+                fn()
+            spent += time.perf_counter() - t0
+        torch.cuda.synchronize()
+        res.append(spent / (calls // chunk * chunk) * 1e6)
+    return res
+
+
 def time_calls(plan, n):
     """ms per call over n back-to-back launches, HIP events on the launch stream."""
     import torch
@@ -354,6 +391,9 @@ def main():
                      # an operand rate, not a measurement of HBM traffic (that is `traffic`)
                      "operand_gbs_algorithmic_cache_warm": round(w.bytes / (main_ms * 1e-3) / 1e9, 1)},
     }
+    entry_us, launches_us = host_us_per_call(g)
+    out["host_us_per_call"] = round(entry_us, 1)            # entry point, repeat call on fixed buffers
+    out["host_us_in_hip_launches"] = round(launches_us, 1)  # of which: the C calls (three kernel launches)
     if not a.no_cpu:
         torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))
         reps_cpu = 5 if a.config in (2, 3) else 3

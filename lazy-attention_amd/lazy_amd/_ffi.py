@@ -128,6 +128,12 @@ def dtype_code(dt: torch.dtype) -> int:
 
 
 _workspaces: dict = {}
+_growth_hooks: list = []
+
+
+def on_workspace_growth(fn) -> None:
+    """``fn()`` runs whenever a workspace is replaced by a larger one (its old address dies)."""
+    _growth_hooks.append(fn)
 
 
 def workspace(device: torch.device, nbytes: int, kind: str = "prefill") -> Optional[torch.Tensor]:
@@ -137,6 +143,9 @@ def workspace(device: torch.device, nbytes: int, kind: str = "prefill") -> Optio
     key = (device.type, device.index, kind)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
+        if buf is not None:
+            for fn in _growth_hooks:
+                fn()
         buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
         _workspaces[key] = buf
     return buf

@@ -3,11 +3,59 @@
 ``old_ops/prefix_prefill.py:437-486``) and the hand-off to the C ABI."""
 from __future__ import annotations
 
+from collections import OrderedDict
 from typing import Optional
 
 import torch
 
 from .. import _ffi
+
+# Repeat calls (a serving loop with fixed buffers, a benchmark) skip validation and the filling of the C struct:
+# the entry points keep the plans of their most recent distinct calls, keyed on every tensor's address, shape,
+# strides and dtype plus the scalar arguments.  A plan is a pure function of that key -- it holds no reference to
+# the caller's tensors -- unless making it had to convert an operand (int64 tables, a host-side scale, a 0/1
+# ``is_lazy``), whose copy depends on the operand's contents: such calls are validated every time.
+_calls: "OrderedDict" = OrderedDict()
+_CALLS_MAX = 64
+
+
+def call_key(tag, tensors, scalars):
+    return (tag, scalars, tuple([None if t is None else (t.data_ptr(), t.shape, t.stride(), t.dtype)
+                                 for t in tensors]))
+
+
+def recall(key, table):
+    """The plans remembered for this call, or None.  ``table`` is the caller's cos/sin table: its edit counter
+    is compared because the plans point at a re-laid-out copy of it."""
+    hit = _calls.get(key)
+    if hit is None:
+        return None
+    if hit[0] != (None if table is None else _ffi.table_version(table)):
+        del _calls[key]
+        return None
+    _calls.move_to_end(key)
+    return hit[1]
+
+
+def remember(key, plans, table) -> None:
+    if not all(p.repeatable for p in plans):
+        return
+    while len(_calls) >= _CALLS_MAX:
+        _calls.popitem(last=False)
+    _calls[key] = (None if table is None else _ffi.table_version(table), tuple(p.detached() for p in plans))
+
+
+def run_plans(plans) -> None:
+    stream = torch._C._cuda_getCurrentRawStream(plans[0].device.index)
+    for p in plans:
+        p.run(stream)
+
+
+def forget_calls() -> None:
+    _calls.clear()
+
+
+_ffi.on_workspace_growth(forget_calls)      # remembered plans point into the old buffer
 
 
 def _cache_code(kv_cache_dtype: str, k_cache: torch.Tensor, v_cache: torch.Tensor, q_dtype) -> int:
@@ -80,6 +128,7 @@ def launch_prefill(*, q, k, v, o, kv_cache_dtype, k_cache, v_cache, b_loc, b_sta
         raise ValueError("cos_sin_cache is required")
     if packed_block_table is not None:
         assert decode and packed_block_table.dtype == torch.int64
+    given = (b_seq_len, is_lazy, k_scale, v_scale, b_loc, q_offset, q_mask)
     if b_start_loc.dtype != b_seq_len.dtype:
         b_seq_len = b_seq_len.to(b_start_loc.dtype)
     if b_start_loc.dtype not in (torch.int32, torch.int64):
@@ -94,6 +143,9 @@ def launch_prefill(*, q, k, v, o, kv_cache_dtype, k_cache, v_cache, b_loc, b_sta
     else:
         k_scale = v_scale = None
     b_loc, q_offset, q_mask = _i32(b_loc), _i32(q_offset), _i32(q_mask)
+    if cache_code not in (_ffi.FP8_E4M3, _ffi.FP8_E5M2):
+        given = given[:2] + (None, None) + given[4:]
+    repeatable = all(a is b for a, b in zip(given, (b_seq_len, is_lazy, k_scale, v_scale, b_loc, q_offset, q_mask)))
     packed = None
     if not decode and q.dtype in (torch.bfloat16, torch.float16) and pos_mode != _ffi.POS_BLOCK_UNIFORM:
         packed = _ffi.packed_cos_sin(cos_sin_cache)      # built once per table
@@ -107,8 +159,8 @@ def launch_prefill(*, q, k, v, o, kv_cache_dtype, k_cache, v_cache, b_loc, b_sta
         kernel=kernel, num_splits=num_splits, phases=phases, max_seq_len=max_seq_len, packed_table=packed,
         packed_block_table=packed_block_table, rope_freqs=rope_freqs)
     plan = PrefillPlan(p, dev, decode, keep=(q, k, v, o, k_cache, v_cache, b_loc, b_start_loc, b_seq_len,
-                                            cos_sin_cache, q_offset, q_mask, is_lazy, k_scale, v_scale, packed,
-                                            packed_block_table, rope_freqs))
+                                            cos_sin_cache, q_offset, q_mask, is_lazy, k_scale, v_scale,
+                                            packed_block_table, rope_freqs), own=(packed,), repeatable=repeatable)
     if _return_plan:
         return plan
     plan.run()
@@ -119,9 +171,11 @@ class PrefillPlan:
     ``run()`` enqueues it on torch's current stream; calling it again repeats the call
     on the same operands (a serving loop re-uses the plan while shapes stay fixed)."""
 
-    def __init__(self, params, device, decode, keep):
-        self.params, self.device, self.decode, self._keep = params, device, decode, keep
+    def __init__(self, params, device, decode, keep, own=(), repeatable=False):
+        self.params, self.device, self.decode, self._keep, self._own = params, device, decode, keep, own
+        self.repeatable = repeatable        # no operand had to be converted: the struct depends on the key alone
         self._lib = _ffi.lib()
+        self._entry = self._lib.lazyattn_paged_decode_rotary if decode else self._lib.lazyattn_prefix_prefill
         self._ws = None
         nbytes = (self._lib.lazyattn_paged_decode_workspace_bytes(params) if decode
                   else self._lib.lazyattn_prefill_workspace_bytes(params))
@@ -130,13 +184,24 @@ class PrefillPlan:
             params.workspace = self._ws.data_ptr()
             params.workspace_bytes = self._ws.numel()
 
-    def run(self) -> None:
-        stream = torch.cuda.current_stream(self.device).cuda_stream
-        if self.decode:
-            _ffi.check(self._lib.lazyattn_paged_decode_rotary(self.params, stream),
-                       "lazyattn_paged_decode_rotary")
-        else:
-            _ffi.check(self._lib.lazyattn_prefix_prefill(self.params, stream), "lazyattn_prefix_prefill")
+    def run(self, stream: Optional[int] = None) -> None:
+        if stream is None:
+            stream = torch._C._cuda_getCurrentRawStream(self.device.index)
+        rc = self._entry(self.params, stream)
+        if rc:
+            _ffi.check(rc, "lazyattn_paged_decode_rotary" if self.decode else "lazyattn_prefix_prefill")
+
+    def also_keep(self, *tensors) -> None:
+        """Tensors the entry point made for this call whose contents do not depend on the caller's (an all-false
+        ``is_lazy``, a zero ``q_offset``): they live as long as the plan."""
+        self._own = self._own + tensors
+
+    def detached(self) -> "PrefillPlan":
+        """The same call without references to the caller's tensors (what the entry points remember)."""
+        twin = object.__new__(PrefillPlan)
+        twin.__dict__.update(self.__dict__)
+        twin._keep = ()
+        return twin
 
     def run_static_scratch(self) -> None:
         """The same prefill call through the entry point that allocates nothing: the split-KV partials go to

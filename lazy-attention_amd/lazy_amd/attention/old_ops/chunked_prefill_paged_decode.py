@@ -20,24 +20,35 @@ def chunked_prefill_paged_decode(query, key, value, output, kv_cache_dtype, key_
                                  sm_scale=None, rotary_dim=None, cos_sin_cache=None,
                                  is_neox_style=True, q_offset=None, q_mask=None,
                                  is_mepic: bool = True, force_fp32_rotary: bool = False):
+    sig = _launch.call_key(
+        "un-rotated", (query, key, value, output, key_cache, value_cache, block_table, query_start_loc, seq_lens,
+                       k_scale, v_scale, alibi_slopes, cos_sin_cache, q_offset, q_mask),
+        (kv_cache_dtype, max_seq_len, max_query_len, sliding_window, sm_scale, rotary_dim, is_neox_style, is_mepic,
+         force_fp32_rotary))
+    plans = _launch.recall(sig, cos_sin_cache)
+    if plans is not None:
+        return _launch.run_plans(plans)
+    plans = []
     if sm_scale is None:
         sm_scale = 1.0 / (query.shape[1] ** 0.5)        # sic: old_ops/chunked...:311-312
     if sliding_window is None or sliding_window <= 0:
         sliding_window = 0
     if max_query_len > 1:
-        context_attention_fwd(
+        plans.append(context_attention_fwd(
             q=query, k=key, v=value, o=output, kv_cache_dtype=kv_cache_dtype, k_cache=key_cache,
             v_cache=value_cache, b_loc=block_table, b_start_loc=query_start_loc, b_seq_len=seq_lens,
             max_seq_len=max_seq_len, max_input_len=max_query_len, k_scale=k_scale, v_scale=v_scale,
             alibi_slopes=alibi_slopes, sliding_window=sliding_window, sm_scale=sm_scale,
             skip_decode=True, rotary_dim=rotary_dim, cos_sin_cache=cos_sin_cache,
             is_neox_style=is_neox_style, q_mask=q_mask, q_offset=q_offset, is_mepic=is_mepic,
-            force_fp32_rotary=force_fp32_rotary)
-    _launch.launch_prefill(
+            force_fp32_rotary=force_fp32_rotary, _return_plan=True))
+    plans.append(_launch.launch_prefill(
         q=query, k=key, v=value, o=output, kv_cache_dtype=kv_cache_dtype, k_cache=key_cache,
         v_cache=value_cache, b_loc=block_table, b_start_loc=query_start_loc, b_seq_len=seq_lens,
         max_input_len=1, max_seq_len=max_seq_len, k_scale=k_scale, v_scale=v_scale, alibi_slopes=alibi_slopes,
         sliding_window=sliding_window, sm_scale=sm_scale, skip_decode=False,
         cos_sin_cache=cos_sin_cache, rotary_dim=rotary_dim, is_neox_style=is_neox_style,
         is_lazy=None, q_offset=None, q_mask=q_mask, pos_mode=_ffi.POS_NATURAL, rotate_new_k=True,
-        fp32_rotary=force_fp32_rotary, decode=True)
+        fp32_rotary=force_fp32_rotary, decode=True, _return_plan=True))
+    _launch.run_plans(plans)
+    _launch.remember(sig, plans, cos_sin_cache)

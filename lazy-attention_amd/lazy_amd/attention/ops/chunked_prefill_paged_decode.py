@@ -52,6 +52,16 @@ def chunked_prefill_paged_decode(query, key, value, output, kv_cache_dtype, key_
                                  q_offset=None, q_mask=None, packed_block_table=None):
     if _env_flag("NO_LAZY") and is_lazy is not None:
         is_lazy.fill_(False)                             # ops/chunked...:66-67
+    compute = _env_flag("LAZY_DECODE_COMPUTE_COS_SIN")   # ops/chunked...:146-151
+    sig = _launch.call_key(
+        "block-uniform", (query, key, value, output, key_cache, value_cache, block_table, query_start_loc, seq_lens,
+                          k_scale, v_scale, alibi_slopes, freqs, cos_sin_cache, is_lazy, q_offset, q_mask,
+                          packed_block_table),
+        (kv_cache_dtype, max_seq_len, max_query_len, sliding_window, sm_scale, rotary_dim, is_neox_style, compute))
+    plans = _launch.recall(sig, cos_sin_cache)
+    if plans is not None:
+        return _launch.run_plans(plans)
+    plans, pure = [], True
     if sm_scale is None:
         sm_scale = 1.0 / (query.shape[1] ** 0.5)         # sic: ops/chunked...:71-72
     if sliding_window is None or sliding_window <= 0:
@@ -62,15 +72,18 @@ def chunked_prefill_paged_decode(query, key, value, output, kv_cache_dtype, key_
             _, off, msk = unpack_block_table(packed_block_table)
             pq_offset = off if q_offset is None else q_offset
             pq_mask = msk if q_mask is None else q_mask
-        context_attention_fwd(
+            pure = False                                 # copies of the table's contents
+        plans.append(context_attention_fwd(
             q=query, k=key, v=value, o=output, kv_cache_dtype=kv_cache_dtype, k_cache=key_cache,
             v_cache=value_cache, b_loc=block_table, b_start_loc=query_start_loc, b_seq_len=seq_lens,
             max_seq_len=max_seq_len, max_input_len=max_query_len, k_scale=k_scale, v_scale=v_scale,
             alibi_slopes=alibi_slopes, sliding_window=sliding_window, sm_scale=sm_scale,
             skip_decode=True, rotary_dim=rotary_dim, cos_sin_cache=cos_sin_cache,
-            is_neox_style=is_neox_style, is_lazy=is_lazy, q_offset=pq_offset, q_mask=pq_mask)
+            is_neox_style=is_neox_style, is_lazy=is_lazy, q_offset=pq_offset, q_mask=pq_mask, _return_plan=True))
+    made = ()
     if is_lazy is None:
         is_lazy = torch.zeros(seq_lens.shape[0], dtype=torch.bool, device=query.device)
+        made = (is_lazy,)
     streaming = _streaming_decode_covers(query, value_cache)
     packed = packed_block_table if streaming else None
     if packed is None:
@@ -78,16 +91,26 @@ def chunked_prefill_paged_decode(query, key, value, output, kv_cache_dtype, key_
             _, off, msk = unpack_block_table(packed_block_table)
             q_offset = off if q_offset is None else q_offset
             q_mask = msk if q_mask is None else q_mask
+            pure = False
         if q_offset is None:
             q_offset = torch.zeros_like(block_table, dtype=torch.int32)
+            made += (q_offset,)
     rope_freqs = None
-    if streaming and _env_flag("LAZY_DECODE_COMPUTE_COS_SIN"):           # ops/chunked...:146-151
-        rope_freqs = freqs if freqs is not None else _rope.rope_freqs(rope_meta, query.shape[2], query.device)
-    _launch.launch_prefill(
+    if streaming and compute:
+        if freqs is not None:
+            rope_freqs = freqs
+        else:
+            rope_freqs = _rope.rope_freqs(rope_meta, query.shape[2], query.device)
+            pure = False                                 # rope_meta is not part of the key
+    plans.append(_launch.launch_prefill(
         q=query, k=key, v=value, o=output, kv_cache_dtype=kv_cache_dtype, k_cache=key_cache,
         v_cache=value_cache, b_loc=block_table, b_start_loc=query_start_loc, b_seq_len=seq_lens,
         max_input_len=1, max_seq_len=max_seq_len, k_scale=k_scale, v_scale=v_scale, alibi_slopes=alibi_slopes,
         sliding_window=sliding_window, sm_scale=sm_scale, skip_decode=False,
         cos_sin_cache=cos_sin_cache, rotary_dim=rotary_dim, is_neox_style=is_neox_style,
         is_lazy=is_lazy, q_offset=q_offset, q_mask=q_mask, pos_mode=_ffi.POS_BLOCK_UNIFORM,
-        rotate_new_k=False, decode=True, packed_block_table=packed, rope_freqs=rope_freqs)
+        rotate_new_k=False, decode=True, packed_block_table=packed, rope_freqs=rope_freqs, _return_plan=True))
+    plans[-1].also_keep(*made)
+    _launch.run_plans(plans)
+    if pure:
+        _launch.remember(sig, plans, cos_sin_cache)

@@ -150,3 +150,66 @@ def test_tables_made_under_inference_mode():
     # (the q_len==1 rows of this variant are rotated at their natural positions, old_ops/chunked...:204-213)
     err = (out.cpu().float() - ref.float()).abs().max().item()
     assert err < 2e-2, err
+
+
+def _call(entry, variant, g, out, packed=None, lazy=None, block_table=None):
+    bt = g.block_table if block_table is None else block_table
+    if variant == "natural":
+        entry(g.q, g.k, g.v, out, "auto", g.k_cache, g.v_cache, bt, g.b_start_loc, g.b_seq_len,
+              g.max_seq_len, g.max_query_len, g.k_scale, g.v_scale, sm_scale=128 ** -0.5, rotary_dim=128,
+              cos_sin_cache=g.cos_sin_cache, q_mask=g.q_mask)
+    else:
+        entry(g.q, g.k, g.v, out, "auto", g.k_cache, g.v_cache, bt, g.b_start_loc, g.b_seq_len, g.max_seq_len,
+              g.max_query_len, g.k_scale, g.v_scale, sm_scale=128 ** -0.5, rotary_dim=128,
+              cos_sin_cache=g.cos_sin_cache, is_lazy=lazy, q_offset=g.q_offset, q_mask=g.q_mask,
+              packed_block_table=packed)         # all three tables, as backends/triton_attn.py:137-185 passes them
+
+
+@pytest.mark.parametrize("variant", ["natural", "block_uniform"])
+def test_repeat_calls_on_the_same_buffers_follow_their_contents(variant):
+    """A serving loop calls with the same buffers at the same addresses and new contents.  The entry points
+    remember the validated call (addresses, shapes, strides, scalars) and skip straight to the launch: the
+    second result must be that of the NEW contents, and the call must have been served from memory."""
+    from lazy_amd.attention import _launch
+    print(f"case: repeat calls {variant}", flush=True)
+    entry = entry_unrotated if variant == "natural" else entry_block_uniform
+    lazy_host = torch.tensor([True, True, False, False]) if variant == "block_uniform" else None
+    first, second = _mixed(variant, torch.bfloat16, 128, seed=51), _mixed(variant, torch.bfloat16, 128, seed=52)
+    g = first.to(DEV)
+    lazy = lazy_host.to(DEV) if lazy_host is not None else None
+    pack = lambda w: (w.block_table.long() << 32) | (w.q_offset.long() << 16) | w.q_mask.long()
+    packed = pack(g) if variant == "block_uniform" else None
+    out = torch.full_like(g.q, 5.0)
+    _launch.forget_calls()
+    _call(entry, variant, g, out, packed, lazy)
+    assert (out.cpu().float() - _expected(first, lazy_host).float()).abs().max().item() < 2e-2
+    assert len(_launch._calls) == 1
+    for name in ("q", "k", "v", "k_cache", "v_cache", "block_table", "q_mask", "q_offset"):
+        if getattr(g, name) is not None:
+            getattr(g, name).copy_(getattr(second, name))
+    if packed is not None:
+        packed.copy_(pack(second))
+    out.fill_(5.0)
+    _call(entry, variant, g, out, packed, lazy)
+    assert len(_launch._calls) == 1
+    assert (out.cpu().float() - _expected(second, lazy_host).float()).abs().max().item() < 2e-2
+    # an edit of the cos/sin table is seen (the kernels read a re-laid-out copy of it)
+    other = wl.cos_sin_table(second.cos_sin_cache.shape[0], 128, 10000.0, torch.bfloat16)
+    g.cos_sin_cache.copy_(other)
+    second.cos_sin_cache.copy_(other)
+    out.fill_(5.0)
+    _call(entry, variant, g, out, packed, lazy)
+    assert (out.cpu().float() - _expected(second, lazy_host).float()).abs().max().item() < 2e-2
+    # a table that must be converted (int64 here) is converted on every call, so its new contents are seen too
+    wide = g.block_table.long()
+    out.fill_(5.0)
+    _call(entry, variant, g, out, packed, lazy, block_table=wide)
+    assert (out.cpu().float() - _expected(second, lazy_host).float()).abs().max().item() < 2e-2
+    if variant == "natural":
+        wide.copy_(first.block_table)
+        for name in ("q", "k", "v", "k_cache", "v_cache", "q_mask"):
+            getattr(g, name).copy_(getattr(first, name))
+        first.cos_sin_cache.copy_(other)
+        out.fill_(5.0)
+        _call(entry, variant, g, out, packed, lazy, block_table=wide)
+        assert (out.cpu().float() - _expected(first, lazy_host).float()).abs().max().item() < 2e-2
