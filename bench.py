@@ -27,7 +27,9 @@ PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
 # WRITE_SIZE, each scaled by what the same counter reads for a 256 MiB copy; summary under profiles/).
 # Counters cannot be read from inside this script, so the figure is the committed measurement of the
 # named workload; workloads without one report null.
-MEASURED_TRAFFIC_BYTES = {"c2_8b_bf16_10x512_q128": 43_400_000, "d1_8b_bf16_decode_32req_20x256": 683_700_000}
+MEASURED_TRAFFIC_BYTES = {"c2_8b_bf16_10x512_q128": 43_200_000, "c3_8b_bf16_pool64x256_16req_x20_q64": 241_400_000,
+                          "c4_8b_bf16_64x1024_q256": 448_400_000, "c5_8b_fp8kv_8req_32x512_q128": 336_100_000,
+                          "d1_8b_bf16_decode_32req_20x256": 683_600_000}
 PEAK_HBM_GBS = 8000.0
 
 
@@ -308,6 +310,8 @@ def main():
     ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5])
     ap.add_argument("--num-splits", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-host-timing", action="store_true",
+                    help="skip the 1 100 entry-point calls that measure host_us_per_call (profiler runs)")
     ap.add_argument("--path", choices=["prefill", "decode", "rope_write", "reposition"], default="prefill",
                     help="prefill: the headline prefix-prefill call (default); decode: the q_len==1 kernel; "
                          "rope_write: Q rotary + paged-cache write of the new tokens; reposition: copy-on-write block "
@@ -391,9 +395,10 @@ def main():
                      # an operand rate, not a measurement of HBM traffic (that is `traffic`)
                      "operand_gbs_algorithmic_cache_warm": round(w.bytes / (main_ms * 1e-3) / 1e9, 1)},
     }
-    entry_us, launches_us = host_us_per_call(g)
-    out["host_us_per_call"] = round(entry_us, 1)            # entry point, repeat call on fixed buffers
-    out["host_us_in_hip_launches"] = round(launches_us, 1)  # of which: the C calls (three kernel launches)
+    if not a.no_host_timing:
+        entry_us, launches_us = host_us_per_call(g)
+        out["host_us_per_call"] = round(entry_us, 1)            # entry point, repeat call on fixed buffers
+        out["host_us_in_hip_launches"] = round(launches_us, 1)  # of which: the C calls (four kernel launches)
     if not a.no_cpu:
         torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))
         reps_cpu = 5 if a.config in (2, 3) else 3
