@@ -35,6 +35,7 @@
 #include "elem16.hpp"
 #include "fastdiv.hpp"
 #include <atomic>
+#include <type_traits>
 
 namespace lazyattn {
 
@@ -118,6 +119,23 @@ template <int KIND> __device__ __forceinline__ f32x2_t cvt_fp8x2(uint32_t w) {
     if constexpr (KIND == 2) return __builtin_amdgcn_cvt_pk_f32_bf8(w, false);
     else return __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
 }
+// 8 fp8 bytes -> floats, unscaled
+template <int KIND> __device__ __forceinline__ void unpack8_fp8_raw(uint32_t lo, uint32_t hi, float *f) {
+    f32x2_t a, b, c, d;
+    if constexpr (KIND == 2) {
+        a = __builtin_amdgcn_cvt_pk_f32_bf8(lo, false); b = __builtin_amdgcn_cvt_pk_f32_bf8(lo, true);
+        c = __builtin_amdgcn_cvt_pk_f32_bf8(hi, false); d = __builtin_amdgcn_cvt_pk_f32_bf8(hi, true);
+    } else {
+        a = __builtin_amdgcn_cvt_pk_f32_fp8(lo, false); b = __builtin_amdgcn_cvt_pk_f32_fp8(lo, true);
+        c = __builtin_amdgcn_cvt_pk_f32_fp8(hi, false); d = __builtin_amdgcn_cvt_pk_f32_fp8(hi, true);
+    }
+    f[0] = a[0]; f[1] = a[1]; f[2] = b[0]; f[3] = b[1]; f[4] = c[0]; f[5] = c[1]; f[6] = d[0]; f[7] = d[1];
+}
+// two fp8 bytes (low or high half of w) -> two bf16 in one word, exact (every fp8 value is a bf16 value)
+template <int KIND, bool HIGH> __device__ __forceinline__ uint32_t fp8x2_to_bf16x2(uint32_t w) {
+    if constexpr (KIND == 2) return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_bf8(w, 1.0f, HIGH));
+    else return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, HIGH));
+}
 // 8 fp8 bytes -> (float * scale) rounded to the query type, as floats  (old_ops:239-241)
 template <typename T, int KIND> __device__ __forceinline__ void unpack8_fp8(uint32_t lo, uint32_t hi, float scale, float *f) {
     const f32x2_t a = cvt_fp8x2<KIND>(lo), b = cvt_fp8x2<KIND>(lo >> 16);
@@ -164,6 +182,14 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     constexpr int KV_BYTES = G::KV_BYTES, KS = G::KS, DT = G::DT;
     constexpr int KI = G::K_ITEMS, VI = G::V_ITEMS;   // a page has HD K items (HD/16 chunk pairs x 16 slots) and 2 HD V items
     constexpr int VI_CTX = FP8 ? VI / 2 : VI;        // an fp8 page row of 16 slots is one 16-byte item
+    // fp8 pages under bf16 operands: the cache scales leave the gather.  Rotation and P.V are linear, so
+    // k_scale goes into the factor Q is multiplied by anyway and v_scale into the final 1/l; the pages' bytes are
+    // converted and used as they are (fp8 -> bf16 is exact), and the few new-token keys and values, which are
+    // not quantised, are divided by the scales instead.  Against scaling every element and rounding it to bf16
+    // first (old_ops:239-241) this saves the gathering waves a multiply and a rounding per element and differs by
+    // less than that one rounding (nothing at all for power-of-two scales, 1.0 included).  float16 operands keep
+    // the element-wise scaling: raw e5m2 values can leave the half range.
+    constexpr bool FOLD = FP8 != 0 && std::is_same<T, bf16_t>::value;
     constexpr uint32_t TSZ = sizeof(TT);
     using E = Elem<T>;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -356,6 +382,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         const bool rot_new = p.rotate_new_k && !vanilla;
         const float k_scale = FP8 ? *p.k_scale : 1.f;
         const float v_scale = FP8 ? *p.v_scale : 1.f;
+        const float k_unscale = FOLD ? 1.f / k_scale : 1.f, v_unscale = FOLD ? 1.f / v_scale : 1.f;
         const uint8_t *kc_base = (const uint8_t *)p.k_cache + (int64_t)g * p.kc_stride[1] * (FP8 ? 1 : 2);
         const uint8_t *vc_base = (const uint8_t *)p.v_cache + (int64_t)g * p.vc_stride[1] * (FP8 ? 1 : 2);
         const int64_t kc_page_bytes = p.kc_stride[0] * (FP8 ? 1 : 2);
@@ -527,7 +554,10 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         // ---- rotate the K items in fp32 and write them to a K tile ----
         auto store_k_item = [&](int i, uint8_t *ktile, int kind) {
             float a[8], bb[8], cs[8], sn[8];
-            if (FP8 && kind != TILE_NEW) {
+            if (FOLD && kind != TILE_NEW) {
+                unpack8_fp8_raw<FP8>(kr[i].k1.x, kr[i].k1.y, a);
+                unpack8_fp8_raw<FP8>(kr[i].k2.x, kr[i].k2.y, bb);
+            } else if (FP8 && kind != TILE_NEW) {
                 unpack8_fp8<T, FP8>(kr[i].k1.x, kr[i].k1.y, k_scale, a);
                 unpack8_fp8<T, FP8>(kr[i].k2.x, kr[i].k2.y, k_scale, bb);
             } else {
@@ -541,6 +571,10 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             for (int e = 0; e < 8; ++e) {
                 x[e] = a[e] * cs[e] - bb[e] * sn[e];                             // old_ops:253
                 y[e] = a[e] * sn[e] + bb[e] * cs[e];                             // old_ops:254
+            }
+            if (FOLD && kind == TILE_NEW) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) { x[e] *= k_unscale; y[e] *= k_unscale; }
             }
             *reinterpret_cast<uint4 *>(ktile + kr[i].lds_off) = make_uint4(
                 E::pack(x[0], x[1]), E::pack(x[2], x[3]), E::pack(x[4], x[5]), E::pack(x[6], x[7]));
@@ -561,6 +595,16 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                 uint32_t o2[4][2];
 #pragma unroll
                 for (int q4 = 0; q4 < 4; ++q4) {
+                    if constexpr (FOLD) {
+                        o2[q4][0] = fp8x2_to_bf16x2<FP8, false>(w[q4]);
+                        o2[q4][1] = fp8x2_to_bf16x2<FP8, true>(w[q4]);
+                        if (kind == TILE_EDGE) {                 // masked slots contribute nothing, whatever they hold
+#pragma unroll
+                            for (int s = 0; s < 4; ++s)
+                                if (q4 * 4 + s >= lim) o2[q4][s >> 1] &= (s & 1) ? 0x0000ffffu : 0xffff0000u;
+                        }
+                        continue;
+                    }
                     const f32x2_t lo = cvt_fp8x2<FP8>(w[q4]);
                     const f32x2_t hi = cvt_fp8x2<FP8>(w[q4] >> 16);
                     float f[4] = {lo[0] * v_scale, lo[1] * v_scale, hi[0] * v_scale, hi[1] * v_scale};
@@ -603,7 +647,11 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                     const int dc = idx & (D / 8 - 1), slot = idx / (D / 8);
                     uint8_t *dst = vtile + gw * V_PAGE + ((slot >> 2) & 1) * V_G + (dc * 8) * 16 + (slot >> 3) * 8 +
                                    (slot & 3) * 2;
-                    const uint32_t w[4] = {vr[i].x, vr[i].y, vr[i].z, vr[i].w};
+                    uint32_t w[4] = {vr[i].x, vr[i].y, vr[i].z, vr[i].w};
+                    if constexpr (FOLD) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) w[e] = E::pack(E::lo(w[e]) * v_unscale, E::hi(w[e]) * v_unscale);
+                    }
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         *reinterpret_cast<uint16_t *>(dst + (2 * e) * 16) = (uint16_t)(w[e] & 0xffffu);
@@ -695,7 +743,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     // delivers the scores in log2 units and no per-score multiply is left in the tile loop (the
     // reference scales the fp32 scores, old_ops:287; the extra rounding of Q is one more relative
     // 2^-9 per element, like the one the rotated K already carries).
-    const float cs2 = p.sm_scale * 1.4426950408889634f;
+    const float cs2 = p.sm_scale * 1.4426950408889634f * (FOLD ? *p.k_scale : 1.f);
     uint8_t *qlds = lds + KV_BYTES + (QREG ? 0 : wave * G::Q_WAVE) + lane * 16;
     uint4 qreg[QREG ? KS : 1];
     {
@@ -956,7 +1004,8 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     // 5 K keys and 5 % longer at 65 K, where every finishing workgroup's cache invalidation hits the others.)
     l_run += partner32(l_run, gh != 0);
     if (!row_ok) return;
-    const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+    const float out_scale = FOLD ? *p.v_scale : 1.f;
+    const float inv = l_run > 0.f ? out_scale / l_run : 0.f;
     if (nsplit == 1) {
         T *op = (T *)p.o + (qs + row) * p.o_stride[0] + (int64_t)h * p.o_stride[1];
 #pragma unroll
