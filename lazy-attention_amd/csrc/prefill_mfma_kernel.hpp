@@ -455,12 +455,24 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         // wherever q_offset is not consulted, nat_step is 0 wherever the fallback is row 0.
         // A page past the context (its slots are all masked) takes the last page's position: the
         // table only has to cover the positions of real keys.
-        struct PageBase { const uint8_t *kb, *tb, *vb; };
+        // The lane offsets are handed out as fresh 32-bit values per page: a load then is "scalar base + 32-bit
+        // lane offset" as it stands.  Left to itself the compiler widens the loop-invariant offsets to 64 bits
+        // once, outside the loop, and then forms every address with a 64-bit vector add.
+        struct PageBase { const uint8_t *kb, *tb, *ts, *vb; uint32_t ko, vo, to[KI]; };
         auto page_base = [&](int tile, const PageMeta &pm) -> PageBase {
             const int j = tile * PAGES + gw;
             const int jp = j < n_pages ? j : n_pages - 1;
             const int pos0 = pm.qo ? pm.qo - 1 + part_pos : jp * nat_step;
-            return PageBase{kc_base + pm.bt * kc_page_bytes, ctab_base + (int64_t)pos0 * pos_bytes, vc_base + pm.bt * vc_page_bytes};
+            PageBase pb;
+            pb.kb = kc_base + pm.bt * kc_page_bytes;
+            pb.tb = ctab_base + (int64_t)pos0 * pos_bytes;
+            pb.ts = pb.tb + sin_delta;
+            pb.vb = vc_base + pm.bt * vc_page_bytes;
+            pb.ko = k_goff; pb.vo = v_goff;
+            asm volatile("" : "+v"(pb.ko), "+v"(pb.vo));
+#pragma unroll
+            for (int i = 0; i < KI; ++i) { pb.to[i] = k_toff[i]; asm volatile("" : "+v"(pb.to[i])); }
+            return pb;
         };
         auto load_k_item = [&](int i, const PageBase &pb) {
             const uint8_t *kb = pb.kb;
@@ -479,22 +491,22 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                 kr[i].k1 = pk_ok[i] ? k1 : z;
                 kr[i].k2 = pk_ok[i] ? k2 : z;
             } else if (FP8) {
-                const uint2 a = ldg8(kb + i * k_item, k_goff), a2 = ldg8(kb + i * k_item + pair, k_goff);
+                const uint2 a = ldg8(kb + i * k_item, pb.ko), a2 = ldg8(kb + i * k_item + pair, pb.ko);
                 kr[i].k1 = make_uint4(a.x, a.y, 0, 0);
                 kr[i].k2 = make_uint4(a2.x, a2.y, 0, 0);
             } else {
-                kr[i].k1 = ldg16(kb + i * k_item, k_goff);
-                kr[i].k2 = ldg16(kb + i * k_item + pair, k_goff);
+                kr[i].k1 = ldg16(kb + i * k_item, pb.ko);
+                kr[i].k2 = ldg16(kb + i * k_item + pair, pb.ko);
             }
-            kr[i].c.load(pb.tb, k_toff[i]);
-            kr[i].s.load(pb.tb, k_toff[i] + sin_delta);
+            kr[i].c.load(pb.tb, pb.to[i]);
+            kr[i].s.load(pb.ts, pb.to[i]);
         };
         auto load_v_item = [&](int i, const PageBase &pb) {
             if constexpr (PAD) {
                 const uint4 t = ldg16(pb.vb, pv[i]);
                 vr[i] = pv_ok[i] ? t : make_uint4(0, 0, 0, 0);
             } else {
-                vr[i] = ldg16(pb.vb + i * v_item, v_goff);
+                vr[i] = ldg16(pb.vb + i * v_item, pb.vo);
             }
         };
         auto issue_loads_ctx = [&](int tile, const PageMeta &pm) {
@@ -986,6 +998,10 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                 for (int i = 0; i < 8 / (2 * DT); ++i) exp_piece(s1, h1, j * (8 / (2 * DT)) + i);
             });
             if (lazy && __builtin_amdgcn_ballot_w64(!(h1.ta + h1.tb <= SUM_LIMIT))) {
+                // (the scores are made opaque here: otherwise half of the row maximum below is computed ahead
+                // of the branch, on every tile)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) asm volatile("" : "+v"(s1[i]));
                 bump(s1, nullptr, &sum0);
                 exp_half(s1, h1);
             }
