@@ -81,8 +81,10 @@ typedef struct lazyattn_prefill_params {
     const void *cos_sin_packed; /* optional: the same table re-laid out by lazyattn_pack_cos_sin_cache()
                                    as [2][rotary_dim/16][packed_rows][8], so that the 16 slots of a page
                                    read 16 consecutive 16-byte chunks; NULL = read the row-major table */
-    const float *k_scale;       /* 1 element, read only for fp8 caches */
-    const float *v_scale;
+    const float *k_scale;       /* 1 element, read only for fp8 caches: key = fp8 value * k_scale (old_ops/prefix_prefill.py:239-241). */
+    const float *v_scale;       /* The matrix-core kernel with bf16 operands applies the two scales to Q and to the final 1/l
+                                   instead of to every cached element (linear, so the same result up to the one rounding of
+                                   the scaled element the reference makes; identical for power-of-two scales). */
     void *workspace;            /* split-KV partials; lazyattn_prefill_workspace_bytes() */
     int64_t workspace_bytes;
 
