@@ -45,5 +45,10 @@ template <typename T> __device__ __forceinline__ float round_to(float x) {
 __device__ __forceinline__ int64_t load_index(const void *p, int64_t i, int bits) {
     return bits == 64 ? ((const int64_t *)p)[i] : (int64_t)((const int32_t *)p)[i];
 }
+// the same for entries known to be non-negative (offsets, lengths): a 32-bit entry is zero-extended, which pairs
+// it with a zero register instead of computing on the loaded value
+__device__ __forceinline__ int64_t load_index_nonneg(const void *p, int64_t i, int bits) {
+    return bits == 64 ? ((const int64_t *)p)[i] : (int64_t)(uint32_t)((const int32_t *)p)[i];
+}
 
 }  // namespace lazyattn

@@ -279,16 +279,96 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         g = (int)dv.kv_heads.rem(bg, b);
     }
 
-    const int64_t qs = load_index(p.b_start_loc, b, p.index_bits);
-    const int q_len = (int)(load_index(p.b_start_loc, b + 1, p.index_bits) - qs);
-    const int ctx_len = (int)(load_index(p.b_seq_len, b, p.index_bits) - q_len);
+    // The request's lengths are requested here, ahead of the gathering waves' per-lane constants: nothing in
+    // those depends on the lengths, and they are a couple of hundred instructions from a cold instruction cache.
+    // (Measured against scalar loads of the three entries in flight together, with and without all kernel
+    // arguments fetched at entry: this form, a vector load per entry, is the fastest of the three by 1-1.5 %.)
+    const int64_t qs = load_index_nonneg(p.b_start_loc, b, p.index_bits);
+    const int64_t qe = load_index_nonneg(p.b_start_loc, b + 1, p.index_bits);
+    const int64_t seq = load_index_nonneg(p.b_seq_len, b, p.index_bits);
+    const float k_scale = FP8 ? *p.k_scale : 1.f;
+    const float v_scale = FP8 ? *p.v_scale : 1.f;
+    const uint8_t lazy_raw = p.is_lazy ? p.is_lazy[b] : (uint8_t)1;
+    __builtin_amdgcn_sched_barrier(0);
+    const int pos_mode = p.pos_mode;
+    // A cache page of 32 slots is handled as two parts of 16: "page" j below is the j-th run of 16 context
+    // slots, part j & 1 of cache page j >> 1.  Its valid slots follow from the page's pad count.
+    const int pshift = p.block_size == 2 * BS ? 1 : 0, part_mask = pshift;
+    const int cache_bs = BS << pshift;
+    const int gw = wave - NC;                                    // gathering waves: this wave's page of every tile
+    // (an un-rotated request of the block-uniform mode reads row 0 for every page, like the mode's other requests
+    // read one row per page: what depends on the request's own flag is decided later)
+    const int nat_step = pos_mode == LAZYATTN_POS_BLOCK_UNIFORM ? 0 : BS;
+    const bool per_token = pos_mode != LAZYATTN_POS_BLOCK_UNIFORM;
+    const uint8_t *tab_base = (const uint8_t *)p.cos_sin_cache;
+    const uint32_t row_bytes = (uint32_t)p.table_stride * TSZ;
+    // per-token rotation of context pages reads the packed table [2][D/16][rows][8]: the 16
+    // slots of a page are 16 consecutive 16-byte chunks there
+    const bool packed_tab = p.cos_sin_packed != nullptr && per_token;
+    // this wave's part of its cache pages (pages of 32 slots: the tile's pages 0, 1 are the two parts of
+    // one cache page, 2, 3 of the next): first slot, and the position step that goes with it
+    const int slot0 = (gw & part_mask) * BS;
+    // K items of a page: 128 = (8 chunks of 8 (d, d+64) pairs) x 16 slots, two per lane
+    uint32_t k_toff[KI];
+    // Cache offsets of a lane's items: item i = item 0 + i * (a wave-uniform stride), so one offset register
+    // serves all of them and the strides go into the scalar page base.
+    // K bf16: [D/8][slots][8] -> item (cp, o) at (cp*slots + o)*16 bytes, cp = lane/16 + 4 i
+    //   fp8 : [D/16][slots][16] -> 8 bytes at chunk cp/2, half cp&1
+    // V bf16: row d = lane/2 + 32 i of `slots` slots, 8 slots (16 bytes) per item; fp8: row d = lane + 64 i, 16 slots
+    uint32_t k_goff = FP8 ? (uint32_t)(((lane >> 5) * cache_bs + slot0 + (lane & 15)) * 16 + ((lane >> 4) & 1) * 8)
+                          : (uint32_t)(((lane >> 4) * cache_bs + slot0 + (lane & 15)) * 16);
+    uint32_t v_goff = FP8 ? (uint32_t)(lane * cache_bs + slot0)
+                          : (uint32_t)((lane >> 1) * cache_bs * 2 + slot0 * 2 + (lane & 1) * 16);
+#pragma unroll
+    for (int i = 0; i < KI; ++i) {
+        const int idx = lane + i * 64;
+        const int o = idx & 15, cp = PAD && (idx >> 4) >= CPr ? 0 : idx >> 4;   // (a padded chunk reads chunk 0 and is zeroed)
+        // block-uniform rotation and un-rotated requests use one table row for the whole page
+        k_toff[i] = packed_tab ? ((uint32_t)cp * (uint32_t)p.packed_rows + (uint32_t)o) * 8 * TSZ
+                               : (per_token ? (uint32_t)o * row_bytes : 0u) + (uint32_t)cp * 8 * TSZ;
+    }
+    // PAD: per-item cache offsets (the chunk of d + Dr/2 is not a fixed distance away in an fp8 page) and
+    // which of the lane's items exist
+    uint32_t pk1[PAD ? KI : 1], pk2[PAD ? KI : 1], pv[PAD ? VI_CTX : 1];
+    bool pk_ok[PAD ? KI : 1], pv_ok[PAD ? VI_CTX : 1];
+    if constexpr (PAD) {
+#pragma unroll
+        for (int i = 0; i < KI; ++i) {
+            const int idx = lane + i * 64, o = idx & 15;
+            pk_ok[i] = (idx >> 4) < CPr;
+            const int c1 = pk_ok[i] ? idx >> 4 : 0, c2 = CPr + c1;                  // 8-element chunks of d and d + Dr/2
+            pk1[i] = FP8 ? (uint32_t)(((c1 >> 1) * cache_bs + slot0 + o) * 16 + (c1 & 1) * 8) : (uint32_t)((c1 * cache_bs + slot0 + o) * 16);
+            pk2[i] = FP8 ? (uint32_t)(((c2 >> 1) * cache_bs + slot0 + o) * 16 + (c2 & 1) * 8) : (uint32_t)((c2 * cache_bs + slot0 + o) * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < VI_CTX; ++i) {
+            const int idx = lane + i * 64;
+            const int d = FP8 ? idx : idx >> 1;
+            pv_ok[i] = d < Dr;
+            const int dc = pv_ok[i] ? d : 0;
+            pv[i] = FP8 ? (uint32_t)(dc * cache_bs + slot0) : (uint32_t)(dc * cache_bs * 2 + slot0 * 2 + (idx & 1) * 16);
+        }
+    }
+    // (pinned here: the values are only used by the gathering waves' code further down, and the compiler would
+    // otherwise move their computation there, behind the wait for the lengths)
+    asm volatile("" : "+v"(k_goff), "+v"(v_goff));
+#pragma unroll
+    for (int i = 0; i < KI; ++i) asm volatile("" : "+v"(k_toff[i]));
+    if constexpr (PAD) {
+#pragma unroll
+        for (int i = 0; i < KI; ++i) asm volatile("" : "+v"(pk1[i]), "+v"(pk2[i]));
+#pragma unroll
+        for (int i = 0; i < VI_CTX; ++i) asm volatile("" : "+v"(pv[i]));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    const int q_len = (int)(qe - qs);
+    const int ctx_len = (int)(seq - q_len);
     if (q_len <= 0 || ctx_len < 0) return;
     if (p.skip_decode && q_len == 1) return;                     // old_ops:109-110
     const int n_chunks = (q_len + UNIT - 1) / UNIT;
     const int n_units = n_chunks * group;
     if (mt * NC >= n_units) return;                              // block_mask, old_ops:322-328
-    const bool lazy_b = p.is_lazy ? p.is_lazy[b] != 0 : true;
-    const int pos_mode = p.pos_mode;
+    const bool lazy_b = lazy_raw != 0;
     const bool vanilla = pos_mode == LAZYATTN_POS_BLOCK_UNIFORM && !lazy_b;   // ops:398
     const bool use_qmask = !vanilla && p.q_mask != nullptr;
     const int n_pages = (ctx_len + BS - 1) / BS;
@@ -344,10 +424,6 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     const int64_t qo_s1 = use_qo ? p.qo_stride[1] : p.bt_stride[1];
     const int64_t qm_s1 = use_qmask ? p.qm_stride[1] : p.bt_stride[1];
     const int qo_and = use_qo ? -1 : 0, qm_and = use_qmask ? -1 : 0;
-    // A cache page of 32 slots is handled as two parts of 16: "page" j below is the j-th run of 16 context
-    // slots, part j & 1 of cache page j >> 1.  Its valid slots follow from the page's pad count.
-    const int pshift = p.block_size == 2 * BS ? 1 : 0, part_mask = pshift;
-    const int cache_bs = BS << pshift;
     auto load_page = [&](int j) -> PageMeta {
         PageMeta m;
         int jc = j < n_pages ? j : n_pages - 1;
@@ -371,80 +447,25 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
 
     if (gatherer) {
         // ====================================================================== gather
-        const int gw = wave - NC;                                // this wave's page of every tile
-        // The block-table entries of the first three tiles are requested before anything else is set up: the
-        // scalar loads are a memory round trip, the per-lane set-up below a few hundred instructions from a
-        // cold instruction cache -- the two run side by side.
+        // The block-table entries of the first three tiles are requested before anything else: the scalar
+        // loads are a memory round trip.
         const PageMeta pm0 = load_page(tile_begin * PAGES + gw);
         const PageMeta pm1 = load_page((tile_begin + 1) * PAGES + gw);
         PageMeta pm_pend = load_page((tile_begin + 2) * PAGES + gw);
-        const int nat_step = (vanilla || pos_mode == LAZYATTN_POS_BLOCK_UNIFORM) ? 0 : BS;
         const bool rot_new = p.rotate_new_k && !vanilla;
-        const float k_scale = FP8 ? *p.k_scale : 1.f;
-        const float v_scale = FP8 ? *p.v_scale : 1.f;
         const float k_unscale = FOLD ? 1.f / k_scale : 1.f, v_unscale = FOLD ? 1.f / v_scale : 1.f;
         const uint8_t *kc_base = (const uint8_t *)p.k_cache + (int64_t)g * p.kc_stride[1] * (FP8 ? 1 : 2);
         const uint8_t *vc_base = (const uint8_t *)p.v_cache + (int64_t)g * p.vc_stride[1] * (FP8 ? 1 : 2);
         const int64_t kc_page_bytes = p.kc_stride[0] * (FP8 ? 1 : 2);
         const int64_t vc_page_bytes = p.vc_stride[0] * (FP8 ? 1 : 2);
-        const uint8_t *tab_base = (const uint8_t *)p.cos_sin_cache;
-        const uint32_t row_bytes = (uint32_t)p.table_stride * TSZ;
-        // per-token rotation of context pages reads the packed table [2][D/16][rows][8]: the 16
-        // slots of a page are 16 consecutive 16-byte chunks there
-        const bool per_token = !vanilla && pos_mode != LAZYATTN_POS_BLOCK_UNIFORM;
-        const bool packed_tab = p.cos_sin_packed != nullptr && per_token;
         const uint8_t *ctab_base = packed_tab ? (const uint8_t *)p.cos_sin_packed : tab_base;
         const uint32_t pos_bytes = packed_tab ? 8 * TSZ : row_bytes;       // bytes per unit of position
         const uint32_t sin_delta = packed_tab ? (uint32_t)(HALFr / 8) * (uint32_t)p.packed_rows * 8 * TSZ : HALFr * TSZ;
-        // this wave's part of its cache pages (pages of 32 slots: the tile's pages 0, 1 are the two parts of
-        // one cache page, 2, 3 of the next): first slot, and the position step that goes with it
-        const int slot0 = (gw & part_mask) * BS;
         const int part_pos = nat_step ? slot0 : 0;               // block-uniform: one position for the whole page
-        // K items of a page: 128 = (8 chunks of 8 (d, d+64) pairs) x 16 slots, two per lane
-        uint32_t k_toff[KI];
-        // Cache offsets of a lane's items: item i = item 0 + i * (a wave-uniform stride), so one offset register
-        // serves all of them and the strides go into the scalar page base.
-        // K bf16: [D/8][slots][8] -> item (cp, o) at (cp*slots + o)*16 bytes, cp = lane/16 + 4 i
-        //   fp8 : [D/16][slots][16] -> 8 bytes at chunk cp/2, half cp&1
-        // V bf16: row d = lane/2 + 32 i of `slots` slots, 8 slots (16 bytes) per item; fp8: row d = lane + 64 i, 16 slots
-        const uint32_t k_goff = FP8 ? (uint32_t)(((lane >> 5) * cache_bs + slot0 + (lane & 15)) * 16 + ((lane >> 4) & 1) * 8)
-                                    : (uint32_t)(((lane >> 4) * cache_bs + slot0 + (lane & 15)) * 16);
         const uint32_t k_item = (uint32_t)((FP8 ? 2 : 4) * cache_bs * 16);
-        const uint32_t v_goff = FP8 ? (uint32_t)(lane * cache_bs + slot0)
-                                    : (uint32_t)((lane >> 1) * cache_bs * 2 + slot0 * 2 + (lane & 1) * 16);
         const uint32_t v_item = (uint32_t)(64 * cache_bs);
         // bytes from the chunk of d to the chunk of d + HD/2 in the cache page
         const uint32_t pair = (uint32_t)(FP8 ? G::PAIR8 : G::PAIR) << pshift;
-#pragma unroll
-        for (int i = 0; i < KI; ++i) {
-            const int idx = lane + i * 64;
-            const int o = idx & 15, cp = PAD && (idx >> 4) >= CPr ? 0 : idx >> 4;   // (a padded chunk reads chunk 0 and is zeroed)
-            // block-uniform rotation and un-rotated requests use one table row for the whole page
-            k_toff[i] = packed_tab ? ((uint32_t)cp * (uint32_t)p.packed_rows + (uint32_t)o) * 8 * TSZ
-                                   : (per_token ? (uint32_t)o * row_bytes : 0u) + (uint32_t)cp * 8 * TSZ;
-        }
-        // PAD: per-item cache offsets (the chunk of d + Dr/2 is not a fixed distance away in an fp8 page) and
-        // which of the lane's items exist
-        uint32_t pk1[PAD ? KI : 1], pk2[PAD ? KI : 1], pv[PAD ? VI_CTX : 1];
-        bool pk_ok[PAD ? KI : 1], pv_ok[PAD ? VI_CTX : 1];
-        if constexpr (PAD) {
-#pragma unroll
-            for (int i = 0; i < KI; ++i) {
-                const int idx = lane + i * 64, o = idx & 15;
-                pk_ok[i] = (idx >> 4) < CPr;
-                const int c1 = pk_ok[i] ? idx >> 4 : 0, c2 = CPr + c1;                  // 8-element chunks of d and d + Dr/2
-                pk1[i] = FP8 ? (uint32_t)(((c1 >> 1) * cache_bs + slot0 + o) * 16 + (c1 & 1) * 8) : (uint32_t)((c1 * cache_bs + slot0 + o) * 16);
-                pk2[i] = FP8 ? (uint32_t)(((c2 >> 1) * cache_bs + slot0 + o) * 16 + (c2 & 1) * 8) : (uint32_t)((c2 * cache_bs + slot0 + o) * 16);
-            }
-#pragma unroll
-            for (int i = 0; i < VI_CTX; ++i) {
-                const int idx = lane + i * 64;
-                const int d = FP8 ? idx : idx >> 1;
-                pv_ok[i] = d < Dr;
-                const int dc = pv_ok[i] ? d : 0;
-                pv[i] = FP8 ? (uint32_t)(dc * cache_bs + slot0) : (uint32_t)(dc * cache_bs * 2 + slot0 * 2 + (idx & 1) * 16);
-            }
-        }
         KRegs<TT> kr[KI];
         uint4 vr[VI];
 
@@ -688,10 +709,31 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         int nxt_kind = TILE_FULL, nxt_lim = BS;
         if (tile_begin < tile_end) {
             const int k0 = issue_loads(tile_begin, pm0);
-            store_tile(0, k0, pm0.lim);
-            if (tile_begin + 1 < tile_end) {
-                nxt_kind = issue_loads(tile_begin + 1, pm1);
-                nxt_lim = pm1.lim;
+            if (k0 == TILE_FULL && tile_begin + 1 < n_ctx_tiles && tile_begin + 1 < tile_end && pm1.lim == BS) {
+                // two full context tiles: as in the steady state below, each item of the second tile is requested
+                // into the registers its counterpart of the first has just left, so the requests pass through the
+                // CU's memory pipeline while the first tile is rotated instead of in one burst before the barrier
+                const PageBase pb = page_base(tile_begin + 1, pm1);
+                uint8_t *kt = lds, *vt = lds + 2 * K_TILE;
+#pragma unroll
+                for (int i = 0; i < KI; ++i) {
+                    store_k_item(i, kt, TILE_FULL);
+                    load_k_item(i, pb);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int i = 0; i < VI_CTX; ++i) {
+                    store_v_item(i, vt, TILE_FULL, BS);
+                    load_v_item(i, pb);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if (lane == 0) page_lims[gw] = BS;
+            } else {
+                store_tile(0, k0, pm0.lim);
+                if (tile_begin + 1 < tile_end) {
+                    nxt_kind = issue_loads(tile_begin + 1, pm1);
+                    nxt_lim = pm1.lim;
+                }
             }
         }
         __syncthreads();
@@ -755,7 +797,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     // delivers the scores in log2 units and no per-score multiply is left in the tile loop (the
     // reference scales the fp32 scores, old_ops:287; the extra rounding of Q is one more relative
     // 2^-9 per element, like the one the rotated K already carries).
-    const float cs2 = p.sm_scale * 1.4426950408889634f * (FOLD ? *p.k_scale : 1.f);
+    const float cs2 = p.sm_scale * 1.4426950408889634f * (FOLD ? k_scale : 1.f);
     uint8_t *qlds = lds + KV_BYTES + (QREG ? 0 : wave * G::Q_WAVE) + lane * 16;
     uint4 qreg[QREG ? KS : 1];
     {
@@ -1020,7 +1062,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     // 5 K keys and 5 % longer at 65 K, where every finishing workgroup's cache invalidation hits the others.)
     l_run += partner32(l_run, gh != 0);
     if (!row_ok) return;
-    const float out_scale = FOLD ? *p.v_scale : 1.f;
+    const float out_scale = FOLD ? v_scale : 1.f;
     const float inv = l_run > 0.f ? out_scale / l_run : 0.f;
     if (nsplit == 1) {
         T *op = (T *)p.o + (qs + row) * p.o_stride[0] + (int64_t)h * p.o_stride[1];
