@@ -12,56 +12,7 @@ extern template int launch_mfma_family<f16_t, 0>(const lazyattn_prefill_params &
 extern template int launch_mfma_family<f16_t, 1>(const lazyattn_prefill_params &, int, int, int, int, hipStream_t);
 extern template int launch_mfma_family<f16_t, 2>(const lazyattn_prefill_params &, int, int, int, int, hipStream_t);
 
-// One 16-byte piece (8 elements from column d) of an output row, merged from the row's nsplit partial rows
-// (row0 = token x q-heads + head; consecutive splits are split_rows rows apart).  Log-sum-exps and partial rows of
-// NB splits are requested together and before the first use: one memory round trip per batch; batches are chained
-// like the tiles of the main kernel, by a running maximum.
-template <typename T, int HD, int NB>
-__device__ __forceinline__ uint4 merge_piece(const _Float16 *wo, const float2 *wl, int64_t row0, int64_t split_rows, int nsplit, int d) {
-    using E = Elem<T>;
-    float mx = -INFINITY, wsum = 0.f;
-    float o[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) o[i] = 0.f;
-    for (int s0 = 0; s0 < nsplit; s0 += NB) {
-        float2 e[NB];                                        // (log2-sum-exp, scale of the row's halves)
-        uint4 v[NB];
-#pragma unroll
-        for (int j = 0; j < NB; ++j) {
-            const int64_t ri = (int64_t)(s0 + j < nsplit ? s0 + j : nsplit - 1) * split_rows + row0;
-            e[j] = wl[ri];
-            v[j] = *reinterpret_cast<const uint4 *>(wo + ri * HD + d);
-        }
-        float bm = e[0].x;
-#pragma unroll
-        for (int j = 1; j < NB; ++j) bm = fmaxf(bm, e[j].x);
-        const float m_new = fmaxf(mx, bm);
-        if (m_new == -INFINITY) continue;                    // nothing visible so far
-        const float keep = __builtin_amdgcn_exp2f(mx - m_new);   // mx = -inf -> 0
-#pragma unroll
-        for (int i = 0; i < 8; ++i) o[i] *= keep;
-        wsum *= keep;
-        mx = m_new;
-#pragma unroll
-        for (int j = 0; j < NB; ++j) {
-            const float w = s0 + j < nsplit ? __builtin_amdgcn_exp2f(e[j].x - mx) : 0.f;
-            const float ws = w * e[j].y;
-            const uint32_t u[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const f16x2_t hh = *reinterpret_cast<const f16x2_t *>(&u[i]);
-                o[2 * i] = fmaf(ws, (float)hh[0], o[2 * i]);
-                o[2 * i + 1] = fmaf(ws, (float)hh[1], o[2 * i + 1]);
-            }
-            wsum += w;
-        }
-    }
-    const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
-    return make_uint4(E::pack(o[0] * inv, o[1] * inv), E::pack(o[2] * inv, o[3] * inv),
-                      E::pack(o[4] * inv, o[5] * inv), E::pack(o[6] * inv, o[7] * inv));
-}
-
-// ---- merge split-KV partials: one 16-lane group (head size 128) per (token, q-head) row ----
+// ---- merge split-KV partials ----
 // The few fields the merge needs, not the whole parameter block: a launch with ~450 bytes of kernel
 // arguments costs about a microsecond more than one with 64 on this part.
 struct MergeArgs {
@@ -69,53 +20,117 @@ struct MergeArgs {
     void *o;
     int64_t o_stride[2];
     int32_t num_tokens, num_q_heads, index_bits, skip_decode;
-    int32_t batch, token_grid;      // token_grid: rows are numbered over all tokens instead of per request
+    int32_t batch, token_grid;      // token_grid: the 32-token windows are cut over all tokens instead of per request
     int32_t head_dim;               // elements of an output row (below HD when the partial rows are padded)
     int32_t group, unit_cap;        // q-heads per kv-head; 32-row units per (request, kv-head) the main grid covers
 };
-// NB = splits taken per batch of loads: 2, 4 or 8, the smallest that covers nsplit (more only when nsplit > 8)
+// One workgroup = 32 consecutive tokens x one q-head; wave dt merges the columns dt*32 .. +31, lane (gh, l32) the
+// 4-column groups 8*i4 + 4*gh of token l32 -- the mapping of the main kernel's accumulators, so that a load
+// instruction reads one contiguous run of the partial rows as the main kernel wrote them (see its epilogue: the R
+// rows of a request's 32-token chunk are stored [head][piece][gh][row][4 halves]).  Log-sum-exps and row pieces of NB
+// splits (2, 4 or 8, the smallest that covers nsplit; more only when nsplit > 8) are requested together and before
+// the first use: one memory round trip per batch; batches are chained like the tiles of the main kernel, by a
+// running maximum.  The merged tile is turned through LDS (rows padded by 8 bytes: conflict-free both ways) so
+// that the output leaves as whole rows, 32 bytes per thread.  The windows are cut per request (grid y = request),
+// or over all tokens of the call when that grid is at most half as large (one long request among one-token
+// requests): then the 32 tokens of a workgroup need not belong to one request, and every lane finds its own by a
+// binary search of the offsets.
 template <typename T, int HD, int NB>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(HD * 2)
 prefill_combine_kernel(const MergeArgs p, const int nsplit) {
-    constexpr int D = HD, LPR = HD / 8;                       // lanes per row (8 elements = one 16-byte load each)
-    const int64_t r = (int64_t)blockIdx.x * (256 / LPR) + threadIdx.x / LPR;
-    int64_t tok;
-    int b;
+    using E = Elem<T>;
+    constexpr int D = HD, ROW = HD * 2 + 8;                   // bytes of a tile row in LDS
+    __shared__ __attribute__((aligned(16))) uint8_t tile[UNIT * ROW];
+    __shared__ int row_ok[UNIT];
+    const int lane = threadIdx.x & 63, dt = threadIdx.x >> 6, l32 = lane & 31, gh = lane >> 5;
+    const int h = (int)(blockIdx.x % (unsigned)p.num_q_heads);
+    const int64_t win = (int64_t)(blockIdx.x / (unsigned)p.num_q_heads) * UNIT;   // first token of the window
+    int b = blockIdx.y;
+    bool valid = true;
     if (p.token_grid) {
-        // Rows over all tokens of the call: no workgroup is launched for rows a request does not have (a grid
-        // of batch x longest request is mostly empty when one long request sits among one-token requests).
-        // The row's request is found by a binary search of the offsets.
-        tok = r / p.num_q_heads;
-        if (tok >= load_index(p.b_start_loc, p.batch, p.index_bits)) return;
-        int lo = 0, hi = p.batch;                             // offsets[lo] <= tok < offsets[hi]
+        valid = win + l32 < load_index(p.b_start_loc, p.batch, p.index_bits);
+        int lo = 0, hi = p.batch;                             // offsets[lo] <= token < offsets[hi]
         while (hi - lo > 1) {
             const int mid = (lo + hi) >> 1;
-            if (load_index(p.b_start_loc, mid, p.index_bits) <= tok) lo = mid; else hi = mid;
+            if (load_index(p.b_start_loc, mid, p.index_bits) <= win + l32) lo = mid; else hi = mid;
         }
         b = lo;
-    } else {
-        b = blockIdx.y;
-        tok = load_index(p.b_start_loc, b, p.index_bits) + r / p.num_q_heads;
     }
     // Exactly the rows the main kernel wrote partials for: anything else would merge whatever an earlier call
     // left in the workspace.
-    {
-        const int64_t qs = load_index(p.b_start_loc, b, p.index_bits);
-        const int64_t q_len = load_index(p.b_start_loc, b + 1, p.index_bits) - qs;
-        const int64_t row = tok - qs;
-        if (q_len <= 0 || (p.skip_decode && q_len == 1)) return;
-        if (row >= q_len) return;
-        if ((row / UNIT) * p.group + (r % p.num_q_heads) % p.group >= p.unit_cap) return;   // past the grid sized by max_q_len
-        if (load_index(p.b_seq_len, b, p.index_bits) - q_len < 0) return;
+    const int64_t qs = load_index(p.b_start_loc, b, p.index_bits);
+    const int64_t q_len = load_index(p.b_start_loc, b + 1, p.index_bits) - qs;
+    const int64_t tok0 = p.token_grid ? win : qs + win;       // token of the window's row 0
+    const int64_t row = tok0 + l32 - qs;
+    valid = valid && q_len > 0 && !(p.skip_decode && q_len == 1) && row < q_len &&
+            (row / UNIT) * p.group + h % p.group < p.unit_cap &&                 // (past the grid sized by max_q_len)
+            load_index(p.b_seq_len, b, p.index_bits) - q_len >= 0;
+    float o[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) o[i] = 0.f;
+    float wsum = 0.f;
+    if (valid) {
+        const int64_t t0 = (row / UNIT) * UNIT;
+        const int R = (int)(q_len - t0 < UNIT ? q_len - t0 : UNIT), lr = (int)(row - t0);
+        const int64_t NTOK = p.num_tokens, split_rows = NTOK * p.num_q_heads;
+        const _Float16 *wo = (const _Float16 *)p.workspace;
+        const float2 *wl = reinterpret_cast<const float2 *>(wo + (int64_t)nsplit * split_rows * D);
+        const int64_t blk = (qs + t0) * p.num_q_heads + (int64_t)h * R;                  // in rows, split 0
+        const _Float16 *wb = wo + blk * D + (dt * 4 * 2 * R + gh * R + lr) * 4;
+        const float2 *we = wl + blk + lr;
+        float mx = -INFINITY;
+        for (int s0 = 0; s0 < nsplit; s0 += NB) {
+            float2 e[NB];                                        // (log2-sum-exp, scale of the row's halves)
+            uint2 v[NB][4];
+#pragma unroll
+            for (int j = 0; j < NB; ++j) {
+                const int64_t so = (int64_t)(s0 + j < nsplit ? s0 + j : nsplit - 1) * split_rows;
+                e[j] = we[so];
+#pragma unroll
+                for (int i4 = 0; i4 < 4; ++i4) v[j][i4] = *reinterpret_cast<const uint2 *>(wb + so * D + i4 * (2 * R * 4));
+            }
+            float bm = e[0].x;
+#pragma unroll
+            for (int j = 1; j < NB; ++j) bm = fmaxf(bm, e[j].x);
+            const float m_new = fmaxf(mx, bm);
+            if (m_new == -INFINITY) continue;                    // nothing visible so far
+            const float keep = __builtin_amdgcn_exp2f(mx - m_new);   // mx = -inf -> 0
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o[i] *= keep;
+            wsum *= keep;
+            mx = m_new;
+#pragma unroll
+            for (int j = 0; j < NB; ++j) {
+                const float w = s0 + j < nsplit ? __builtin_amdgcn_exp2f(e[j].x - mx) : 0.f;
+                const float ws = w * e[j].y;
+#pragma unroll
+                for (int i4 = 0; i4 < 4; ++i4) {
+                    const f16x2_t a = *reinterpret_cast<const f16x2_t *>(&v[j][i4].x), c = *reinterpret_cast<const f16x2_t *>(&v[j][i4].y);
+                    o[4 * i4] = fmaf(ws, (float)a[0], o[4 * i4]);
+                    o[4 * i4 + 1] = fmaf(ws, (float)a[1], o[4 * i4 + 1]);
+                    o[4 * i4 + 2] = fmaf(ws, (float)c[0], o[4 * i4 + 2]);
+                    o[4 * i4 + 3] = fmaf(ws, (float)c[1], o[4 * i4 + 3]);
+                }
+                wsum += w;
+            }
+        }
     }
-    const int h = (int)(r % p.num_q_heads);
-    const int d = (threadIdx.x % LPR) * 8;
-    if (d >= p.head_dim) return;
-    const int64_t NTOK = p.num_tokens;
-    const _Float16 *wo = (const _Float16 *)p.workspace;
-    const float2 *wl = reinterpret_cast<const float2 *>(wo + (int64_t)nsplit * NTOK * p.num_q_heads * D);
-    const uint4 v = merge_piece<T, HD, NB>(wo, wl, tok * p.num_q_heads + h, NTOK * p.num_q_heads, nsplit, d);
-    *reinterpret_cast<uint4 *>((T *)p.o + tok * p.o_stride[0] + (int64_t)h * p.o_stride[1] + d) = v;
+    const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4)
+        *reinterpret_cast<uint2 *>(tile + l32 * ROW + (dt * 32 + 8 * i4 + 4 * gh) * 2) =
+            make_uint2(E::pack(o[4 * i4] * inv, o[4 * i4 + 1] * inv), E::pack(o[4 * i4 + 2] * inv, o[4 * i4 + 3] * inv));
+    if (dt == 0 && gh == 0) row_ok[l32] = valid;
+    __syncthreads();
+    // whole rows out: 32 bytes per thread, HD/16 threads per row
+    const int r = threadIdx.x / (HD / 16), seg = threadIdx.x % (HD / 16);
+    if (row_ok[r] && seg * 16 < p.head_dim) {                 // (beyond head_dim: padding columns of the partial rows)
+        const uint4 a = *reinterpret_cast<const uint4 *>(tile + r * ROW + seg * 32);
+        const uint4 c = *reinterpret_cast<const uint4 *>(tile + r * ROW + seg * 32 + 16);
+        T *op = (T *)p.o + (tok0 + r) * p.o_stride[0] + (int64_t)h * p.o_stride[1] + seg * 16;
+        *reinterpret_cast<uint4 *>(op) = a;
+        *reinterpret_cast<uint4 *>(op + 8) = c;
+    }
 }
 
 // ------------------------------------------------------------------ host side
@@ -230,19 +245,19 @@ int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
         if (rc != LAZYATTN_OK) return rc;
     }
     if (nsplit > 1 && (phases & LAZYATTN_PHASE_COMBINE)) {
-        // rows per request x requests, or rows over all tokens when that is at most half as many
+        // windows per request x requests, or windows over all tokens when that is at most half as many
         const int token_grid = p.batch > 1 && 2 * (int64_t)p.num_tokens <= (int64_t)p.batch * p.max_q_len;
-        const int64_t rows = (int64_t)(token_grid ? p.num_tokens : p.max_q_len) * p.num_q_heads;
         const MergeArgs m{p.workspace, p.b_start_loc, p.b_seq_len, p.o, {p.o_stride[0], p.o_stride[1]}, p.num_tokens, p.num_q_heads,
                           p.index_bits, p.skip_decode, p.batch, token_grid, p.head_dim, p.num_q_heads / p.num_kv_heads,
                           mt_total > 0 ? 0x7fffffff : n_mt * nw};
-        const int rows_wg = 256 / (tile_dim(p) / 8);
-        const dim3 grid((unsigned)((rows + rows_wg - 1) / rows_wg), token_grid ? 1 : p.batch);
+        // 32 tokens x one q-head per workgroup
+        const int64_t windows = ((int64_t)(token_grid ? p.num_tokens : p.max_q_len) + UNIT - 1) / UNIT;
+        const dim3 grid((unsigned)(windows * p.num_q_heads), token_grid ? 1 : p.batch);
         const bool f16 = p.dtype == LAZYATTN_F16;
-#define LAZYATTN_COMBINE(HD, NB)                                                                              \
-    {                                                                                                         \
-        if (f16) hipLaunchKernelGGL((prefill_combine_kernel<f16_t, HD, NB>), grid, dim3(256), 0, stream, m, nsplit); \
-        else hipLaunchKernelGGL((prefill_combine_kernel<bf16_t, HD, NB>), grid, dim3(256), 0, stream, m, nsplit);    \
+#define LAZYATTN_COMBINE(HD, NB)                                                                                  \
+    {                                                                                                             \
+        if (f16) hipLaunchKernelGGL((prefill_combine_kernel<f16_t, HD, NB>), grid, dim3(HD * 2), 0, stream, m, nsplit); \
+        else hipLaunchKernelGGL((prefill_combine_kernel<bf16_t, HD, NB>), grid, dim3(HD * 2), 0, stream, m, nsplit);    \
     }
         if (p.head_dim == 64) {
             if (nsplit <= 2) LAZYATTN_COMBINE(64, 2) else if (nsplit <= 4) LAZYATTN_COMBINE(64, 4) else LAZYATTN_COMBINE(64, 8)

@@ -1091,23 +1091,30 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         eb = eb > 252u ? 252u : eb;
         const float down = __uint_as_float((253u - eb) << 23) * inv;   // 2^-(eb-126) / l
         const float up = __uint_as_float((eb + 1u) << 23);            // 2^(eb-126)
+        // Where the rows go: the R rows of a 32-token chunk (R < 32 only at a request's end), all q-heads, fill
+        // the same stretch of the workspace as in [token][head][D] order, but laid out [head][piece][gh][row][4]:
+        // one store instruction of this wave then writes one contiguous run (512 bytes for a full chunk) instead of
+        // 32 runs of 16 bytes a row apart -- the partial rows leave in a quarter of the time (measured with the
+        // bytes kept and only the addresses changed: 1.8 of the 3.2 us the stores cost at 5 K keys).  The merge
+        // kernel reads with the same lane mapping.  (piece = the 8 columns dt*32 + 8*i4 .. +7, gh its half)
         const int64_t NTOK = p.num_tokens;
         _Float16 *wo = (_Float16 *)p.workspace;
         float2 *wl = reinterpret_cast<float2 *>(wo + (int64_t)nsplit * NTOK * p.num_q_heads * D);
-        const int64_t r_idx = ((int64_t)split * NTOK + (qs + row)) * p.num_q_heads + h;
+        const int R = q_len - t0 < UNIT ? q_len - t0 : UNIT;
+        const int64_t blk = ((int64_t)split * NTOK + (qs + t0)) * p.num_q_heads + (int64_t)h * R;   // in rows
+        _Float16 *wb = wo + blk * D + (gh * R + l32) * 4;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) {
-                const int d = dt * 32 + 8 * i4 + 4 * gh;
                 const f32x2_t lo = {acc[dt][4 * i4] * down, acc[dt][4 * i4 + 1] * down};
                 const f32x2_t hi = {acc[dt][4 * i4 + 2] * down, acc[dt][4 * i4 + 3] * down};
                 const f16x2_t hl = __builtin_convertvector(lo, f16x2_t), hh = __builtin_convertvector(hi, f16x2_t);   // RNE
-                *reinterpret_cast<uint2 *>(wo + r_idx * D + d) =
+                *reinterpret_cast<uint2 *>(wb + (dt * 4 + i4) * (2 * R * 4)) =
                     make_uint2(*reinterpret_cast<const uint32_t *>(&hl), *reinterpret_cast<const uint32_t *>(&hh));
             }
         if (gh == 0)
-            wl[r_idx] = make_float2(l_run > 0.f ? m_ref + __builtin_amdgcn_logf(l_run) : -INFINITY, up);
+            wl[blk + l32] = make_float2(l_run > 0.f ? m_ref + __builtin_amdgcn_logf(l_run) : -INFINITY, up);
     }
 }
 
