@@ -51,4 +51,13 @@ __device__ __forceinline__ int64_t load_index_nonneg(const void *p, int64_t i, i
     return bits == 64 ? ((const int64_t *)p)[i] : (int64_t)(uint32_t)((const int32_t *)p)[i];
 }
 
+// The low 32 bits of a wave-uniform entry below 2^31 (token offsets, lengths) as one scalar load, with no branch
+// on the width: several of these in a row are in flight together, where load_index() compiles to a vector load
+// and a wait per call.
+__device__ __forceinline__ int64_t load_index_uniform(const void *p, int64_t i, int bits) {
+    typedef const uint32_t __attribute__((address_space(4))) *sptr_u32;
+    const char *a = (const char *)p + i * (int64_t)(bits >> 3);
+    return (int64_t)*(sptr_u32)(const void *)a;
+}
+
 }  // namespace lazyattn

@@ -58,13 +58,24 @@ prefill_combine_kernel(const MergeArgs p, const int nsplit) {
     }
     // Exactly the rows the main kernel wrote partials for: anything else would merge whatever an earlier call
     // left in the workspace.
-    const int64_t qs = load_index(p.b_start_loc, b, p.index_bits);
-    const int64_t q_len = load_index(p.b_start_loc, b + 1, p.index_bits) - qs;
+    // (per-request windows: the request is the same for the whole workgroup and its three entries come as scalar
+    // loads in flight together -- this kernel is a chain of memory round trips and little else)
+    int64_t qs, qe, seq;
+    if (p.token_grid) {
+        qs = load_index(p.b_start_loc, b, p.index_bits);
+        qe = load_index(p.b_start_loc, b + 1, p.index_bits);
+        seq = load_index(p.b_seq_len, b, p.index_bits);
+    } else {
+        qs = load_index_uniform(p.b_start_loc, b, p.index_bits);
+        qe = load_index_uniform(p.b_start_loc, b + 1, p.index_bits);
+        seq = load_index_uniform(p.b_seq_len, b, p.index_bits);
+    }
+    const int64_t q_len = qe - qs;
     const int64_t tok0 = p.token_grid ? win : qs + win;       // token of the window's row 0
     const int64_t row = tok0 + l32 - qs;
     valid = valid && q_len > 0 && !(p.skip_decode && q_len == 1) && row < q_len &&
             (row / UNIT) * p.group + h % p.group < p.unit_cap &&                 // (past the grid sized by max_q_len)
-            load_index(p.b_seq_len, b, p.index_bits) - q_len >= 0;
+            seq - q_len >= 0;
     float o[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) o[i] = 0.f;
