@@ -310,6 +310,8 @@ def main():
     ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5])
     ap.add_argument("--num-splits", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--min-warmup", type=int, default=300,
+                    help="floor on the untimed warm-up calls, whatever --warmup says (profiler runs lower it)")
     ap.add_argument("--no-host-timing", action="store_true",
                     help="skip the 1 100 entry-point calls that measure host_us_per_call (profiler runs)")
     ap.add_argument("--path", choices=["prefill", "decode", "rope_write", "reposition"], default="prefill",
@@ -348,11 +350,11 @@ def main():
     plan, o = make_plan(g, a.num_splits, _ffi.PHASE_ALL)
     main_only, _ = make_plan(g, a.num_splits, _ffi.PHASE_MAIN)
 
-    # The first dozens of launches of a process run 10-40 % slow (clocks, caches, code upload): whatever the
-    # command line says, at least MIN_WARMUP untimed calls come first, and the dominant kernel is timed as the
+    # The first hundreds of launches of a process run up to 10-40 % slow (clocks, caches, code upload): whatever
+    # --warmup says, at least --min-warmup untimed calls come first, and the dominant kernel is timed as the
     # median of 7 runs of at least 50 launches (the discipline of the reference's own kernel benchmark,
     # benchmarks/bench_rope_cos_sin.py:451-461,514-522).  The K timed steps of the whole call stay exactly K.
-    MIN_WARMUP, MIN_MAIN_LAUNCHES = 20, 50
+    MIN_WARMUP, MIN_MAIN_LAUNCHES = a.min_warmup, 50
     for _ in range(max(a.warmup, MIN_WARMUP)):
         plan.run()
     torch.cuda.synchronize()
