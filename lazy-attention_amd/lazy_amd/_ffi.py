@@ -132,7 +132,8 @@ _growth_hooks: list = []
 
 
 def on_workspace_growth(fn) -> None:
-    """``fn()`` runs whenever a workspace is replaced by a larger one (its old address dies)."""
+    """``fn()`` runs whenever something a remembered call may point at goes away: a workspace replaced by a larger
+    one, the re-laid-out tables dropped by ``invalidate_packed_tables()``."""
     _growth_hooks.append(fn)
 
 
@@ -162,9 +163,12 @@ def table_version(table: torch.Tensor) -> Optional[int]:
 
 
 def invalidate_packed_tables() -> None:
-    """Drop every re-laid-out copy.  Needed only after writing in place to a table that was created under
-    ``torch.inference_mode()``: such an edit cannot be seen from here (other tables are re-packed on their own)."""
+    """Drop every re-laid-out copy, and every remembered call that points at one.  Needed only after writing in
+    place to a table that was created under ``torch.inference_mode()``: such an edit cannot be seen from here (other
+    tables are re-packed on their own)."""
     _packed_tables.clear()
+    for fn in _growth_hooks:
+        fn()
 
 
 def packed_cos_sin(table: torch.Tensor) -> Optional[torch.Tensor]:

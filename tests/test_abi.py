@@ -127,6 +127,41 @@ def test_table_version_of_inference_tensors():
     assert _ffi.table_version(u) == v0 + 1
 
 
+def test_remembered_calls_keying_and_invalidation():
+    """Host logic of the entry points' call memory: the key tells apart views of one buffer that differ in shape,
+    strides or dtype; a remembered call is dropped when the cos/sin table it was made for has been edited in place,
+    and all of them when the re-laid-out tables are invalidated by hand."""
+    from lazy_amd.attention import _launch
+    base = torch.zeros(8, 16)
+    k0 = _launch.call_key("t", (base, None), (1, 2.0, None))
+    assert k0 == _launch.call_key("t", (base, None), (1, 2.0, None))
+    assert k0 != _launch.call_key("t", (base.t(), None), (1, 2.0, None))            # same address, other strides
+    assert k0 != _launch.call_key("t", (base[:4], None), (1, 2.0, None))            # same address, other shape
+    assert k0 != _launch.call_key("t", (base.view(torch.int32), None), (1, 2.0, None))
+    assert k0 != _launch.call_key("t", (base, None), (1, 2.5, None))
+    assert k0 != _launch.call_key("u", (base, None), (1, 2.0, None))
+
+    class Plan:                                       # stands in for a validated call
+        repeatable = True
+        def detached(self): return self
+    _launch.forget_calls()
+    table = torch.ones(4, 16)
+    _launch.remember(k0, (Plan(),), table)
+    assert _launch.recall(k0, table) is not None
+    table.mul_(2.0)                                   # in-place edit: the plans point at a copy of the old contents
+    assert _launch.recall(k0, table) is None and len(_launch._calls) == 0
+    unrepeatable = Plan(); unrepeatable.repeatable = False
+    _launch.remember(k0, (Plan(), unrepeatable), table)
+    assert len(_launch._calls) == 0                   # a call with a converted operand is validated every time
+    _launch.remember(k0, (Plan(),), table)
+    _ffi.invalidate_packed_tables()
+    assert len(_launch._calls) == 0
+    for i in range(_launch._CALLS_MAX + 5):           # bounded: the oldest entries leave
+        _launch.remember(("k", i), (Plan(),), None)
+    assert len(_launch._calls) == _launch._CALLS_MAX and _launch.recall(("k", 0), None) is None
+    _launch.forget_calls()
+
+
 def test_fast_division_is_exact(tmp_path):
     """csrc/fastdiv.hpp (the kernel prologue's divisions by launch-time constants): the multiply-high form equals
     n / d for divisors from 1 to 2^32 - 1 and numerators over the whole 32-bit range, edges included."""
