@@ -154,34 +154,43 @@ template <typename TT> struct KRegs {
 
 }  // namespace
 
-// Workgroup = 8 waves: waves 0-3 compute (32 query rows each), waves 4-7 gather.  The
-// hardware places wave w on SIMD w % 4, so every SIMD hosts one computing and one
-// gathering wave: the gather's address arithmetic, fp32 rotation and LDS writes run in
-// the shadow of the other wave's MFMAs, and neither role ever waits for the other's
+// Workgroup = NC computing waves (32 query rows each) followed by the gathering waves.  The
+// hardware places wave w on SIMD w % 4, so every SIMD hosts computing and gathering
+// waves: the gather's address arithmetic, fp32 rotation and LDS writes run in
+// the shadow of the other waves' MFMAs, and neither role ever waits for the other's
 // memory latency -- they only meet at one barrier per tile.
-// NC = computing waves = 32-row units per workgroup: 8 (12 waves, three per SIMD) for long
-// key ranges, 4 (8 waves) when the call is small and more, lighter workgroups fill the chip
-// with fewer key-axis splits.
-// With four computing waves two waves share a SIMD's registers and the Q^T fragments stay in registers; with eight
-// (three waves per SIMD) they live in LDS and are re-read every tile.
-constexpr bool q_in_registers(int nc) { return nc == 4; }
+// NC = computing waves = 32-row units per workgroup: 8 for long key ranges, 4 when the call is small and more,
+// lighter workgroups fill the chip with fewer key-axis splits.  Either way twelve waves (three per SIMD, 168
+// registers each) at head size 128: 8 + 4 or 4 + 8; the Q^T fragments then live in LDS and are re-read every tile.
+// At head size 64 the four-unit shape has eight waves, two per SIMD, and keeps Q^T in registers.
+// Gathering waves: four, one per 16-key page of a tile -- or eight, two per page with half of its items each, for
+// the four-unit shape at head size 128: there the gathering wave's serial instruction stream is the longest of a
+// SIMD's (one computing + one gathering wave), and two half-length streams beside it are shorter than one.  Twelve
+// waves leave 168 registers each, so that shape reads Q^T from LDS as well.
+constexpr int gather_waves(int nc, int hd) { return nc == 4 && hd == 128 ? 8 : 4; }
+constexpr bool q_in_registers(int nc, int hd) { return nc == 4 && gather_waves(nc, hd) == 4; }
 template <int HD> constexpr int lds_bytes(int nc) {      // K and V tiles + Q^T fragments (if in LDS) + page limits
-    return Geo<HD>::KV_BYTES + (q_in_registers(nc) ? 0 : nc * Geo<HD>::Q_WAVE) + 2 * PAGES * 4;
+    return Geo<HD>::KV_BYTES + (q_in_registers(nc, HD) ? 0 : nc * Geo<HD>::Q_WAVE) + 2 * PAGES * 4;
 }
 
 // WIN: built with the sliding-window code (calls without a window run the instantiation without it)
 // PAD: the head size is a multiple of 16 below HD = 128: Q, K and V sit zero-padded in the 128-wide tiles, the two
 // halves of the real head at (0 .., 64 ..) so that the rotation pairs stay (d, 64 + d)
 template <int NC, int HD, int FP8, bool WIN, bool PAD, typename T, typename TT>
-__global__ void __launch_bounds__((NC + 4) * 64)
+__global__ void __launch_bounds__((NC + gather_waves(NC, HD)) * 64)
 prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int n_mt, const int mt_total, const MfmaDivs dv) {
     using G = Geo<HD>;
     constexpr int D = HD, HALF = HD / 2;
     const int Dr = PAD ? p.head_dim : D, HALFr = Dr / 2, CPr = Dr / 16;   // real head size, its half, its chunk pairs
     constexpr int K_PAGE = G::K_PAGE, K_TILE = G::K_TILE, V_G = G::V_G, V_PAGE = G::V_PAGE, V_TILE = G::V_TILE;
     constexpr int KV_BYTES = G::KV_BYTES, KS = G::KS, DT = G::DT;
-    constexpr int KI = G::K_ITEMS, VI = G::V_ITEMS;   // a page has HD K items (HD/16 chunk pairs x 16 slots) and 2 HD V items
-    constexpr int VI_CTX = FP8 ? VI / 2 : VI;        // an fp8 page row of 16 slots is one 16-byte item
+    // a page has HD K items (HD/16 chunk pairs x 16 slots) and 2 HD V items (an fp8 page row of 16 slots is one
+    // 16-byte item): per lane of the NH gathering waves that share the page.  Item i of a wave's registers is item
+    // i * NH + half of the page.
+    constexpr int NG = gather_waves(NC, HD), NH = NG / 4;
+    constexpr int KI = G::K_ITEMS / NH, VI = G::V_ITEMS / NH;
+    constexpr int VI_CTX = FP8 ? VI / 2 : VI;
+    static_assert(KI >= 1 && VI_CTX >= 1, "a page's items do not split over this many gathering waves");
     // fp8 pages under bf16 operands: the cache scales leave the gather.  Rotation and P.V are linear, so
     // k_scale goes into the factor Q is multiplied by anyway and v_scale into the final 1/l; the pages' bytes are
     // converted and used as they are (fp8 -> bf16 is exact), and the few new-token keys and values, which are
@@ -295,7 +304,9 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     // slots, part j & 1 of cache page j >> 1.  Its valid slots follow from the page's pad count.
     const int pshift = p.block_size == 2 * BS ? 1 : 0, part_mask = pshift;
     const int cache_bs = BS << pshift;
-    const int gw = wave - NC;                                    // gathering waves: this wave's page of every tile
+    const int gw = (wave - NC) & 3;                              // gathering waves: this wave's page of every tile
+    const int half = NH == 2 ? (wave - NC) >> 2 : 0;             // ... and which of the page's items
+    auto item = [&](int i) { return i * NH + half; };
     // (an un-rotated request of the block-uniform mode reads row 0 for every page, like the mode's other requests
     // read one row per page: what depends on the request's own flag is decided later)
     const int nat_step = pos_mode == LAZYATTN_POS_BLOCK_UNIFORM ? 0 : BS;
@@ -321,7 +332,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                           : (uint32_t)((lane >> 1) * cache_bs * 2 + slot0 * 2 + (lane & 1) * 16);
 #pragma unroll
     for (int i = 0; i < KI; ++i) {
-        const int idx = lane + i * 64;
+        const int idx = lane + item(i) * 64;
         const int o = idx & 15, cp = PAD && (idx >> 4) >= CPr ? 0 : idx >> 4;   // (a padded chunk reads chunk 0 and is zeroed)
         // block-uniform rotation and un-rotated requests use one table row for the whole page
         k_toff[i] = packed_tab ? ((uint32_t)cp * (uint32_t)p.packed_rows + (uint32_t)o) * 8 * TSZ
@@ -334,7 +345,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     if constexpr (PAD) {
 #pragma unroll
         for (int i = 0; i < KI; ++i) {
-            const int idx = lane + i * 64, o = idx & 15;
+            const int idx = lane + item(i) * 64, o = idx & 15;
             pk_ok[i] = (idx >> 4) < CPr;
             const int c1 = pk_ok[i] ? idx >> 4 : 0, c2 = CPr + c1;                  // 8-element chunks of d and d + Dr/2
             pk1[i] = FP8 ? (uint32_t)(((c1 >> 1) * cache_bs + slot0 + o) * 16 + (c1 & 1) * 8) : (uint32_t)((c1 * cache_bs + slot0 + o) * 16);
@@ -342,7 +353,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         }
 #pragma unroll
         for (int i = 0; i < VI_CTX; ++i) {
-            const int idx = lane + i * 64;
+            const int idx = lane + item(i) * 64;
             const int d = FP8 ? idx : idx >> 1;
             pv_ok[i] = d < Dr;
             const int dc = pv_ok[i] ? d : 0;
@@ -441,7 +452,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     };
     // Valid-slot counts of the four pages of a context tile, one int per page and LDS buffer:
     // written by the gathering waves with the tile, read by the computing waves for the masks.
-    constexpr bool QREG = q_in_registers(NC);
+    constexpr bool QREG = q_in_registers(NC, HD);
     constexpr int Q_BYTES = QREG ? 0 : NC * G::Q_WAVE;
     int *page_lims = reinterpret_cast<int *>(lds + KV_BYTES + Q_BYTES);
 
@@ -497,7 +508,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         };
         auto load_k_item = [&](int i, const PageBase &pb) {
             const uint8_t *kb = pb.kb;
-            kr[i].lds_off = (uint32_t)(gw * K_PAGE + (lane + i * 64) * 16);
+            kr[i].lds_off = (uint32_t)(gw * K_PAGE + (lane + item(i) * 64) * 16);
             if constexpr (PAD) {
                 uint4 k1, k2;
                 if (FP8) {
@@ -512,12 +523,12 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                 kr[i].k1 = pk_ok[i] ? k1 : z;
                 kr[i].k2 = pk_ok[i] ? k2 : z;
             } else if (FP8) {
-                const uint2 a = ldg8(kb + i * k_item, pb.ko), a2 = ldg8(kb + i * k_item + pair, pb.ko);
+                const uint2 a = ldg8(kb + item(i) * k_item, pb.ko), a2 = ldg8(kb + item(i) * k_item + pair, pb.ko);
                 kr[i].k1 = make_uint4(a.x, a.y, 0, 0);
                 kr[i].k2 = make_uint4(a2.x, a2.y, 0, 0);
             } else {
-                kr[i].k1 = ldg16(kb + i * k_item, pb.ko);
-                kr[i].k2 = ldg16(kb + i * k_item + pair, pb.ko);
+                kr[i].k1 = ldg16(kb + item(i) * k_item, pb.ko);
+                kr[i].k2 = ldg16(kb + item(i) * k_item + pair, pb.ko);
             }
             kr[i].c.load(pb.tb, pb.to[i]);
             kr[i].s.load(pb.ts, pb.to[i]);
@@ -527,7 +538,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                 const uint4 t = ldg16(pb.vb, pv[i]);
                 vr[i] = pv_ok[i] ? t : make_uint4(0, 0, 0, 0);
             } else {
-                vr[i] = ldg16(pb.vb + i * v_item, pb.vo);
+                vr[i] = ldg16(pb.vb + item(i) * v_item, pb.vo);
             }
         };
         auto issue_loads_ctx = [&](int tile, const PageMeta &pm) {
@@ -542,7 +553,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             const int m0 = (tile - n_ctx_tiles) * NT + gw * BS;
 #pragma unroll
             for (int i = 0; i < KI; ++i) {
-                const int idx = lane + i * 64;
+                const int idx = lane + item(i) * 64;
                 const int cp = idx & (D / 16 - 1), kl = idx / (D / 16), m = m0 + kl;
                 kr[i].lds_off = (uint32_t)(gw * K_PAGE + cp * 256 + kl * 16);
                 uint4 k1 = make_uint4(0, 0, 0, 0), k2 = k1;
@@ -562,7 +573,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             }
 #pragma unroll
             for (int i = 0; i < VI; ++i) {
-                const int idx = lane + i * 64;
+                const int idx = lane + item(i) * 64;
                 const int dc = idx & (D / 8 - 1), m = m0 + idx / (D / 8);
                 // (the value is chosen before the one store: a store under the branch lets the compiler merge
                 // the iterations' stores behind a pointer phi, and the array then stays in scratch memory)
@@ -620,7 +631,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         };
         // one V item of a context page (16 bytes of one row of d) -> its two 8-byte LDS entries
         auto store_v_item = [&](int i, uint8_t *vtile, int kind, int lim) {
-            const int idx = lane + i * 64;
+            const int idx = lane + item(i) * 64;
             if (FP8) {
                 // 16 fp8 slots of one d: entry g=0 <- slots 0-3 | 8-11, entry g=1 <- slots 4-7 | 12-15
                 const int d = idx;
@@ -676,7 +687,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                 // item = 8 d of one new-token key: scatter 2-byte entries
 #pragma unroll
                 for (int i = 0; i < VI; ++i) {
-                    const int idx = lane + i * 64;
+                    const int idx = lane + item(i) * 64;
                     const int dc = idx & (D / 8 - 1), slot = idx / (D / 8);
                     uint8_t *dst = vtile + gw * V_PAGE + ((slot >> 2) & 1) * V_G + (dc * 8) * 16 + (slot >> 3) * 8 +
                                    (slot & 3) * 2;
@@ -700,7 +711,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         auto store_tile = [&](int buf, int kind, int lim) {
             store_k(lds + buf * K_TILE, kind);
             store_v(lds + 2 * K_TILE + buf * V_TILE, kind, lim);
-            if (lane == 0) page_lims[buf * PAGES + gw] = lim;
+            if (lane == 0 && half == 0) page_lims[buf * PAGES + gw] = lim;
         };
 
         // At the top of iteration `tile` the raw K/V of tile+1 sit in registers (loaded during
@@ -727,7 +738,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                     load_v_item(i, pb);
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                if (lane == 0) page_lims[gw] = BS;
+                if (lane == 0 && half == 0) page_lims[gw] = BS;
             } else {
                 store_tile(0, k0, pm0.lim);
                 if (tile_begin + 1 < tile_end) {
@@ -761,7 +772,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                     load_v_item(i, pb);
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                if (lane == 0) page_lims[(cur ^ 1) * PAGES + gw] = BS;
+                if (lane == 0 && half == 0) page_lims[(cur ^ 1) * PAGES + gw] = BS;
                 pm_pend = pm_new;
                 ++tile;
                 __syncthreads();
@@ -1136,7 +1147,7 @@ int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt, int mt
     if (nb <= 0 || nb > 0x7fffffff) return LAZYATTN_E_SHAPE;
     const MfmaDivs dv{FastDiv((uint32_t)n_mt), FastDiv((uint32_t)nsplit), FastDiv((uint32_t)p.num_kv_heads),
                       FastDiv((uint32_t)(p.num_q_heads / p.num_kv_heads))};
-    hipLaunchKernelGGL(kern, dim3((unsigned)nb), dim3((NC + 4) * 64), LDS_BYTES, stream, p, nsplit, n_mt, mt_total, dv);
+    hipLaunchKernelGGL(kern, dim3((unsigned)nb), dim3((NC + gather_waves(NC, HD)) * 64), LDS_BYTES, stream, p, nsplit, n_mt, mt_total, dv);
     return hipGetLastError() == hipSuccess ? LAZYATTN_OK : LAZYATTN_E_LAUNCH;
 }
 
