@@ -456,8 +456,7 @@ paged_decode_kernel(const lazyattn_prefill_params p, const int nsplit) {
 }
 
 // merge of the slices: one 32-lane group per (request, q head); it is given the few fields it
-// needs rather than the whole parameter block (a launch with ~450 bytes of kernel arguments
-// costs about a microsecond more than one with 64)
+// needs rather than the whole parameter block
 struct DecodeMergeArgs {
     const void *workspace, *b_start_loc;
     void *o;

@@ -13,8 +13,7 @@ extern template int launch_mfma_family<f16_t, 1>(const lazyattn_prefill_params &
 extern template int launch_mfma_family<f16_t, 2>(const lazyattn_prefill_params &, int, int, int, int, hipStream_t);
 
 // ---- merge split-KV partials ----
-// The few fields the merge needs, not the whole parameter block: a launch with ~450 bytes of kernel
-// arguments costs about a microsecond more than one with 64 on this part.
+// The few fields the merge needs, not the whole parameter block.
 struct MergeArgs {
     const void *workspace, *b_start_loc, *b_seq_len;
     void *o;
