@@ -13,7 +13,7 @@ from .. import _ffi
 # Repeat calls (a serving loop with fixed buffers, a benchmark) skip validation and the filling of the C struct:
 # the entry points keep the plans of their most recent distinct calls, keyed on every tensor's address, shape,
 # strides and dtype plus the scalar arguments.  A plan is a pure function of that key -- it holds no reference to
-# the caller's tensors -- unless making it had to convert an operand (int64 tables, a host-side scale, a 0/1
+# the caller's tensors except the cos/sin table -- unless making it had to convert an operand (int64 tables, a host-side scale, a 0/1
 # ``is_lazy``), whose copy depends on the operand's contents: such calls are validated every time.
 _calls: "OrderedDict" = OrderedDict()
 _CALLS_MAX = 64
@@ -42,7 +42,9 @@ def remember(key, plans, table) -> None:
         return
     while len(_calls) >= _CALLS_MAX:
         _calls.popitem(last=False)
-    _calls[key] = (None if table is None else _ffi.table_version(table), tuple(p.detached() for p in plans))
+    # (the entry holds the cos/sin table as well: the plans point at a re-laid-out copy of its contents, and while
+    # the table lives its address cannot pass to another table that would then be taken for it)
+    _calls[key] = (None if table is None else _ffi.table_version(table), tuple(p.detached() for p in plans), table)
 
 
 def run_plans(plans) -> None:
