@@ -97,7 +97,11 @@ prefill_combine_kernel(const MergeArgs p, const int nsplit) {
                 const int64_t so = (int64_t)(s0 + j < nsplit ? s0 + j : nsplit - 1) * split_rows;
                 e[j] = we[so];
 #pragma unroll
-                for (int i4 = 0; i4 < 4; ++i4) v[j][i4] = *reinterpret_cast<const uint2 *>(wb + so * D + i4 * (2 * R * 4));
+                for (int i4 = 0; i4 < 4; ++i4) {
+                    typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+                    const u32x2_t t = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t *>(wb + so * D + i4 * (2 * R * 4)));
+                    v[j][i4] = make_uint2(t[0], t[1]);
+                }
             }
             float bm = e[0].x;
 #pragma unroll
