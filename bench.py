@@ -114,7 +114,9 @@ def cpu_baseline(w, reps):
                            k_scale=w.k_scale, v_scale=w.v_scale)
         return time.perf_counter() - t
     once()
-    return statistics.median(once() for _ in range(reps))
+    if reps is None:                     # about ten seconds of host work, at least five calls
+        reps = max(5, min(1000, int(10.0 / max(min(once(), once()), 1e-4))))
+    return statistics.median(once() for _ in range(reps)), reps
 
 
 def bench_decode(a):
@@ -403,9 +405,8 @@ def main():
         out["host_us_in_hip_launches"] = round(launches_us, 1)  # of which: the C calls (four kernel launches)
     if not a.no_cpu:
         torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))
-        reps_cpu = 5 if a.config in (2, 3) else 3
         wc = w if a.config in (2, 3) else wl.config(a.config, shrink=8)
-        sec = cpu_baseline(wc, reps_cpu)
+        sec, reps_cpu = cpu_baseline(wc, None)
         out["cpu_baseline"] = {"value": round(wc.flops / sec / 1e12, 4), "unit": "TFLOP/s",
                                "cores": torch.get_num_threads(), "kind": "port",
                                "sample": f"{wc.name}: {reps_cpu} full calls, median {sec * 1e3:.1f} ms/call"
