@@ -464,7 +464,7 @@ struct DecodeMergeArgs {
     int32_t batch, num_q_heads, index_bits;
     int32_t head_dim;              // elements of an output row (below HD when the partial rows are padded)
 };
-template <typename T, int HD>
+template <typename T, int HD, int NB>
 __global__ void __launch_bounds__(256)
 paged_decode_merge_kernel(const DecodeMergeArgs p, const int nsplit) {
     using E = Elem<T>;
@@ -472,29 +472,35 @@ paged_decode_merge_kernel(const DecodeMergeArgs p, const int nsplit) {
     const int64_t r = (int64_t)blockIdx.x * (256 / LPR) + threadIdx.x / LPR;
     if (r >= (int64_t)p.batch * p.num_q_heads) return;
     const int b = (int)(r / p.num_q_heads), h = (int)(r % p.num_q_heads);
-    const int64_t qs = load_index(p.b_start_loc, b, p.index_bits);
-    if (load_index(p.b_start_loc, b + 1, p.index_bits) - qs != 1) return;
+    // (the two offsets without a branch on their width -- their low words; they are below 2^31 -- so that both
+    // loads are in flight together)
+    const int es = p.index_bits >> 3;
+    const uint32_t qs32 = *(const uint32_t *)((const char *)p.b_start_loc + (int64_t)b * es);
+    const uint32_t qe32 = *(const uint32_t *)((const char *)p.b_start_loc + (int64_t)(b + 1) * es);
+    const int64_t qs = qs32;
+    if (qe32 - qs32 != 1) return;
     const int d = (threadIdx.x % LPR) * 4;
     if (d >= p.head_dim) return;
     const float *wo = (const float *)p.workspace;
     const float *wl = wo + (int64_t)nsplit * p.batch * p.num_q_heads * D;
     const int64_t rows = (int64_t)p.batch * p.num_q_heads;
-    // eight slices per batch, log-sum-exps and partial rows requested together: one memory round trip
-    // per batch; batches are chained by a running maximum
+    // NB slices per batch (8, or 32 when there are more than 8 slices: a short single request is cut into up to
+    // 64), log-sum-exps and partial rows requested together: one memory round trip per batch; batches are
+    // chained by a running maximum
     float mx = -INFINITY, wsum = 0.f;
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int s0 = 0; s0 < nsplit; s0 += 8) {
-        float e[8];
-        float4 v[8];
+    for (int s0 = 0; s0 < nsplit; s0 += NB) {
+        float e[NB];
+        float4 v[NB];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < NB; ++j) {
             const int64_t ri = (int64_t)(s0 + j < nsplit ? s0 + j : nsplit - 1) * rows + r;
             e[j] = wl[ri];
             v[j] = *reinterpret_cast<const float4 *>(wo + ri * D + d);
         }
         float bm = e[0];
 #pragma unroll
-        for (int j = 1; j < 8; ++j) bm = fmaxf(bm, e[j]);
+        for (int j = 1; j < NB; ++j) bm = fmaxf(bm, e[j]);
         const float m_new = fmaxf(mx, bm);
         if (m_new == -INFINITY) continue;
         const float keep = __builtin_amdgcn_exp2f(mx - m_new);
@@ -502,7 +508,7 @@ paged_decode_merge_kernel(const DecodeMergeArgs p, const int nsplit) {
         wsum *= keep;
         mx = m_new;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < NB; ++j) {
             const float w = s0 + j < nsplit ? __builtin_amdgcn_exp2f(e[j] - mx) : 0.f;
             o.x = fmaf(w, v[j].x, o.x); o.y = fmaf(w, v[j].y, o.y); o.z = fmaf(w, v[j].z, o.z); o.w = fmaf(w, v[j].w, o.w);
             wsum += w;
@@ -541,14 +547,17 @@ bool decode_mfma_supports(const lazyattn_prefill_params &p) {
 
 // slices of the page axis per (request, kv head): enough waves to fill the chip, at least twelve
 // pages (six loop iterations) per slice -- shorter slices cost more in prologue, partials and merge
-// than they gain in parallelism (5 K keys, one request: 16-32 slices 32 us, 64 slices 43 us)
+// than they gain in parallelism -- but down to five pages for a single request and ten for a handful, where
+// nothing else fills the chip (5 K keys, call = both launches: one request 16 / 32 / 64 slices 27.4 / 19.8 /
+// 18.0 us; four requests 30.0 / 23.3 / 26.1 us)
 static int decode_splits(const lazyattn_prefill_params &p) {
     if (p.num_splits > 0) return p.num_splits > 64 ? 64 : p.num_splits;
     const int64_t natural = (int64_t)p.batch * p.num_kv_heads * ((p.num_q_heads / p.num_kv_heads + 15) / 16);
     if (natural <= 0) return 1;
     int64_t s = (256 * 8 + natural - 1) / natural;
     const int64_t pages = p.max_seq_len > 0 ? (p.max_seq_len + BS - 1) / BS : 64;
-    if (s > pages / 12) s = pages / 12;
+    const int64_t min_pages = natural <= 8 ? 5 : natural <= 32 ? 10 : 12;
+    if (s > pages / min_pages) s = pages / min_pages;
     if (s > 64) s = 64;
     return s < 1 ? 1 : (int)s;
 }
@@ -604,13 +613,17 @@ int launch_decode_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
         const int rows_wg = 256 / (decode_tile_dim(p) / 4);
         const dim3 mgrid((unsigned)((rows + rows_wg - 1) / rows_wg));
         const bool f16 = p.dtype == LAZYATTN_F16;
+#define LAZYATTN_DECODE_MERGE(HD, NB)                                                                                   \
+    {                                                                                                                   \
+        if (f16) hipLaunchKernelGGL((paged_decode_merge_kernel<f16_t, HD, NB>), mgrid, dim3(256), 0, stream, m, nsplit); \
+        else hipLaunchKernelGGL((paged_decode_merge_kernel<bf16_t, HD, NB>), mgrid, dim3(256), 0, stream, m, nsplit);    \
+    }
         if (p.head_dim == 64) {
-            if (f16) hipLaunchKernelGGL((paged_decode_merge_kernel<f16_t, 64>), mgrid, dim3(256), 0, stream, m, nsplit);
-            else hipLaunchKernelGGL((paged_decode_merge_kernel<bf16_t, 64>), mgrid, dim3(256), 0, stream, m, nsplit);
+            if (nsplit <= 8) LAZYATTN_DECODE_MERGE(64, 8) else LAZYATTN_DECODE_MERGE(64, 32)
         } else {
-            if (f16) hipLaunchKernelGGL((paged_decode_merge_kernel<f16_t, 128>), mgrid, dim3(256), 0, stream, m, nsplit);
-            else hipLaunchKernelGGL((paged_decode_merge_kernel<bf16_t, 128>), mgrid, dim3(256), 0, stream, m, nsplit);
+            if (nsplit <= 8) LAZYATTN_DECODE_MERGE(128, 8) else LAZYATTN_DECODE_MERGE(128, 32)
         }
+#undef LAZYATTN_DECODE_MERGE
         if (hipGetLastError() != hipSuccess) return LAZYATTN_E_LAUNCH;
     }
     return LAZYATTN_OK;
