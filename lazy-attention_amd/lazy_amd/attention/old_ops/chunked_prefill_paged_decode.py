@@ -42,6 +42,11 @@ def chunked_prefill_paged_decode(query, key, value, output, kv_cache_dtype, key_
             skip_decode=True, rotary_dim=rotary_dim, cos_sin_cache=cos_sin_cache,
             is_neox_style=is_neox_style, q_mask=q_mask, q_offset=q_offset, is_mepic=is_mepic,
             force_fp32_rotary=force_fp32_rotary, _return_plan=True))
+    if plans and seq_lens.shape[0] == 1 and query.shape[0] > 1:
+        # the only request has more than one new token: the q_len == 1 launches would find no row of theirs
+        _launch.run_plans(plans)
+        _launch.remember(sig, plans, cos_sin_cache)
+        return
     plans.append(_launch.launch_prefill(
         q=query, k=key, v=value, o=output, kv_cache_dtype=kv_cache_dtype, k_cache=key_cache,
         v_cache=value_cache, b_loc=block_table, b_start_loc=query_start_loc, b_seq_len=seq_lens,

@@ -80,6 +80,12 @@ def chunked_prefill_paged_decode(query, key, value, output, kv_cache_dtype, key_
             alibi_slopes=alibi_slopes, sliding_window=sliding_window, sm_scale=sm_scale,
             skip_decode=True, rotary_dim=rotary_dim, cos_sin_cache=cos_sin_cache,
             is_neox_style=is_neox_style, is_lazy=is_lazy, q_offset=pq_offset, q_mask=pq_mask, _return_plan=True))
+    if plans and seq_lens.shape[0] == 1 and query.shape[0] > 1:
+        # the only request has more than one new token: the q_len == 1 launches would find no row of theirs
+        _launch.run_plans(plans)
+        if pure:
+            _launch.remember(sig, plans, cos_sin_cache)
+        return
     made = ()
     if is_lazy is None:
         is_lazy = torch.zeros(seq_lens.shape[0], dtype=torch.bool, device=query.device)

@@ -213,3 +213,36 @@ def test_repeat_calls_on_the_same_buffers_follow_their_contents(variant):
         out.fill_(5.0)
         _call(entry, variant, g, out, packed, lazy, block_table=wide)
         assert (out.cpu().float() - _expected(first, lazy_host).float()).abs().max().item() < 2e-2
+
+
+@pytest.mark.parametrize("variant", ["natural", "block_uniform"])
+def test_single_request_with_many_new_tokens_needs_no_single_token_launch(variant):
+    """One request with more than one new token: the q_len==1 launches have no row to work on and are left out
+    (the reference's second kernel finds nothing to do there: old_ops/chunked_prefill_paged_decode.py:396-442);
+    the output is the prefill kernel's."""
+    from lazy_amd.attention import _launch
+    print(f"case: single request {variant}", flush=True)
+    d = 128
+    w = wl.make_workload("single", dtype=torch.bfloat16, hq=8, hkv=2, d=d, theta=500000.0, block_size=16,
+                         doc_lens=[40, 16, 33], requests=[[2, 0, 1]], q_lens=[21], variant=variant, seed=5)
+    lazy = torch.tensor([True]) if variant == "block_uniform" else None
+    ref = torch.full_like(w.q, 5.0)
+    orc.prefix_prefill(w.q, w.k, w.v, w.k_cache, w.v_cache, w.block_table, w.b_start_loc, w.b_seq_len,
+                       w.cos_sin_cache, w.q_offset, w.q_mask, pos_mode=w.pos_mode,
+                       rotate_new_k=w.rotate_new_k, is_lazy=lazy, skip_decode=True, out=ref)
+    g = w.to(DEV)
+    out = torch.full_like(g.q, 5.0)
+    _launch.forget_calls()
+    if variant == "natural":
+        entry_unrotated(g.q, g.k, g.v, out, "auto", g.k_cache, g.v_cache, g.block_table, g.b_start_loc, g.b_seq_len,
+                        g.max_seq_len, g.max_query_len, g.k_scale, g.v_scale, sm_scale=d ** -0.5, rotary_dim=d,
+                        cos_sin_cache=g.cos_sin_cache, q_mask=g.q_mask)
+    else:
+        entry_block_uniform(g.q, g.k, g.v, out, "auto", g.k_cache, g.v_cache, g.block_table, g.b_start_loc,
+                            g.b_seq_len, g.max_seq_len, g.max_query_len, g.k_scale, g.v_scale, sm_scale=d ** -0.5,
+                            rotary_dim=d, cos_sin_cache=g.cos_sin_cache, is_lazy=lazy.to(DEV), q_offset=g.q_offset,
+                            q_mask=g.q_mask)
+    err = (out.cpu().float() - ref.float()).abs().max().item()
+    assert err < 2e-2, err
+    (entry,) = _launch._calls.values()
+    assert len(entry[1]) == 1 and not entry[1][0].decode
