@@ -86,7 +86,7 @@ def _err(a, b):
 
 
 @pytest.mark.parametrize("variant", ["natural", "block_uniform"])
-@pytest.mark.parametrize("nsplit", [0, 1, 3, 7])
+@pytest.mark.parametrize("nsplit", [0, 1, 3, 7, 8, 9, 33, 64])      # the merge loads 8 or 32 slices at a time
 def test_decode_ragged(variant, nsplit):
     print(f"case: decode ragged {variant} nsplit={nsplit}", flush=True)
     w = _decode_batch(variant)
