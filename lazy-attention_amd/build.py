@@ -1,4 +1,5 @@
-"""Compile the HIP sources in csrc/ into lazy_amd/_lib/liblazyattn.so for gfx950.
+"""Compile the HIP sources in csrc/ into lazy_amd/_lib/liblazyattn.so for gfx950, and the host helper
+csrc/host/callkey.cpp into lazy_amd/_lib/_callkey.so.
 
 Usage: python build.py [--jobs N].  hipcc cross-compiles without a GPU.
 """
@@ -42,9 +43,29 @@ def build_library(jobs: int = 4, extra: list[str] | None = None, verbose: bool =
     return LIB
 
 
+def build_callkey(verbose: bool = True) -> str:
+    """The host helper csrc/host/callkey.cpp (a CPython module, no GPU code): g++ against torch's headers."""
+    import sysconfig
+    from torch.utils import cpp_extension as ce
+    import torch
+    os.makedirs(OUT_DIR, exist_ok=True)
+    out = os.path.join(OUT_DIR, "_callkey.so")
+    libdirs = ce.library_paths()
+    cmd = ["g++", "-O2", "-shared", "-fPIC", "-std=c++17", "-w",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           *[f"-I{d}" for d in ce.include_paths()], f"-I{sysconfig.get_paths()['include']}",
+           os.path.join(CSRC, "host", "callkey.cpp"), "-o", out,
+           *[f"-L{d}" for d in libdirs], "-ltorch_python", *[f"-Wl,-rpath,{d}" for d in libdirs]]
+    subprocess.check_call(cmd)
+    if verbose:
+        print(f"built {out}", file=sys.stderr)
+    return out
+
+
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--jobs", type=int, default=4)
     ap.add_argument("--save-temps", action="store_true")
     a = ap.parse_args()
     build_library(a.jobs, ["-save-temps=obj"] if a.save_temps else [])
+    build_callkey()

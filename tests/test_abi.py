@@ -127,12 +127,28 @@ def test_table_version_of_inference_tensors():
     assert _ffi.table_version(u) == v0 + 1
 
 
-def test_remembered_calls_keying_and_invalidation():
+@pytest.mark.parametrize("compiled", [True, False])
+def test_remembered_calls_keying_and_invalidation(compiled, monkeypatch):
     """Host logic of the entry points' call memory: the key tells apart views of one buffer that differ in shape,
     strides or dtype; a remembered call is dropped when the cos/sin table it was made for has been edited in place,
-    and all of them when the re-laid-out tables are invalidated by hand."""
+    and all of them when the re-laid-out tables are invalidated by hand.  Both forms of the key: the compiled
+    helper (csrc/host/callkey.cpp) and the Python tuple used when it is not built."""
     from lazy_amd.attention import _launch
+    if compiled:
+        assert _launch._tensor_key is not None, "lazy_amd/_lib/_callkey.so is not built (python lazy-attention_amd/build.py)"
+    else:
+        monkeypatch.setattr(_launch, "_tensor_key", None)
     base = torch.zeros(8, 16)
+    scalar = torch.tensor(3.0)                            # zero-dimensional
+    assert _launch.call_key("t", (base, None, scalar), ()) == _launch.call_key("t", (base, None, scalar), ())
+    assert _launch.call_key("t", (base, None), ()) != _launch.call_key("t", (None, base), ())
+    assert _launch.call_key("t", (base,), ()) != _launch.call_key("t", (base[1:],), ())             # other address
+    assert _launch.call_key("t", (base[:4], base), ()) != _launch.call_key("t", (base, base[:4]), ())
+    with torch.inference_mode():
+        inf = torch.zeros(8, 16)
+    assert _launch.call_key("t", (inf,), ()) == _launch.call_key("t", (inf,), ())
+    with pytest.raises((TypeError, AttributeError)):
+        _launch.call_key("t", (1.0,), ())
     k0 = _launch.call_key("t", (base, None), (1, 2.0, None))
     assert k0 == _launch.call_key("t", (base, None), (1, 2.0, None))
     assert k0 != _launch.call_key("t", (base.t(), None), (1, 2.0, None))            # same address, other strides
