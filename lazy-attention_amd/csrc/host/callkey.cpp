@@ -1,5 +1,5 @@
 // Host helper of the Python entry points (no GPU code): the key under which a validated call is remembered.
-// tensor_key(tuple) packs address, dtype, sizes and strides of every tensor of the tuple (None: a marker) into one
+// tensor_key(tuple[, open_dim0]) packs address, dtype, sizes and strides of every tensor of the tuple (None: a marker) into one
 // bytes object -- hashable, compared bytewise -- in a fifth of a microsecond; the same tuple built in Python from
 // data_ptr() / shape / stride() / dtype costs six.  A CPython module linked against libtorch_python for
 // THPVariable_Unpack; lazy_amd/attention/_launch.py falls back to the Python tuple when it is not built.
@@ -9,9 +9,16 @@
 #include <string>
 
 static PyObject *tensor_key(PyObject *, PyObject *const *args, Py_ssize_t nargs) {
-    if (nargs != 1 || !PyTuple_Check(args[0])) {
-        PyErr_SetString(PyExc_TypeError, "tensor_key(tuple of tensors or None)");
+    if (nargs < 1 || nargs > 2 || !PyTuple_Check(args[0])) {
+        PyErr_SetString(PyExc_TypeError, "tensor_key(tuple of tensors or None[, open_dim0: int])");
         return nullptr;
+    }
+    // bit i set: the first dimension of tensor i is left out of the key (a per-token or per-request count that the
+    // caller handles itself)
+    unsigned long long open_dim0 = 0;
+    if (nargs == 2) {
+        open_dim0 = PyLong_AsUnsignedLongLongMask(args[1]);
+        if (PyErr_Occurred()) return nullptr;
     }
     PyObject *tup = args[0];
     const Py_ssize_t n = PyTuple_GET_SIZE(tup);
@@ -34,7 +41,8 @@ static PyObject *tensor_key(PyObject *, PyObject *const *args, Py_ssize_t nargs)
         }
         buf[m++] = (int64_t)(intptr_t)t.data_ptr();
         buf[m++] = ((int64_t)t.scalar_type() << 8) | (int64_t)sizes.size();
-        for (auto s : sizes) buf[m++] = s;
+        const bool open = i < 64 && ((open_dim0 >> i) & 1ull) && !sizes.empty();
+        for (size_t j = 0; j < sizes.size(); ++j) buf[m++] = (open && j == 0) ? -2 : sizes[j];
         for (auto s : strides) buf[m++] = s;
     }
     } catch (const std::exception &e) {             // (a tensor without storage has no address)

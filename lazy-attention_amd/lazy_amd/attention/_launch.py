@@ -15,8 +15,13 @@ from .. import _ffi
 # strides and dtype plus the scalar arguments.  A plan is a pure function of that key -- it holds no reference to
 # the caller's tensors except the cos/sin table -- unless making it had to convert an operand (int64 tables, a host-side scale, a 0/1
 # ``is_lazy``), whose copy depends on the operand's contents: such calls are validated every time.
+# The backend's entry points (``chunked_prefill_paged_decode``) leave the counts that change from one engine step to
+# the next out of the key -- the first dimension of the per-token and per-request tensors (views ``buf[:n]`` of
+# persistent buffers share an address), ``max_seq_len``, ``max_query_len`` -- and write them into the remembered
+# structs before the launch (``PrefillPlan.resize``): they are four fields there, and nothing else in a plan depends
+# on them.  A plan that owns a tensor sized by such a count is bound to the counts it was made for.
 _calls: "OrderedDict" = OrderedDict()
-_CALLS_MAX = 64
+_CALLS_MAX = 256                            # (one per layer and kind of step of a served model)
 
 
 def _load_tensor_key():
@@ -38,34 +43,47 @@ def _load_tensor_key():
 _tensor_key = _load_tensor_key()
 
 
-def call_key(tag, tensors, scalars):
+def call_key(tag, tensors, scalars, open_dim0: int = 0):
+    """``open_dim0``: bit i set = the first dimension of ``tensors[i]`` is not part of the key."""
     if _tensor_key is not None:
-        return (tag, scalars, _tensor_key(tensors))      # 0.2 us for fifteen tensors; the tuple below takes 6
-    return (tag, scalars, tuple([None if t is None else (t.data_ptr(), t.shape, t.stride(), t.dtype)
-                                 for t in tensors]))
+        return (tag, scalars, _tensor_key(tensors, open_dim0))      # 0.2 us for fifteen tensors; the tuple below takes 6
+    return (tag, scalars, tuple([None if t is None else
+                                 (t.data_ptr(), t.shape[1:] if (open_dim0 >> i) & 1 else t.shape, t.stride(), t.dtype)
+                                 for i, t in enumerate(tensors)]))
 
 
-def recall(key, table):
+def recall(key, table, counts=None, bound=None):
     """The plans remembered for this call, or None.  ``table`` is the caller's cos/sin table: its edit counter
-    is compared because the plans point at a re-laid-out copy of it."""
+    is compared because the plans point at a re-laid-out copy of it.  ``counts`` = (batch, num_tokens, max_seq_len,
+    max_q_len) of this call when the key leaves them open: the plans are set to them (None when their workspace
+    is too small for these counts).  ``bound``: what a plan that owns count-sized tensors must have been made for."""
     hit = _calls.get(key)
     if hit is None:
         return None
     if hit[0] != (None if table is None else _ffi.table_version(table)):
         del _calls[key]
         return None
+    if hit[3] is not None and hit[3] != bound:
+        return None
+    if counts is not None and hit[4] != counts:
+        for p in hit[1]:
+            if not p.resize(*counts):
+                del _calls[key]
+                return None
+        hit[4] = counts
     _calls.move_to_end(key)
     return hit[1]
 
 
-def remember(key, plans, table) -> None:
+def remember(key, plans, table, counts=None, bound=None) -> None:
     if not all(p.repeatable for p in plans):
         return
     while len(_calls) >= _CALLS_MAX:
         _calls.popitem(last=False)
     # (the entry holds the cos/sin table as well: the plans point at a re-laid-out copy of its contents, and while
     # the table lives its address cannot pass to another table that would then be taken for it)
-    _calls[key] = (None if table is None else _ffi.table_version(table), tuple(p.detached() for p in plans), table)
+    _calls[key] = [None if table is None else _ffi.table_version(table), tuple(p.detached() for p in plans), table,
+                   bound if any(p.count_sized for p in plans) else None, counts]
 
 
 def run_plans(plans) -> None:
@@ -197,6 +215,7 @@ class PrefillPlan:
     def __init__(self, params, device, decode, keep, own=(), repeatable=False):
         self.params, self.device, self.decode, self._keep, self._own = params, device, decode, keep, own
         self.repeatable = repeatable        # no operand had to be converted: the struct depends on the key alone
+        self.count_sized = False            # owns tensors sized by the batch (made by the entry point for this call)
         self._lib = _ffi.lib()
         self._entry = self._lib.lazyattn_paged_decode_rotary if decode else self._lib.lazyattn_prefix_prefill
         self._ws = None
@@ -214,10 +233,23 @@ class PrefillPlan:
         if rc:
             _ffi.check(rc, "lazyattn_paged_decode_rotary" if self.decode else "lazyattn_prefix_prefill")
 
+    def resize(self, batch: int, num_tokens: int, max_seq_len: int, max_q_len: int) -> bool:
+        """Set the counts of the call (the struct's only fields that depend on the first dimension of the per-token
+        and per-request tensors, and the two host-side maxima).  False: the plan's workspace is too small for them."""
+        pr = self.params
+        pr.batch, pr.num_tokens, pr.max_seq_len = batch, num_tokens, int(max_seq_len or 0)
+        if not self.decode:
+            pr.max_q_len = max_q_len
+        need = (self._lib.lazyattn_paged_decode_workspace_bytes(pr) if self.decode
+                else self._lib.lazyattn_prefill_workspace_bytes(pr))
+        return need <= (self._ws.numel() if self._ws is not None else 0)
+
     def also_keep(self, *tensors) -> None:
         """Tensors the entry point made for this call whose contents do not depend on the caller's (an all-false
-        ``is_lazy``, a zero ``q_offset``): they live as long as the plan."""
+        ``is_lazy``, a zero ``q_offset``): they live as long as the plan, and being sized by the batch they bind a
+        remembered plan to the batch it was made for."""
         self._own = self._own + tensors
+        self.count_sized = self.count_sized or len(tensors) > 0
 
     def detached(self) -> "PrefillPlan":
         """The same call without references to the caller's tensors (what the entry points remember)."""

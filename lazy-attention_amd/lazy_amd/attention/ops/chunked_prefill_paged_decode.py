@@ -44,6 +44,11 @@ def unpack_block_table(packed: torch.Tensor):
     return blk, off, msk
 
 
+# tensors of the key whose first dimension is a token or request count: query, key, value, output, block_table,
+# query_start_loc, seq_lens, is_lazy, q_offset, q_mask, packed_block_table (positions in the tuple below)
+_OPEN_DIM0 = sum(1 << i for i in (0, 1, 2, 3, 6, 7, 8, 14, 15, 16, 17))
+
+
 def chunked_prefill_paged_decode(query, key, value, output, kv_cache_dtype, key_cache, value_cache,
                                  block_table, query_start_loc, seq_lens, max_seq_len, max_query_len,
                                  k_scale, v_scale, alibi_slopes=None, sliding_window=None,
@@ -53,14 +58,21 @@ def chunked_prefill_paged_decode(query, key, value, output, kv_cache_dtype, key_
     if _env_flag("NO_LAZY") and is_lazy is not None:
         is_lazy.fill_(False)                             # ops/chunked...:66-67
     compute = _env_flag("LAZY_DECODE_COMPUTE_COS_SIN")   # ops/chunked...:146-151
+    # the counts that change from step to step are not part of the key: views [:n] of persistent buffers find the
+    # call made for another n, and its structs are set to this call's counts
+    batch, single = seq_lens.shape[0], seq_lens.shape[0] == 1
+    counts = (batch, output.shape[0], max_seq_len, max_query_len)
+    bound = (batch, block_table.shape[0])                # what a plan that owns batch-sized tensors stays tied to
     sig = _launch.call_key(
         "block-uniform", (query, key, value, output, key_cache, value_cache, block_table, query_start_loc, seq_lens,
                           k_scale, v_scale, alibi_slopes, freqs, cos_sin_cache, is_lazy, q_offset, q_mask,
                           packed_block_table),
-        (kv_cache_dtype, max_seq_len, max_query_len, sliding_window, sm_scale, rotary_dim, is_neox_style, compute))
-    plans = _launch.recall(sig, cos_sin_cache)
-    if plans is not None:
-        return _launch.run_plans(plans)
+        (kv_cache_dtype, sliding_window, sm_scale, rotary_dim, is_neox_style, compute, max_query_len > 1, single),
+        _OPEN_DIM0)
+    if query_start_loc.shape[0] == batch + 1:            # (anything else goes to the checks below)
+        plans = _launch.recall(sig, cos_sin_cache, counts, bound)
+        if plans is not None:
+            return _launch.run_plans(plans)
     plans, pure = [], True
     if sm_scale is None:
         sm_scale = 1.0 / (query.shape[1] ** 0.5)         # sic: ops/chunked...:71-72
@@ -80,11 +92,11 @@ def chunked_prefill_paged_decode(query, key, value, output, kv_cache_dtype, key_
             alibi_slopes=alibi_slopes, sliding_window=sliding_window, sm_scale=sm_scale,
             skip_decode=True, rotary_dim=rotary_dim, cos_sin_cache=cos_sin_cache,
             is_neox_style=is_neox_style, is_lazy=is_lazy, q_offset=pq_offset, q_mask=pq_mask, _return_plan=True))
-    if plans and seq_lens.shape[0] == 1 and query.shape[0] > 1:
+    if plans and single:
         # the only request has more than one new token: the q_len == 1 launches would find no row of theirs
         _launch.run_plans(plans)
         if pure:
-            _launch.remember(sig, plans, cos_sin_cache)
+            _launch.remember(sig, plans, cos_sin_cache, counts, bound)
         return
     made = ()
     if is_lazy is None:
@@ -119,4 +131,4 @@ def chunked_prefill_paged_decode(query, key, value, output, kv_cache_dtype, key_
     plans[-1].also_keep(*made)
     _launch.run_plans(plans)
     if pure:
-        _launch.remember(sig, plans, cos_sin_cache)
+        _launch.remember(sig, plans, cos_sin_cache, counts, bound)

@@ -144,6 +144,11 @@ def test_remembered_calls_keying_and_invalidation(compiled, monkeypatch):
     assert _launch.call_key("t", (base, None), ()) != _launch.call_key("t", (None, base), ())
     assert _launch.call_key("t", (base,), ()) != _launch.call_key("t", (base[1:],), ())             # other address
     assert _launch.call_key("t", (base[:4], base), ()) != _launch.call_key("t", (base, base[:4]), ())
+    # the first dimension of chosen tensors left open (views [:n] of one buffer share a key)
+    assert _launch.call_key("t", (base[:4], base), (), 0b01) == _launch.call_key("t", (base[:6], base), (), 0b01)
+    assert _launch.call_key("t", (base[:4], base), (), 0b10) != _launch.call_key("t", (base[:6], base), (), 0b10)
+    assert _launch.call_key("t", (base[:, :4],), (), 0b1) != _launch.call_key("t", (base[:, :6],), (), 0b1)
+    assert _launch.call_key("t", (base[:4],), (), 0b1) != _launch.call_key("t", (base[:4],), (), 0)
     with torch.inference_mode():
         inf = torch.zeros(8, 16)
     assert _launch.call_key("t", (inf,), ()) == _launch.call_key("t", (inf,), ())
@@ -159,6 +164,7 @@ def test_remembered_calls_keying_and_invalidation(compiled, monkeypatch):
 
     class Plan:                                       # stands in for a validated call
         repeatable = True
+        count_sized = False
         def detached(self): return self
     _launch.forget_calls()
     table = torch.ones(4, 16)
@@ -172,6 +178,22 @@ def test_remembered_calls_keying_and_invalidation(compiled, monkeypatch):
     _launch.remember(k0, (Plan(),), table)
     _ffi.invalidate_packed_tables()
     assert len(_launch._calls) == 0
+    # counts left out of the key are written into the remembered plans; a plan whose workspace is too small for
+    # them is dropped; a plan that owns batch-sized tensors only serves the batch it was made for
+    class Sized(Plan):
+        def __init__(self): self.seen, self.fits = None, True
+        def resize(self, *counts): self.seen = counts; return self.fits
+    sp = Sized()
+    _launch.remember(k0, (sp,), None, (4, 80, 100, 70))
+    assert _launch.recall(k0, None, (4, 80, 100, 70)) is not None and sp.seen is None        # same counts: nothing to set
+    assert _launch.recall(k0, None, (2, 71, 90, 70)) is not None and sp.seen == (2, 71, 90, 70)
+    sp.fits = False
+    assert _launch.recall(k0, None, (3, 80, 95, 70)) is None and len(_launch._calls) == 0
+    sp.fits, sp.count_sized = True, True
+    _launch.remember(k0, (sp,), None, (4, 80, 100, 70), bound=(4, 4))
+    assert _launch.recall(k0, None, (2, 71, 90, 70), bound=(2, 2)) is None and len(_launch._calls) == 1
+    assert _launch.recall(k0, None, (4, 71, 90, 70), bound=(4, 4)) is not None
+    _launch.forget_calls()
     for i in range(_launch._CALLS_MAX + 5):           # bounded: the oldest entries leave
         _launch.remember(("k", i), (Plan(),), None)
     assert len(_launch._calls) == _launch._CALLS_MAX and _launch.recall(("k", 0), None) is None

@@ -246,3 +246,52 @@ def test_single_request_with_many_new_tokens_needs_no_single_token_launch(varian
     assert err < 2e-2, err
     (entry,) = _launch._calls.values()
     assert len(entry[1]) == 1 and not entry[1][0].decode
+
+
+def _sub_batch_call(entry, variant, g, w, b, out, packed, lazy, clone=False):
+    """The first ``b`` requests of the batch as views of its buffers (or as fresh copies of those views)."""
+    ntok = int(w.b_start_loc[b])
+    f = (lambda t: None if t is None else t.clone()) if clone else (lambda t: t)
+    q_lens = (w.b_start_loc[1:b + 1] - w.b_start_loc[:b])
+    args = (f(g.q[:ntok]), f(g.k[:ntok]), f(g.v[:ntok]), out[:ntok], "auto", g.k_cache, g.v_cache, f(g.block_table[:b]),
+            f(g.b_start_loc[:b + 1]), f(g.b_seq_len[:b]), int(w.b_seq_len[:b].max()), int(q_lens.max()),
+            g.k_scale, g.v_scale)
+    kw = dict(sm_scale=128 ** -0.5, rotary_dim=128, cos_sin_cache=g.cos_sin_cache, q_mask=f(g.q_mask[:b]))
+    if variant == "natural":
+        entry(*args, **kw)
+    else:
+        entry(*args, is_lazy=None if lazy is None else f(lazy[:b]), q_offset=f(g.q_offset[:b]),
+              packed_block_table=None if packed is None else f(packed[:b]), **kw)
+
+
+@pytest.mark.parametrize("variant,lazy_given", [("natural", False), ("block_uniform", True), ("block_uniform", False)])
+def test_views_of_persistent_buffers_reuse_the_call_made_for_other_counts(variant, lazy_given):
+    """An engine step passes views ``buf[:n]`` of persistent buffers, with a new ``n``, ``max_seq_len`` and
+    ``max_query_len`` every step (backends/triton_attn.py:146-187).  Those counts are not part of the remembered
+    call's key: the call made for one step serves the next, with its counts set anew.  Results must equal those of
+    calls validated from scratch (fresh copies of the same views, which share no address with the buffers), and
+    rows past the step's tokens must stay untouched.  Without ``is_lazy`` the entry point owns an all-false one sized
+    by the batch: such a call is tied to its batch size."""
+    from lazy_amd.attention import _launch
+    print(f"case: views of persistent buffers {variant} lazy_given={lazy_given}", flush=True)
+    entry = entry_unrotated if variant == "natural" else entry_block_uniform
+    w = _mixed(variant, torch.bfloat16, 128, seed=61)
+    g = w.to(DEV)
+    lazy = torch.tensor([True, True, False, True]).to(DEV) if lazy_given else None
+    packed = ((g.block_table.long() << 32) | (g.q_offset.long() << 16) | g.q_mask.long()) if variant == "block_uniform" else None
+    steps = (2, 3, 4, 2, 1, 4)
+    want = {}
+    for b in set(steps):
+        o = torch.full_like(g.q, 5.0)
+        _sub_batch_call(entry, variant, g, w, b, o, packed, lazy, clone=True)
+        want[b] = o
+    _launch.forget_calls()
+    out = torch.full_like(g.q, 5.0)
+    for b in steps:
+        out.fill_(5.0)
+        _sub_batch_call(entry, variant, g, w, b, out, packed, lazy)
+        assert torch.equal(out, want[b]), b
+        assert bool((out[int(w.b_start_loc[b]):] == 5.0).all())
+    # one remembered call for the steps with several requests (made again at every change of the batch size when it
+    # owns batch-sized tensors), one for the single request (no q_len == 1 launch there)
+    assert len(_launch._calls) == 2
