@@ -450,11 +450,12 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         m.lim = l < 0 ? 0 : l;
         return m;
     };
-    // Valid-slot counts of the four pages of a context tile, one int per page and LDS buffer:
-    // written by the gathering waves with the tile, read by the computing waves for the masks.
+    // Valid-slot counts of the four pages of a context tile, one byte per page and LDS buffer (a word per tile:
+    // the computing waves compare it with four times BS to tell a full tile): written by the gathering waves
+    // with the tile, read by the computing waves for the masks.
     constexpr bool QREG = q_in_registers(NC, HD);
     constexpr int Q_BYTES = QREG ? 0 : NC * G::Q_WAVE;
-    int *page_lims = reinterpret_cast<int *>(lds + KV_BYTES + Q_BYTES);
+    uint8_t *page_lims = lds + KV_BYTES + Q_BYTES;
 
     if (gatherer) {
         // ====================================================================== gather
@@ -711,7 +712,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         auto store_tile = [&](int buf, int kind, int lim) {
             store_k(lds + buf * K_TILE, kind);
             store_v(lds + 2 * K_TILE + buf * V_TILE, kind, lim);
-            if (lane == 0 && half == 0) page_lims[buf * PAGES + gw] = lim;
+            if (lane == 0 && half == 0) page_lims[buf * PAGES + gw] = (uint8_t)lim;
         };
 
         // At the top of iteration `tile` the raw K/V of tile+1 sit in registers (loaded during
@@ -738,7 +739,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                     load_v_item(i, pb);
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                if (lane == 0 && half == 0) page_lims[gw] = BS;
+                if (lane == 0 && half == 0) page_lims[gw] = (uint8_t)BS;
             } else {
                 store_tile(0, k0, pm0.lim);
                 if (tile_begin + 1 < tile_end) {
@@ -772,7 +773,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                     load_v_item(i, pb);
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                if (lane == 0 && half == 0) page_lims[(cur ^ 1) * PAGES + gw] = BS;
+                if (lane == 0 && half == 0) page_lims[(cur ^ 1) * PAGES + gw] = (uint8_t)BS;
                 pm_pend = pm_new;
                 ++tile;
                 __syncthreads();
@@ -972,25 +973,26 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     // which of the tile's 64 keys exist: new-token tiles from the token count, context tiles from the
     // page limits the gathering waves left beside the tile
     struct Desc { int kind; uint32_t vlo, vhi; int m0, key0; };
-    auto describe = [&](int tile, const int4 &lims) -> Desc {
+    static_assert(PAGES == 4 && BS < 256, "a tile's page limits travel as the four bytes of one word");
+    constexpr uint32_t FULL_LIMS = (uint32_t)BS * 0x01010101u;
+    auto describe_ctx = [&](int tile, uint32_t limw) -> Desc {
         Desc td{TILE_FULL, ~0u, ~0u, 0, tile * NT};
-        if (tile >= n_ctx_tiles) {
-            td.kind = TILE_NEW;
-            td.m0 = (tile - n_ctx_tiles) * NT;
-            td.key0 = ctx_len + td.m0;
-            const int n = t_end - td.m0;
-            const uint64_t valid = n >= 64 ? ~0ull : (n <= 0 ? 0ull : ((1ull << n) - 1ull));
-            td.vlo = (uint32_t)valid; td.vhi = (uint32_t)(valid >> 32);
-        } else {
-            const int l0 = uniform(lims.x), l1 = uniform(lims.y), l2 = uniform(lims.z), l3 = uniform(lims.w);
-            if ((l0 & l1 & l2 & l3) != BS) {
-                td.kind = TILE_EDGE;
-                td.vlo = ((1u << l0) - 1u) | (((1u << l1) - 1u) << BS);
-                td.vhi = ((1u << l2) - 1u) | (((1u << l3) - 1u) << BS);
-            }
+        if (limw != FULL_LIMS) {
+            const uint32_t l0 = limw & 0xffu, l1 = (limw >> 8) & 0xffu, l2 = (limw >> 16) & 0xffu, l3 = limw >> 24;
+            td.kind = TILE_EDGE;
+            td.vlo = ((1u << l0) - 1u) | (((1u << l1) - 1u) << BS);
+            td.vhi = ((1u << l2) - 1u) | (((1u << l3) - 1u) << BS);
         }
         // a tile that starts before the window of this wave's last row needs the per-row lower bound
         if (window && td.kind == TILE_FULL && td.key0 < ctx_len + t0 + UNIT - window) td.kind = TILE_EDGE;
+        return td;
+    };
+    auto describe_new = [&](int tile) -> Desc {
+        Desc td{TILE_NEW, ~0u, ~0u, (tile - n_ctx_tiles) * NT, 0};
+        td.key0 = ctx_len + td.m0;
+        const int n = t_end - td.m0;
+        const uint64_t valid = n >= 64 ? ~0ull : (n <= 0 ? 0ull : ((1ull << n) - 1ull));
+        td.vlo = (uint32_t)valid; td.vhi = (uint32_t)(valid >> 32);
         return td;
     };
     // The tile body, in the order the instructions are issued.  A wave's own vector work sits behind its own
@@ -1004,52 +1006,66 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     // That is the path of a full tile whose rows have all seen a key (no masks, no row maximum).  Any other
     // tile computes S1 first, masks, takes the maximum over both halves (the reference may move), and then forms
     // P0 in one go; from C on the two paths are the same instructions.
-    __syncthreads();
-    for (int tile = tile_begin; tile < tile_end; ++tile) {
+    // Context tiles and new-token tiles run the same body from two loops: the context loop carries none of the
+    // new-token bookkeeping (between the two score phases a full tile now has a compare and a branch where the
+    // common loop had some thirty scalar instructions, an eighth of the tile's time with one computing wave per SIMD).
+    bool all_seen = false;       // wave-uniform: every row of this wave has met a key (full tiles then need no maximum)
+    auto tile_body = [&](int tile, auto new_tile) {
+        constexpr bool NEWT = decltype(new_tile)::value;
         const int cur = (tile - tile_begin) & 1;
         const uint8_t *ktile = lds + cur * K_TILE;
         const uint8_t *vtile = lds + 2 * K_TILE + cur * V_TILE;
-        const bool is_new = tile >= n_ctx_tiles;
-        // Rows of an idle wave are all-zero queries (harmless, never stored); a new-token tile
-        // entirely in this wave's future contributes nothing (causal) and is skipped.
-        if (!is_new || (tile - n_ctx_tiles) * NT <= t0 + UNIT - 1) {
-            // valid-slot counts of the tile's pages: requested now, looked at after phase A
-            const int4 lims = *reinterpret_cast<const int4 *>(page_lims + cur * PAGES);
-            f32x16_t s0, s1;
-            HalfP h0, h1;
-            __builtin_amdgcn_s_setprio(2);
-            qk_half(ktile, 0, s0, [](int) {});
-            const Desc td = describe(tile, lims);
-            const bool lazy = td.kind == TILE_FULL && __builtin_amdgcn_ballot_w64(!seen) == 0;
+        // valid-slot counts of the tile's pages: requested now, looked at after phase A
+        uint32_t limw = FULL_LIMS;
+        if constexpr (!NEWT) limw = *reinterpret_cast<const uint32_t *>(page_lims + cur * PAGES);
+        f32x16_t s0, s1;
+        HalfP h0, h1;
+        __builtin_amdgcn_s_setprio(2);
+        qk_half(ktile, 0, s0, [](int) {});
+        Desc td;
+        bool lazy = false;
+        if constexpr (NEWT) {
+            td = describe_new(tile);
+            qk_half(ktile, 1, s1, [](int) {});
+        } else {
+            td = describe_ctx(tile, (uint32_t)uniform((int)limw));
+            lazy = td.kind == TILE_FULL && all_seen;
             // (the exponentials of S0 are formed behind these MFMAs on every tile: a tile that is not lazy forms
             // them again after its masks and maximum, and the first set, possibly garbage, is dropped)
             qk_half(ktile, 1, s1, [&](int ks) {
 #pragma unroll
                 for (int i = 0; i < 8 / KS; ++i) exp_piece(s0, h0, ks * (8 / KS) + i);
             });
-            // The maximum is needed when the tile is not lazy, or when a lazy tile's row sums say that some P of
-            // the first half left the comfortable range: one path for both (then P0 is formed again).
-            bool slow = !lazy;
+        }
+        // The maximum is needed when the tile is not lazy, or when a lazy tile's row sums say that some P of
+        // the first half left the comfortable range: one path for both (then P0 is formed again).
+        bool slow = !lazy;
+        if constexpr (!NEWT) {
             if (lazy) slow = __builtin_amdgcn_ballot_w64(!(h0.ta + h0.tb <= SUM_LIMIT)) != 0;
-            if (slow) {
-                // (the first set of P0 counts as used here too: otherwise the compiler moves its exponentials
-                // out from behind the MFMAs into the branch that keeps them)
+        }
+        if (slow) {
+            // (the first set of P0 counts as used here too: otherwise the compiler moves its exponentials
+            // out from behind the MFMAs into the branch that keeps them)
+            if constexpr (!NEWT) {
 #pragma unroll
                 for (int i = 0; i < 8; ++i) asm volatile("" ::"v"(h0.w[i]));
-                __builtin_amdgcn_s_setprio(0);
-                if (td.kind != TILE_FULL) {
-                    mask_half(s0, td.vlo, 0, td.kind, td.m0, td.key0);
-                    mask_half(s1, td.vhi, 1, td.kind, td.m0, td.key0);
-                }
-                rebase(s0, s1);
-                exp_half(s0, h0);
-                __builtin_amdgcn_s_setprio(2);
             }
-            float sum0 = h0.ta + h0.tb;
-            pv_half(vtile, 0, h0, [&](int j) {
+            __builtin_amdgcn_s_setprio(0);
+            if (td.kind != TILE_FULL) {
+                mask_half(s0, td.vlo, 0, td.kind, td.m0, td.key0);
+                mask_half(s1, td.vhi, 1, td.kind, td.m0, td.key0);
+            }
+            rebase(s0, s1);
+            all_seen = __builtin_amdgcn_ballot_w64(!seen) == 0;
+            exp_half(s0, h0);
+            __builtin_amdgcn_s_setprio(2);
+        }
+        float sum0 = h0.ta + h0.tb;
+        pv_half(vtile, 0, h0, [&](int j) {
 #pragma unroll
-                for (int i = 0; i < 8 / (2 * DT); ++i) exp_piece(s1, h1, j * (8 / (2 * DT)) + i);
-            });
+            for (int i = 0; i < 8 / (2 * DT); ++i) exp_piece(s1, h1, j * (8 / (2 * DT)) + i);
+        });
+        if constexpr (!NEWT) {
             if (lazy && __builtin_amdgcn_ballot_w64(!(h1.ta + h1.tb <= SUM_LIMIT))) {
                 // (the scores are made opaque here: otherwise half of the row maximum below is computed ahead
                 // of the branch, on every tile)
@@ -1058,10 +1074,22 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                 bump(s1, nullptr, &sum0);
                 exp_half(s1, h1);
             }
-            pv_half(vtile, 1, h1, [](int) {});
-            __builtin_amdgcn_s_setprio(0);
-            l_run += sum0 + (h1.ta + h1.tb);
         }
+        pv_half(vtile, 1, h1, [](int) {});
+        __builtin_amdgcn_s_setprio(0);
+        l_run += sum0 + (h1.ta + h1.tb);
+    };
+    __syncthreads();
+    int tile = tile_begin;
+    const int ctx_stop = tile_end < n_ctx_tiles ? tile_end : n_ctx_tiles;
+    for (; tile < ctx_stop; ++tile) {
+        tile_body(tile, std::false_type{});
+        __syncthreads();
+    }
+    for (; tile < tile_end; ++tile) {
+        // Rows of an idle wave are all-zero queries (harmless, never stored); a new-token tile
+        // entirely in this wave's future contributes nothing (causal) and is skipped.
+        if ((tile - n_ctx_tiles) * NT <= t0 + UNIT - 1) tile_body(tile, std::true_type{});
         __syncthreads();
     }
 
