@@ -945,6 +945,11 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         h.w[i] = E::pack(__builtin_amdgcn_exp2f(s[2 * i]), __builtin_amdgcn_exp2f(s[2 * i + 1]));
         if (i & 1) h.tb = E::dot2_ones(h.w[i], i == 1 ? 0.f : h.tb);
         else h.ta = E::dot2_ones(h.w[i], i == 0 ? 0.f : h.ta);
+        // (the sums count as used where they are formed: the first set of a tile is only read on the lazy path, and
+        // the compiler would otherwise collect its eight dot instructions in front of that path's check, between
+        // two MFMA phases, instead of leaving them behind the MFMAs)
+        if (i & 1) asm volatile("" : "+v"(h.tb));
+        else asm volatile("" : "+v"(h.ta));
     };
     auto exp_half = [&](const f32x16_t &s, HalfP &h) {
 #pragma unroll
