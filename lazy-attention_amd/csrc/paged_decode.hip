@@ -519,6 +519,72 @@ paged_decode_merge_kernel(const DecodeMergeArgs p, const int nsplit) {
     *reinterpret_cast<uint2 *>(op) = make_uint2(E::pack(o.x * inv, o.y * inv), E::pack(o.z * inv, o.w * inv));
 }
 
+// The same merge for a handful of rows and many slices (one or a few requests cut into up to 64 slices): a whole
+// workgroup per row, its 256 lanes = G groups of HD/4; group g takes slices g, g + G, ... (at most eight: all of
+// their loads are in flight together), and the G partial results meet in LDS.  With one 32-lane group per row the
+// four workgroups of a single request's 32 rows each pulled 160 KB through one CU in two dependent rounds.
+template <typename T, int HD>
+__global__ void __launch_bounds__(256)
+paged_decode_merge_wide_kernel(const DecodeMergeArgs p, const int nsplit) {
+    using E = Elem<T>;
+    constexpr int D = HD, LPR = HD / 4, G = 256 / LPR, PER = 64 / G;      // PER: slices per group when there are 64
+    __shared__ float sm[G][LPR][4];
+    __shared__ float se[G][2];
+    const int64_t r = blockIdx.x;
+    const int b = (int)(r / p.num_q_heads), h = (int)(r % p.num_q_heads);
+    const int es = p.index_bits >> 3;
+    const uint32_t qs32 = *(const uint32_t *)((const char *)p.b_start_loc + (int64_t)b * es);
+    const uint32_t qe32 = *(const uint32_t *)((const char *)p.b_start_loc + (int64_t)(b + 1) * es);
+    if (qe32 - qs32 != 1) return;                               // (the whole workgroup: one row)
+    const int g = threadIdx.x / LPR, ln = threadIdx.x % LPR, d = ln * 4;
+    const float *wo = (const float *)p.workspace;
+    const float *wl = wo + (int64_t)nsplit * p.batch * p.num_q_heads * D;
+    const int64_t rows = (int64_t)p.batch * p.num_q_heads;
+    float e[PER];
+    float4 v[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int sl = g + j * G;
+        const int64_t ri = (int64_t)(sl < nsplit ? sl : nsplit - 1) * rows + r;
+        e[j] = wl[ri];
+        v[j] = *reinterpret_cast<const float4 *>(wo + ri * D + d);
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) mx = fmaxf(mx, g + j * G < nsplit ? e[j] : -INFINITY);
+    float wsum = 0.f;
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (mx != -INFINITY) {
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const float w = g + j * G < nsplit ? __builtin_amdgcn_exp2f(e[j] - mx) : 0.f;
+            o.x = fmaf(w, v[j].x, o.x); o.y = fmaf(w, v[j].y, o.y); o.z = fmaf(w, v[j].z, o.z); o.w = fmaf(w, v[j].w, o.w);
+            wsum += w;
+        }
+    }
+    *reinterpret_cast<float4 *>(&sm[g][ln][0]) = o;
+    if (ln == 0) { se[g][0] = mx; se[g][1] = wsum; }
+    __syncthreads();
+    if (g != 0 || d >= p.head_dim) return;
+    float m_all = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < G; ++k) m_all = fmaxf(m_all, se[k][0]);
+    float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+    float w_all = 0.f;
+    if (m_all != -INFINITY) {
+#pragma unroll
+        for (int k = 0; k < G; ++k) {
+            const float c = __builtin_amdgcn_exp2f(se[k][0] - m_all);        // (a group without keys: exp2(-inf) = 0)
+            const float4 ok = *reinterpret_cast<const float4 *>(&sm[k][ln][0]);
+            t.x = fmaf(c, ok.x, t.x); t.y = fmaf(c, ok.y, t.y); t.z = fmaf(c, ok.z, t.z); t.w = fmaf(c, ok.w, t.w);
+            w_all = fmaf(c, se[k][1], w_all);
+        }
+    }
+    const float inv = w_all > 0.f ? 1.f / w_all : 0.f;
+    T *op = (T *)p.o + (int64_t)qs32 * p.o_stride[0] + (int64_t)h * p.o_stride[1] + d;
+    *reinterpret_cast<uint2 *>(op) = make_uint2(E::pack(t.x * inv, t.y * inv), E::pack(t.z * inv, t.w * inv));
+}
+
 // ------------------------------------------------------------------ host side
 // width of the lane layout and of a partial row: the head size, or 128 for the head sizes that are padded to it
 static int decode_tile_dim(const lazyattn_prefill_params &p) { return p.head_dim == 64 ? 64 : 128; }
@@ -618,7 +684,17 @@ int launch_decode_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
         if (f16) hipLaunchKernelGGL((paged_decode_merge_kernel<f16_t, HD, NB>), mgrid, dim3(256), 0, stream, m, nsplit); \
         else hipLaunchKernelGGL((paged_decode_merge_kernel<bf16_t, HD, NB>), mgrid, dim3(256), 0, stream, m, nsplit);    \
     }
-        if (p.head_dim == 64) {
+        if (nsplit > 8 && rows <= 512) {
+            // few rows, many slices: a workgroup per row
+            const dim3 wgrid((unsigned)rows);
+            if (p.head_dim == 64) {
+                if (f16) hipLaunchKernelGGL((paged_decode_merge_wide_kernel<f16_t, 64>), wgrid, dim3(256), 0, stream, m, nsplit);
+                else hipLaunchKernelGGL((paged_decode_merge_wide_kernel<bf16_t, 64>), wgrid, dim3(256), 0, stream, m, nsplit);
+            } else {
+                if (f16) hipLaunchKernelGGL((paged_decode_merge_wide_kernel<f16_t, 128>), wgrid, dim3(256), 0, stream, m, nsplit);
+                else hipLaunchKernelGGL((paged_decode_merge_wide_kernel<bf16_t, 128>), wgrid, dim3(256), 0, stream, m, nsplit);
+            }
+        } else if (p.head_dim == 64) {
             if (nsplit <= 8) LAZYATTN_DECODE_MERGE(64, 8) else LAZYATTN_DECODE_MERGE(64, 32)
         } else {
             if (nsplit <= 8) LAZYATTN_DECODE_MERGE(128, 8) else LAZYATTN_DECODE_MERGE(128, 32)
