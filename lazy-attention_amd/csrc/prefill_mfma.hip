@@ -22,6 +22,11 @@ struct MergeArgs {
     int32_t batch, token_grid;      // token_grid: the 32-token windows are cut over all tokens instead of per request
     int32_t head_dim;               // elements of an output row (below HD when the partial rows are padded)
     int32_t group, unit_cap;        // q-heads per kv-head; 32-row units per (request, kv-head) the main grid covers
+    // xcd_map: one-dimensional grid in which the workgroups of a (request, kv-head) go to the XCD whose L2 the main
+    // kernel's workgroups of that (request, kv-head) wrote the partial rows through (consecutive workgroup ids go
+    // round the eight XCDs; a hint only: any placement gives the same result)
+    int32_t xcd_map;
+    FastDiv by_group, by_windows, by_kv_heads;
 };
 // One workgroup = 32 consecutive tokens x one q-head; wave dt merges the columns dt*32 .. +31, lane (gh, l32) the
 // 4-column groups 8*i4 + 4*gh of token l32 -- the mapping of the main kernel's accumulators, so that a load
@@ -42,9 +47,21 @@ prefill_combine_kernel(const MergeArgs p, const int nsplit) {
     __shared__ __attribute__((aligned(16))) uint8_t tile[UNIT * ROW];
     __shared__ int row_ok[UNIT];
     const int lane = threadIdx.x & 63, dt = threadIdx.x >> 6, l32 = lane & 31, gh = lane >> 5;
-    const int h = (int)(blockIdx.x % (unsigned)p.num_q_heads);
-    const int64_t win = (int64_t)(blockIdx.x / (unsigned)p.num_q_heads) * UNIT;   // first token of the window
-    int b = blockIdx.y;
+    int h, b;
+    int64_t win;                                              // first token of the window
+    if (p.xcd_map) {
+        const uint32_t L = blockIdx.x, xcd = L & 7u, q = L >> 3;
+        const uint32_t t = p.by_group.quot(q), hh = p.by_group.rem(q, t);
+        const uint32_t r = p.by_windows.quot(t), w = p.by_windows.rem(t, r);
+        const uint32_t bg = r * 8u + xcd;                     // (request, kv-head): what the main kernel keeps on one XCD
+        b = (int)p.by_kv_heads.quot(bg);
+        h = (int)(p.by_kv_heads.rem(bg, (uint32_t)b) * (uint32_t)p.group + hh);
+        win = (int64_t)w * UNIT;
+    } else {
+        h = (int)(blockIdx.x % (unsigned)p.num_q_heads);
+        win = (int64_t)(blockIdx.x / (unsigned)p.num_q_heads) * UNIT;
+        b = blockIdx.y;
+    }
     bool valid = true;
     if (p.token_grid) {
         valid = win + l32 < load_index(p.b_start_loc, p.batch, p.index_bits);
@@ -261,12 +278,18 @@ int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
     if (nsplit > 1 && (phases & LAZYATTN_PHASE_COMBINE)) {
         // windows per request x requests, or windows over all tokens when that is at most half as many
         const int token_grid = p.batch > 1 && 2 * (int64_t)p.num_tokens <= (int64_t)p.batch * p.max_q_len;
-        const MergeArgs m{p.workspace, p.b_start_loc, p.b_seq_len, p.o, {p.o_stride[0], p.o_stride[1]}, p.num_tokens, p.num_q_heads,
-                          p.index_bits, p.skip_decode, p.batch, token_grid, p.head_dim, p.num_q_heads / p.num_kv_heads,
-                          mt_total > 0 ? 0x7fffffff : n_mt * nw};
         // 32 tokens x one q-head per workgroup
         const int64_t windows = ((int64_t)(token_grid ? p.num_tokens : p.max_q_len) + UNIT - 1) / UNIT;
-        const dim3 grid((unsigned)(windows * p.num_q_heads), token_grid ? 1 : p.batch);
+        const int group = p.num_q_heads / p.num_kv_heads;
+        // (the condition under which the main kernel gives a (request, kv-head) to one XCD)
+        const int xcd_map = !token_grid && mt_total == 0 && ((p.batch * p.num_kv_heads) & 7) == 0 &&
+                            windows * p.num_q_heads * p.batch <= 0x7fffffff;
+        const MergeArgs m{p.workspace, p.b_start_loc, p.b_seq_len, p.o, {p.o_stride[0], p.o_stride[1]}, p.num_tokens, p.num_q_heads,
+                          p.index_bits, p.skip_decode, p.batch, token_grid, p.head_dim, group,
+                          mt_total > 0 ? 0x7fffffff : n_mt * nw, xcd_map,
+                          FastDiv((uint32_t)group), FastDiv((uint32_t)windows), FastDiv((uint32_t)p.num_kv_heads)};
+        const dim3 grid = xcd_map ? dim3((unsigned)(windows * p.num_q_heads * p.batch))
+                                  : dim3((unsigned)(windows * p.num_q_heads), token_grid ? 1 : p.batch);
         const bool f16 = p.dtype == LAZYATTN_F16;
 #define LAZYATTN_COMBINE(HD, NB)                                                                                  \
     {                                                                                                             \
