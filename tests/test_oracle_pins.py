@@ -533,3 +533,28 @@ def test_reposition_blocks_equals_rotation_of_the_unrotated_keys():
     assert torch.allclose(got, want, atol=1e-9)
     assert torch.allclose(got.norm(dim=-1), raw.norm(dim=-1), atol=1e-9)
     assert torch.equal(vc[3], v_old) and torch.equal(kc[1].permute(2, 0, 1, 3).reshape(bs, hkv, d), stored)
+
+
+def test_reference_known_answers_from_the_golden_file():
+    """tests/golden/reference_known_answers.json holds what the reference's own unit tests assert about the metadata
+    path (inputs and expected outputs, with the lines they come from): the host function and the oracle's
+    restatement must both reproduce them."""
+    import json
+    import os
+    from lazy_amd.core.sched import metadata as host
+    with open(os.path.join(os.path.dirname(__file__), "golden", "reference_known_answers.json")) as f:
+        kat = json.load(f)
+    expand = lambda v: [v["repeat"]] * v["times"] if isinstance(v, dict) else v
+    for case in kat["metadata_for_lazy_attention"]:
+        want = (case["q_offset"], case["q_mask"])
+        args = (case["document_lens"], case["document_lens_padded"], case["block_size"])
+        assert host.metadata_for_lazy_attention(*args) == want, case["cite"]
+        assert tuple(list(map(int, x)) for x in orc.metadata_for_lazy_attention(*args)) == want, case["cite"]
+    for case in kat["metadata_for_mepic"]:
+        args = (case["document_lens"], case["document_lens_padded"], case["block_size"])
+        assert host.metadata_for_mepic(*args) == (case["q_offset"], case["q_mask"]), case["cite"]
+    for case in kat["max_rotation_offset"]:
+        assert host.max_rotation_offset(expand(case["document_lens"]), expand(case["document_lens_padded"])) == case["expected"], case["cite"]
+    for case in kat["packed_block_table"]:
+        packed = (case["block"] << 32) | (case["q_offset"] << 16) | case["q_mask"]
+        assert (packed >> 32) & 0xFFFFFFFF == case["unpacked_block"] and (packed >> 16) & 0xFFFF == case["unpacked_q_offset"]
