@@ -27,6 +27,7 @@ def chunked_prefill_paged_decode(query, key, value, output, kv_cache_dtype, key_
                                  is_mepic: bool = True, force_fp32_rotary: bool = False):
     # the counts that change from step to step are not part of the key: views [:n] of persistent buffers find the
     # call made for another n, and its structs are set to this call's counts
+    max_seq_len, max_query_len = int(max_seq_len or 0), int(max_query_len)      # (plain numbers from here on)
     batch, single = seq_lens.shape[0], seq_lens.shape[0] == 1
     counts = (batch, output.shape[0], max_seq_len, max_query_len)
     sig = _launch.call_key(

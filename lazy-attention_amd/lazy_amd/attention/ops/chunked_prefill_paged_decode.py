@@ -60,6 +60,7 @@ def chunked_prefill_paged_decode(query, key, value, output, kv_cache_dtype, key_
     compute = _env_flag("LAZY_DECODE_COMPUTE_COS_SIN")   # ops/chunked...:146-151
     # the counts that change from step to step are not part of the key: views [:n] of persistent buffers find the
     # call made for another n, and its structs are set to this call's counts
+    max_seq_len, max_query_len = int(max_seq_len or 0), int(max_query_len)      # (plain numbers from here on)
     batch, single = seq_lens.shape[0], seq_lens.shape[0] == 1
     counts = (batch, output.shape[0], max_seq_len, max_query_len)
     bound = (batch, block_table.shape[0])                # what a plan that owns batch-sized tensors stays tied to
