@@ -611,19 +611,28 @@ bool decode_mfma_supports(const lazyattn_prefill_params &p) {
     return true;
 }
 
-// slices of the page axis per (request, kv head): enough waves to fill the chip, at least twelve
-// pages (six loop iterations) per slice -- shorter slices cost more in prologue, partials and merge
-// than they gain in parallelism -- but down to five pages for a single request and ten for a handful, where
-// nothing else fills the chip (5 K keys, call = both launches: one request 16 / 32 / 64 slices 27.4 / 19.8 /
-// 18.0 us; four requests 30.0 / 23.3 / 26.1 us)
+// Slices of the page axis per (request, kv head).  A workgroup is four independent waves, one work item each; the
+// launch is fastest when its workgroups fit the chip's 256 CUs in one round with none left over -- a few CUs with a
+// second workgroup make the tail of the launch (32 requests of 5 K keys: 4 / 6 / 8 slices = 256 / 384 / 512
+// workgroups take 118 / 141 / 123 us; 12 requests: 8 / 12 / 16 slices = 192 / 288 / 384 workgroups 49 / 60 / 50 us) --
+// so: as many slices as keep the work items at or below 1 024, of at least five pages each (5 K keys, call = both
+// launches: one request 16 / 32 / 64 slices 27.4 / 19.8 / 13.7 us).
 static int decode_splits(const lazyattn_prefill_params &p) {
     if (p.num_splits > 0) return p.num_splits > 64 ? 64 : p.num_splits;
     const int64_t natural = (int64_t)p.batch * p.num_kv_heads * ((p.num_q_heads / p.num_kv_heads + 15) / 16);
     if (natural <= 0) return 1;
-    int64_t s = (256 * 8 + natural - 1) / natural;
+    // (or at or below two, three, four times as many -- whole rounds -- when that fills the rounds at least a tenth
+    // better: 48 requests = 384 items, 2 / 5 slices fill 75 % of one / 94 % of two rounds: 189 / 181 us)
+    const int64_t round = 256 * WAVES;
+    int64_t s = round / natural;
+    double fill = (double)(natural * s) / (double)round;
+    for (int64_t k = 2; k <= 4; ++k) {
+        const int64_t sk = k * round / natural;
+        const double fk = (double)(natural * sk) / (double)(k * round);
+        if (fk > fill * 1.1) { s = sk; fill = fk; }
+    }
     const int64_t pages = p.max_seq_len > 0 ? (p.max_seq_len + BS - 1) / BS : 64;
-    const int64_t min_pages = natural <= 8 ? 5 : natural <= 32 ? 10 : 12;
-    if (s > pages / min_pages) s = pages / min_pages;
+    if (s > pages / 5) s = pages / 5;
     if (s > 64) s = 64;
     return s < 1 ? 1 : (int)s;
 }
