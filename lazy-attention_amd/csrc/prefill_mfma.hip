@@ -216,7 +216,25 @@ static int mfma_splits(const lazyattn_prefill_params &p, int nw) {
     if (p.num_splits > 0) return p.num_splits > 64 ? 64 : p.num_splits;
     const int64_t natural = p.num_kv_heads * mfma_mtiles_estimate(p, nw);
     const int64_t ctx_tiles = p.max_seq_len > 0 ? (p.max_seq_len + NT - 1) / NT : 1;
-    int64_t s = (256 + natural - 1) / natural;        // one workgroup per CU
+    // One workgroup per CU and none left over: a CU holds one workgroup at a time, so a few workgroups beyond the
+    // chip's 256 CUs are a second round that most CUs sit out (3 requests of 128 new tokens over 5 K keys, 96
+    // workgroups per split: 2 / 3 splits = 192 / 288 workgroups take 55 / 77 us; 6 x 64 over 8 K, 48 per split:
+    // 5 / 6 splits 65 / 90 us).  Long workgroups (64 tiles and more) may take two to four whole rounds when that
+    // fills the rounds at least a fifth better (3 x 512 new tokens over 16 K keys, 192 per split: 1 / 4 splits =
+    // 75 % of one round / three full rounds: 448 / 427 us).
+    constexpr int64_t CUS = 256;
+    int64_t s = natural <= CUS ? CUS / natural : 1;
+    auto fill = [&](int64_t sp) {
+        const int64_t w = natural * sp, rounds = (w + CUS - 1) / CUS;
+        return (double)w / (double)(rounds * CUS);
+    };
+    if (ctx_tiles / s >= 64) {
+        double best = fill(s);
+        for (int64_t k = 2; k <= 4; ++k) {
+            const int64_t sk = k * CUS / natural;
+            if (sk > s && fill(sk) > best * 1.2) { s = sk; best = fill(sk); }
+        }
+    }
     if (s > ctx_tiles / 2) s = ctx_tiles / 2;        // at least two tiles per split
     if (s > 64) s = 64;
     return s < 1 ? 1 : (int)s;
