@@ -200,16 +200,24 @@ static bool mfma_compact(const lazyattn_prefill_params &p, int nw) {
     return p.batch > 1 && mfma_mtiles_bound(p, nw) * 2 <= (int64_t)p.batch * mfma_mtiles(p, nw);
 }
 
-// units (computing waves) per workgroup
+static int mfma_splits(const lazyattn_prefill_params &p, int nw);
+
+// units (computing waves) per workgroup: the shape with the lower estimated time.  Per workgroup a 64-key tile takes
+// about 1.34 us in the four-unit shape (128 rows) and 1.98 us in the eight-unit shape (256 rows: a third less per
+// row), a workgroup has some 8 us of launch, prologue, first-tile latency and epilogue, the workgroups run in rounds
+// of 256, and split partials cost about 2 us plus half a microsecond per split to write and merge.  (Measured on
+// this part with bf16 operands at head size 128; the other element types and head sizes shift both shapes alike.)
 static int mfma_waves(const lazyattn_prefill_params &p) {
     if (p.kernel == LAZYATTN_KERNEL_MFMA4) return 4;
     if (p.kernel == LAZYATTN_KERNEL_MFMA8) return 8;
-    const int units = mfma_units(p);
-    if (units <= 4) return 4;
-    // 64-key tiles of work per CU if the 8-unit kernel is used: small calls take the lighter one
-    const int64_t wgs8 = p.num_kv_heads * mfma_mtiles_estimate(p, 8);
+    if (mfma_units(p) <= 4) return 4;
     const int64_t tiles = p.max_seq_len > 0 ? (p.max_seq_len + NT - 1) / NT : 64;
-    return wgs8 * tiles >= 16 * 256 ? 8 : 4;
+    auto cost = [&](int nw, double tile_us) {
+        const int64_t s = mfma_splits(p, nw);
+        const int64_t wgs = p.num_kv_heads * mfma_mtiles_estimate(p, nw) * s, rounds = (wgs + 255) / 256;
+        return (double)rounds * ((double)((tiles + s - 1) / s) * tile_us + 8.0) + (s > 1 ? 2.0 + 0.5 * (double)s : 0.0);
+    };
+    return cost(8, 1.98) <= cost(4, 1.34) ? 8 : 4;
 }
 
 static int mfma_splits(const lazyattn_prefill_params &p, int nw) {
