@@ -22,7 +22,7 @@ SOURCES = ["prefill_mfma_bf16.hip", "prefill_mfma_bf16_e4m3.hip", "prefill_mfma_
 # No -ffast-math: the fp32 kernel needs IEEE expf/division and every kernel relies on
 # infinities; the MFMA kernel asks for hardware exp2 explicitly where it wants it.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17",
-         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-Wno-inline-asm"]
 
 
 def _compile(src: str, extra: list[str]) -> str:

@@ -47,13 +47,21 @@ constexpr int NT = 64;          // keys per tile
 constexpr int PAGES = NT / BS;  // pages per tile
 constexpr int UNIT = 32;        // query rows per wave
 // LDS tiles (bytes).  K: [page][d8 = 16][slot = 16][8 bf16].
-// V: [page][g = 2][d = 128][slots 4g..4g+3 | slots 8+4g..8+4g+3] -- the 16 bytes one lane
-// feeds to the PV MFMA as its A operand.
+// V: [page][d = 128][2 chunks of 8 slots] -- a cache page's own [d][16 slots] order, 32 bytes per row of d, with the
+// two 16-byte chunks of a row swapped where bit 3 of d is set (so that lanes writing both chunks of their own row, as
+// the fp8 conversion does, spread over all banks).  A chunk is the 16 bytes one lane feeds to the PV MFMA as its A
+// operand: the computing waves read K slot s of a page as MFMA row (s with bits 2 and 3 swapped), which puts the
+// scores of slots 8*gh .. 8*gh+7 of a page into one lane's accumulator registers -- chunk gh of the V rows.
+// A V tile in LDS is therefore a byte-for-byte copy of four cache pages, and full pages of 16-bit caches go there by
+// global -> LDS loads that pass through no register.
+// V has three buffers (the loads of tile t+2 land while tile t is read and tile t+1 waits), K two (its way leads
+// through the gathering waves' registers, which are the third stage).
 // Sizes that follow from the head size HD (128 or 64); a K page is HD * 32 bytes, a V page as well.
 template <int HD> struct Geo {
     static constexpr int K_PAGE = HD * 32, K_TILE = PAGES * K_PAGE;
-    static constexpr int V_G = HD * 16, V_PAGE = 2 * V_G, V_TILE = PAGES * V_PAGE;
-    static constexpr int KV_BYTES = 2 * K_TILE + 2 * V_TILE;      // K and V tiles, double-buffered: 64 KB at 128
+    static constexpr int V_PAGE = HD * 32, V_TILE = PAGES * V_PAGE;
+    static constexpr int V_BUFS = 3;
+    static constexpr int KV_BYTES = 2 * K_TILE + V_BUFS * V_TILE; // V tiles (first: low LDS addresses), then K tiles: 80 KB at 128
     static constexpr int Q_WAVE = HD * 64;                        // Q^T fragments of one computing wave
     static constexpr int KS = HD / 16, DT = HD / 32;              // k-steps of K.Q^T, 32-row blocks of O^T
     static constexpr int K_ITEMS = HD / 64, V_ITEMS = HD / 32;    // 16-byte items per gathering lane and page
@@ -81,38 +89,70 @@ __device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirs
 struct MfmaDivs { FastDiv n_mt, nsplit, kv_heads, group; };
 
 
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
 __device__ __forceinline__ uint4 ldg16(const uint8_t *base, uint32_t off) {
     return *reinterpret_cast<const uint4 *>(base + off);
+}
+__device__ __forceinline__ u32x4_t ldg16v(const uint8_t *base, uint32_t off) {
+    return *reinterpret_cast<const u32x4_t *>(base + off);
 }
 __device__ __forceinline__ uint2 ldg8(const uint8_t *base, uint32_t off) {
     return *reinterpret_cast<const uint2 *>(base + off);
 }
+// The same 16-byte load, written as asm: the compiler does not count it among the loads it waits for, and takes the
+// value to be there at once.  Whoever uses this owns the wait: settle() below, before anything reads `dst`.
+__device__ __forceinline__ void ldg16_uncounted(u32x4_t &dst, const uint8_t *sbase, uint32_t voff) {
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(dst) : "v"(voff), "s"(sbase) : "memory");
+}
+__device__ __forceinline__ void ldg16_uncounted_hi(u32x4_t &dst, const uint8_t *sbase, uint32_t voff) {
+    asm volatile("global_load_dwordx4 %0, %1, %2 offset:16" : "=v"(dst) : "v"(voff), "s"(sbase) : "memory");
+}
+// 16 bytes per lane from global memory straight into LDS: lane i's bytes (scalar base + its own 32-bit offset) go to
+// lds_addr + i * 16.  m0 carries the LDS address; a scalar write of m0 needs one wait state before such a load reads it.
+__device__ __forceinline__ void dma16(const uint8_t *sbase, uint32_t voff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0" : : "s"(sbase), "v"(voff), "s"(lds_addr) : "memory", "m0");
+}
+// wait until at most N of this wave's vector memory loads are outstanding (they complete in order)
+template <int N> __device__ __forceinline__ void wait_vmem() { asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory"); }
 
 // 8 consecutive cos (or sin) table entries
 template <typename TT> struct TabVec {                     // a 16-bit table
-    uint4 v;
-    __device__ __forceinline__ void load(const uint8_t *base, uint32_t off) { v = ldg16(base, off); }
-    __device__ __forceinline__ void fill(float w) { const uint32_t u = Elem<TT>::splat(w); v = make_uint4(u, u, u, u); }
+    u32x4_t v;
+    static constexpr int LOADS = 1;
+    __device__ __forceinline__ void load(const uint8_t *base, uint32_t off) { v = ldg16v(base, off); }
+    __device__ __forceinline__ void load_uncounted(const uint8_t *base, uint32_t off) { ldg16_uncounted(v, base, off); }
+    __device__ __forceinline__ void fill(float w) { const uint32_t u = Elem<TT>::splat(w); v = u32x4_t{u, u, u, u}; }
     __device__ __forceinline__ void get(float *f) const {
-        f[0] = Elem<TT>::lo(v.x); f[1] = Elem<TT>::hi(v.x); f[2] = Elem<TT>::lo(v.y); f[3] = Elem<TT>::hi(v.y);
-        f[4] = Elem<TT>::lo(v.z); f[5] = Elem<TT>::hi(v.z); f[6] = Elem<TT>::lo(v.w); f[7] = Elem<TT>::hi(v.w);
+        f[0] = Elem<TT>::lo(v[0]); f[1] = Elem<TT>::hi(v[0]); f[2] = Elem<TT>::lo(v[1]); f[3] = Elem<TT>::hi(v[1]);
+        f[4] = Elem<TT>::lo(v[2]); f[5] = Elem<TT>::hi(v[2]); f[6] = Elem<TT>::lo(v[3]); f[7] = Elem<TT>::hi(v[3]);
     }
 };
 template <> struct TabVec<float> {
-    float4 a, b;
+    u32x4_t a, b;
+    static constexpr int LOADS = 2;
     __device__ __forceinline__ void load(const uint8_t *base, uint32_t off) {
-        a = *reinterpret_cast<const float4 *>(base + off);
-        b = *reinterpret_cast<const float4 *>(base + off + 16);
+        a = ldg16v(base, off);
+        b = ldg16v(base, off + 16);
     }
-    __device__ __forceinline__ void fill(float w) { a = make_float4(w, w, w, w); b = a; }
+    __device__ __forceinline__ void load_uncounted(const uint8_t *base, uint32_t off) {
+        ldg16_uncounted(a, base, off);
+        ldg16_uncounted_hi(b, base, off);
+    }
+    __device__ __forceinline__ void fill(float w) { const uint32_t u = __float_as_uint(w); a = u32x4_t{u, u, u, u}; b = a; }
     __device__ __forceinline__ void get(float *f) const {
-        f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { f[i] = __uint_as_float(a[i]); f[4 + i] = __uint_as_float(b[i]); }
     }
 };
 
 template <typename T> __device__ __forceinline__ void unpack8(const uint4 &w, float *f) {
     f[0] = Elem<T>::lo(w.x); f[1] = Elem<T>::hi(w.x); f[2] = Elem<T>::lo(w.y); f[3] = Elem<T>::hi(w.y);
     f[4] = Elem<T>::lo(w.z); f[5] = Elem<T>::hi(w.z); f[6] = Elem<T>::lo(w.w); f[7] = Elem<T>::hi(w.w);
+}
+template <typename T> __device__ __forceinline__ void unpack8(const u32x4_t &w, float *f) {
+    f[0] = Elem<T>::lo(w[0]); f[1] = Elem<T>::hi(w[0]); f[2] = Elem<T>::lo(w[1]); f[3] = Elem<T>::hi(w[1]);
+    f[4] = Elem<T>::lo(w[2]); f[5] = Elem<T>::hi(w[2]); f[6] = Elem<T>::lo(w[3]); f[7] = Elem<T>::hi(w[3]);
 }
 // two fp8 bytes (the low 16 bits of w) -> two floats; KIND 1: e4m3, 2: e5m2
 template <int KIND> __device__ __forceinline__ f32x2_t cvt_fp8x2(uint32_t w) {
@@ -147,10 +187,18 @@ template <typename T, int KIND> __device__ __forceinline__ void unpack8_fp8(uint
 
 // one K item in flight: 8 (d, d+64) pairs of one key
 template <typename TT> struct KRegs {
-    uint4 k1, k2;
+    u32x4_t k1, k2;
     TabVec<TT> c, s;
     uint32_t lds_off;
 };
+// Wait until at most N vector memory loads of this wave are outstanding; the item's registers count as written
+// here, so that nothing that reads them can be placed before the wait.
+template <int N> __device__ __forceinline__ void settle(KRegs<float> &r) {
+    asm volatile("s_waitcnt vmcnt(%6)" : "+v"(r.k1), "+v"(r.k2), "+v"(r.c.a), "+v"(r.c.b), "+v"(r.s.a), "+v"(r.s.b) : "n"(N) : "memory");
+}
+template <int N, typename TT> __device__ __forceinline__ void settle(KRegs<TT> &r) {
+    asm volatile("s_waitcnt vmcnt(%4)" : "+v"(r.k1), "+v"(r.k2), "+v"(r.c.v), "+v"(r.s.v) : "n"(N) : "memory");
+}
 
 }  // namespace
 
@@ -182,7 +230,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     using G = Geo<HD>;
     constexpr int D = HD, HALF = HD / 2;
     const int Dr = PAD ? p.head_dim : D, HALFr = Dr / 2, CPr = Dr / 16;   // real head size, its half, its chunk pairs
-    constexpr int K_PAGE = G::K_PAGE, K_TILE = G::K_TILE, V_G = G::V_G, V_PAGE = G::V_PAGE, V_TILE = G::V_TILE;
+    constexpr int K_PAGE = G::K_PAGE, K_TILE = G::K_TILE, V_PAGE = G::V_PAGE, V_TILE = G::V_TILE, V_BUFS = G::V_BUFS;
     constexpr int KV_BYTES = G::KV_BYTES, KS = G::KS, DT = G::DT;
     // a page has HD K items (HD/16 chunk pairs x 16 slots) and 2 HD V items (an fp8 page row of 16 slots is one
     // 16-byte item): per lane of the NH gathering waves that share the page.  Item i of a wave's registers is item
@@ -325,11 +373,12 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     // serves all of them and the strides go into the scalar page base.
     // K bf16: [D/8][slots][8] -> item (cp, o) at (cp*slots + o)*16 bytes, cp = lane/16 + 4 i
     //   fp8 : [D/16][slots][16] -> 8 bytes at chunk cp/2, half cp&1
-    // V bf16: row d = lane/2 + 32 i of `slots` slots, 8 slots (16 bytes) per item; fp8: row d = lane + 64 i, 16 slots
+    // V bf16: item = one 16-byte chunk of a row, in the order the chunks take in LDS (position lane + 64 i: row
+    //   d = position / 2, chunk = (position & 1) ^ bit 3 of d); fp8: row d = lane + 64 i, 16 slots
     uint32_t k_goff = FP8 ? (uint32_t)(((lane >> 5) * cache_bs + slot0 + (lane & 15)) * 16 + ((lane >> 4) & 1) * 8)
                           : (uint32_t)(((lane >> 4) * cache_bs + slot0 + (lane & 15)) * 16);
     uint32_t v_goff = FP8 ? (uint32_t)(lane * cache_bs + slot0)
-                          : (uint32_t)((lane >> 1) * cache_bs * 2 + slot0 * 2 + (lane & 1) * 16);
+                          : (uint32_t)((lane >> 1) * cache_bs * 2 + slot0 * 2 + ((lane ^ (lane >> 4)) & 1) * 16);
 #pragma unroll
     for (int i = 0; i < KI; ++i) {
         const int idx = lane + item(i) * 64;
@@ -357,7 +406,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             const int d = FP8 ? idx : idx >> 1;
             pv_ok[i] = d < Dr;
             const int dc = pv_ok[i] ? d : 0;
-            pv[i] = FP8 ? (uint32_t)(dc * cache_bs + slot0) : (uint32_t)(dc * cache_bs * 2 + slot0 * 2 + (idx & 1) * 16);
+            pv[i] = FP8 ? (uint32_t)(dc * cache_bs + slot0) : (uint32_t)(dc * cache_bs * 2 + slot0 * 2 + ((idx ^ (idx >> 4)) & 1) * 16);
         }
     }
     // (pinned here: the values are only used by the gathering waves' code further down, and the compiler would
@@ -511,28 +560,37 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             const uint8_t *kb = pb.kb;
             kr[i].lds_off = (uint32_t)(gw * K_PAGE + (lane + item(i) * 64) * 16);
             if constexpr (PAD) {
-                uint4 k1, k2;
+                u32x4_t k1, k2;
                 if (FP8) {
                     const uint2 a = ldg8(kb, pk1[i]), a2 = ldg8(kb, pk2[i]);
-                    k1 = make_uint4(a.x, a.y, 0, 0);
-                    k2 = make_uint4(a2.x, a2.y, 0, 0);
+                    k1 = u32x4_t{a.x, a.y, 0, 0};
+                    k2 = u32x4_t{a2.x, a2.y, 0, 0};
                 } else {
-                    k1 = ldg16(kb, pk1[i]);
-                    k2 = ldg16(kb, pk2[i]);
+                    k1 = ldg16v(kb, pk1[i]);
+                    k2 = ldg16v(kb, pk2[i]);
                 }
-                const uint4 z = make_uint4(0, 0, 0, 0);
+                const u32x4_t z = {0, 0, 0, 0};
                 kr[i].k1 = pk_ok[i] ? k1 : z;
                 kr[i].k2 = pk_ok[i] ? k2 : z;
             } else if (FP8) {
                 const uint2 a = ldg8(kb + item(i) * k_item, pb.ko), a2 = ldg8(kb + item(i) * k_item + pair, pb.ko);
-                kr[i].k1 = make_uint4(a.x, a.y, 0, 0);
-                kr[i].k2 = make_uint4(a2.x, a2.y, 0, 0);
+                kr[i].k1 = u32x4_t{a.x, a.y, 0, 0};
+                kr[i].k2 = u32x4_t{a2.x, a2.y, 0, 0};
             } else {
-                kr[i].k1 = ldg16(kb + item(i) * k_item, pb.ko);
-                kr[i].k2 = ldg16(kb + item(i) * k_item + pair, pb.ko);
+                kr[i].k1 = ldg16v(kb + item(i) * k_item, pb.ko);
+                kr[i].k2 = ldg16v(kb + item(i) * k_item + pair, pb.ko);
             }
             kr[i].c.load(pb.tb, pb.to[i]);
             kr[i].s.load(pb.ts, pb.to[i]);
+        };
+        // the same four loads (full page of a 16-bit cache) outside the compiler's count: the steady state below
+        // places its own waits, because the V loads that go straight to LDS are outside that count anyway
+        auto load_k_item_uncounted = [&](int i, const PageBase &pb) {
+            kr[i].lds_off = (uint32_t)(gw * K_PAGE + (lane + item(i) * 64) * 16);
+            ldg16_uncounted(kr[i].k1, pb.kb + item(i) * k_item, pb.ko);
+            ldg16_uncounted(kr[i].k2, pb.kb + item(i) * k_item + pair, pb.ko);
+            kr[i].c.load_uncounted(pb.tb, pb.to[i]);
+            kr[i].s.load_uncounted(pb.ts, pb.to[i]);
         };
         auto load_v_item = [&](int i, const PageBase &pb) {
             if constexpr (PAD) {
@@ -557,13 +615,13 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                 const int idx = lane + item(i) * 64;
                 const int cp = idx & (D / 16 - 1), kl = idx / (D / 16), m = m0 + kl;
                 kr[i].lds_off = (uint32_t)(gw * K_PAGE + cp * 256 + kl * 16);
-                uint4 k1 = make_uint4(0, 0, 0, 0), k2 = k1;
+                u32x4_t k1 = {0, 0, 0, 0}, k2 = k1;
                 TabVec<TT> c, sn;
                 c.fill(1.f); sn.fill(0.f);
                 if (m < t_end && (!PAD || cp < CPr)) {
                     const T *kn = (const T *)p.k + (qs + m) * p.k_stride[0] + (int64_t)g * p.k_stride[1] + cp * 8;
-                    k1 = *reinterpret_cast<const uint4 *>(kn);
-                    k2 = *reinterpret_cast<const uint4 *>(kn + HALFr);
+                    k1 = *reinterpret_cast<const u32x4_t *>(kn);
+                    k2 = *reinterpret_cast<const u32x4_t *>(kn + HALFr);
                     if (rot_new) {                                               // old_ops:342-343
                         const uint8_t *tb = tab_base + (int64_t)(ctx_len + m) * row_bytes;
                         c.load(tb, (uint32_t)cp * 8 * TSZ);
@@ -592,7 +650,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             if (pm.lim == BS) return TILE_FULL;
             if (tile * PAGES + gw >= n_pages) {
 #pragma unroll
-                for (int i = 0; i < KI; ++i) { kr[i].k1 = make_uint4(0, 0, 0, 0); kr[i].k2 = kr[i].k1; }
+                for (int i = 0; i < KI; ++i) { kr[i].k1 = u32x4_t{0, 0, 0, 0}; kr[i].k2 = kr[i].k1; }
             }
             return TILE_EDGE;
         };
@@ -600,11 +658,11 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         auto store_k_item = [&](int i, uint8_t *ktile, int kind) {
             float a[8], bb[8], cs[8], sn[8];
             if (FOLD && kind != TILE_NEW) {
-                unpack8_fp8_raw<FP8>(kr[i].k1.x, kr[i].k1.y, a);
-                unpack8_fp8_raw<FP8>(kr[i].k2.x, kr[i].k2.y, bb);
+                unpack8_fp8_raw<FP8>(kr[i].k1[0], kr[i].k1[1], a);
+                unpack8_fp8_raw<FP8>(kr[i].k2[0], kr[i].k2[1], bb);
             } else if (FP8 && kind != TILE_NEW) {
-                unpack8_fp8<T, FP8>(kr[i].k1.x, kr[i].k1.y, k_scale, a);
-                unpack8_fp8<T, FP8>(kr[i].k2.x, kr[i].k2.y, k_scale, bb);
+                unpack8_fp8<T, FP8>(kr[i].k1[0], kr[i].k1[1], k_scale, a);
+                unpack8_fp8<T, FP8>(kr[i].k2[0], kr[i].k2[1], k_scale, bb);
             } else {
                 unpack8<T>(kr[i].k1, a);
                 unpack8<T>(kr[i].k2, bb);
@@ -630,14 +688,15 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
 #pragma unroll
             for (int i = 0; i < KI; ++i) store_k_item(i, ktile, kind);
         };
-        // one V item of a context page (16 bytes of one row of d) -> its two 8-byte LDS entries
+        // one V item of a context page -> the page's rows in LDS ([d][2 chunks of 8 slots], chunks swapped where bit 3
+        // of d is set)
         auto store_v_item = [&](int i, uint8_t *vtile, int kind, int lim) {
             const int idx = lane + item(i) * 64;
             if (FP8) {
-                // 16 fp8 slots of one d: entry g=0 <- slots 0-3 | 8-11, entry g=1 <- slots 4-7 | 12-15
+                // 16 fp8 slots of one d -> both chunks of its row
                 const int d = idx;
                 const uint32_t w[4] = {vr[i].x, vr[i].y, vr[i].z, vr[i].w};
-                uint32_t o2[4][2];
+                uint32_t o2[4][2];                               // o2[q][h]: slots 4q + 2h, 4q + 2h + 1
 #pragma unroll
                 for (int q4 = 0; q4 < 4; ++q4) {
                     if constexpr (FOLD) {
@@ -661,12 +720,13 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                     o2[q4][0] = E::pack(f[0], f[1]);
                     o2[q4][1] = E::pack(f[2], f[3]);
                 }
-                uint8_t *dst = vtile + gw * V_PAGE + d * 16;
-                *reinterpret_cast<uint4 *>(dst) = make_uint4(o2[0][0], o2[0][1], o2[2][0], o2[2][1]);
-                *reinterpret_cast<uint4 *>(dst + V_G) = make_uint4(o2[1][0], o2[1][1], o2[3][0], o2[3][1]);
+                uint8_t *dst = vtile + gw * V_PAGE + d * 32;
+                const int sw = ((d >> 3) & 1) * 16;
+                *reinterpret_cast<uint4 *>(dst + sw) = make_uint4(o2[0][0], o2[0][1], o2[1][0], o2[1][1]);
+                *reinterpret_cast<uint4 *>(dst + (sw ^ 16)) = make_uint4(o2[2][0], o2[2][1], o2[3][0], o2[3][1]);
             } else {
-                // 8 bf16 slots (8*hf ..) of one d: slots +0..3 -> entry g=0, +4..7 -> entry g=1, half hf
-                const int d = idx >> 1, hf = idx & 1;
+                // 8 slots (8*hf ..) of one d, already the chunk that belongs at position idx
+                const int hf = (idx ^ (idx >> 4)) & 1;
                 uint4 v = vr[i];
                 if (kind == TILE_EDGE) {
                     uint32_t w[4] = {v.x, v.y, v.z, v.w};
@@ -677,9 +737,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                     }
                     v = make_uint4(w[0], w[1], w[2], w[3]);
                 }
-                uint8_t *dst = vtile + gw * V_PAGE + d * 16 + hf * 8;
-                *reinterpret_cast<uint2 *>(dst) = make_uint2(v.x, v.y);
-                *reinterpret_cast<uint2 *>(dst + V_G) = make_uint2(v.z, v.w);
+                *reinterpret_cast<uint4 *>(vtile + gw * V_PAGE + idx * 16) = v;
             }
         };
         // ---- write the V items to a V tile; lim = valid slots of the page ----
@@ -690,8 +748,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                 for (int i = 0; i < VI; ++i) {
                     const int idx = lane + item(i) * 64;
                     const int dc = idx & (D / 8 - 1), slot = idx / (D / 8);
-                    uint8_t *dst = vtile + gw * V_PAGE + ((slot >> 2) & 1) * V_G + (dc * 8) * 16 + (slot >> 3) * 8 +
-                                   (slot & 3) * 2;
+                    uint8_t *dst = vtile + gw * V_PAGE + (dc * 8) * 32 + (((slot >> 3) ^ dc) & 1) * 16 + (slot & 7) * 2;
                     uint32_t w[4] = {vr[i].x, vr[i].y, vr[i].z, vr[i].w};
                     if constexpr (FOLD) {
 #pragma unroll
@@ -699,8 +756,8 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                     }
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        *reinterpret_cast<uint16_t *>(dst + (2 * e) * 16) = (uint16_t)(w[e] & 0xffffu);
-                        *reinterpret_cast<uint16_t *>(dst + (2 * e + 1) * 16) = (uint16_t)(w[e] >> 16);
+                        *reinterpret_cast<uint16_t *>(dst + (2 * e) * 32) = (uint16_t)(w[e] & 0xffffu);
+                        *reinterpret_cast<uint16_t *>(dst + (2 * e + 1) * 32) = (uint16_t)(w[e] >> 16);
                     }
                 }
                 return;
@@ -708,17 +765,41 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
 #pragma unroll
             for (int i = 0; i < VI_CTX; ++i) store_v_item(i, vtile, kind, lim);
         };
-        // tile + its page limit -> LDS buffer `buf`
-        auto store_tile = [&](int buf, int kind, int lim) {
-            store_k(lds + buf * K_TILE, kind);
-            store_v(lds + 2 * K_TILE + buf * V_TILE, kind, lim);
-            if (lane == 0 && half == 0) page_lims[buf * PAGES + gw] = (uint8_t)lim;
+        uint8_t *const kt0 = lds + V_BUFS * V_TILE;             // the two K tiles follow the three V tiles
+        // K tile + the page's limit -> K buffer `kbuf`; V (unless it is already on its way there) -> V buffer `vb`
+        auto store_tile = [&](int kbuf, int vb, int kind, int lim, bool with_v) {
+            store_k(kt0 + kbuf * K_TILE, kind);
+            if (with_v) store_v(lds + vb * V_TILE, kind, lim);
+            if (lane == 0 && half == 0) page_lims[kbuf * PAGES + gw] = (uint8_t)lim;
         };
+        // Full pages of a 16-bit cache need nothing done to V: their bytes go from the cache to the V tile by
+        // global -> LDS loads (lane i of a load brings 16 bytes to i * 16 of a 1 KB stretch; which 16 bytes, is the
+        // lane's own offset).  They are written as asm, outside the compiler's count of loads in flight: counted,
+        // every later LDS store of this wave would be made to wait for them.  The steady state therefore issues its
+        // K loads the same way and places the waits itself.  Loads complete in order; per tile the wave issues
+        //   K item 0 (LPI loads) | V (VI loads) | K items 1 .. KI-1
+        // so when item i of the next tile is needed, (KI-1) * LPI + VI younger loads have been issued since, and when
+        // V of the next tile must have landed (the barrier at the end of the tile after the one it was issued in),
+        // (2 KI - 1) * LPI + VI.
+        constexpr bool VDMA = !FP8 && !PAD;
+        const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
+        auto dma_v = [&](const PageBase &pb, int vb) {
+#pragma unroll
+            for (int i = 0; i < VI; ++i)
+                dma16(pb.vb + item(i) * v_item, pb.vo, lds0 + (uint32_t)(vb * V_TILE + gw * V_PAGE + item(i) * 1024));
+        };
+        constexpr int LPI = 2 + 2 * TabVec<TT>::LOADS;
+        constexpr int ITEM_YOUNGER = (KI - 1) * LPI + VI, V_YOUNGER = (2 * KI - 1) * LPI + VI;
+        static_assert(V_YOUNGER < 64, "the wait counter holds 6 bits");
 
         // At the top of iteration `tile` the raw K/V of tile+1 sit in registers (loaded during
         // the previous iteration); they are rotated into the other LDS buffer while the
-        // computing waves work on `tile`, then the loads of tile+2 are issued.
+        // computing waves work on `tile`, then the loads of tile+2 are issued.  V buffers go round in threes:
+        // vcur holds V of `tile`.
         int nxt_kind = TILE_FULL, nxt_lim = BS;
+        int vcur = 0;
+        bool v_sent = false;                 // V of tile+1 went (or is going) straight to its LDS buffer
+        auto vnext = [](int v) { return v == V_BUFS - 1 ? 0 : v + 1; };
         if (tile_begin < tile_end) {
             const int k0 = issue_loads(tile_begin, pm0);
             if (k0 == TILE_FULL && tile_begin + 1 < n_ctx_tiles && tile_begin + 1 < tile_end && pm1.lim == BS) {
@@ -726,7 +807,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                 // into the registers its counterpart of the first has just left, so the requests pass through the
                 // CU's memory pipeline while the first tile is rotated instead of in one burst before the barrier
                 const PageBase pb = page_base(tile_begin + 1, pm1);
-                uint8_t *kt = lds, *vt = lds + 2 * K_TILE;
+                uint8_t *kt = kt0, *vt = lds;
 #pragma unroll
                 for (int i = 0; i < KI; ++i) {
                     store_k_item(i, kt, TILE_FULL);
@@ -741,7 +822,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                 }
                 if (lane == 0 && half == 0) page_lims[gw] = (uint8_t)BS;
             } else {
-                store_tile(0, k0, pm0.lim);
+                store_tile(0, 0, k0, pm0.lim, true);
                 if (tile_begin + 1 < tile_end) {
                     nxt_kind = issue_loads(tile_begin + 1, pm1);
                     nxt_lim = pm1.lim;
@@ -760,33 +841,66 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                 // pipeline spread over the tile instead of in one burst at its end (in a burst each of the twelve
                 // loads of a wave waited tens of cycles to be accepted, all of it on this wave's critical path).
                 const PageBase pb = page_base(tile + 2, pm_pend);
-                uint8_t *kt = lds + (cur ^ 1) * K_TILE, *vt = lds + 2 * K_TILE + (cur ^ 1) * V_TILE;
+                const int vn = vnext(vcur), vnn = vnext(vn);
+                uint8_t *kt = kt0 + (cur ^ 1) * K_TILE, *vt = lds + vn * V_TILE;
+                if constexpr (VDMA) {
+                    if (!v_sent) {
+                        // first round: K and V of tile+1 came through counted loads; V leaves its registers first,
+                        // while the compiler's count is still right
 #pragma unroll
-                for (int i = 0; i < KI; ++i) {
-                    store_k_item(i, kt, TILE_FULL);
-                    load_k_item(i, pb);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
+                        for (int i = 0; i < VI_CTX; ++i) store_v_item(i, vt, TILE_FULL, BS);
+                    }
 #pragma unroll
-                for (int i = 0; i < VI_CTX; ++i) {
-                    store_v_item(i, vt, TILE_FULL, BS);
-                    load_v_item(i, pb);
-                    __builtin_amdgcn_sched_barrier(0);
+                    for (int i = 0; i < KI; ++i) {
+                        settle<ITEM_YOUNGER>(kr[i]);
+                        store_k_item(i, kt, TILE_FULL);
+                        load_k_item_uncounted(i, pb);
+                        __builtin_amdgcn_sched_barrier(0);
+                        // V of tile+2 sets out behind the first K item's loads: it has this tile and the next to land
+                        if (i == 0) {
+                            dma_v(pb, vnn);
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
+                    if (v_sent) wait_vmem<V_YOUNGER>();                      // V of tile+1 has landed
+                    v_sent = true;
+                } else {
+#pragma unroll
+                    for (int i = 0; i < KI; ++i) {
+                        store_k_item(i, kt, TILE_FULL);
+                        load_k_item(i, pb);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+#pragma unroll
+                    for (int i = 0; i < VI_CTX; ++i) {
+                        store_v_item(i, vt, TILE_FULL, BS);
+                        load_v_item(i, pb);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                 }
                 if (lane == 0 && half == 0) page_lims[(cur ^ 1) * PAGES + gw] = (uint8_t)BS;
                 pm_pend = pm_new;
                 ++tile;
+                vcur = vn;
                 __syncthreads();
             }
             if (tile >= tile_end) break;
             const int cur = (tile - tile_begin) & 1;
-            if (tile + 1 < tile_end) store_tile(cur ^ 1, nxt_kind, nxt_lim);
+            const int vn = vnext(vcur);
+            if (v_sent) {
+                // out of the steady state: K of tile+1 is in flight uncounted, V on its way to LDS; nothing else
+#pragma unroll
+                for (int i = 0; i < KI; ++i) settle<0>(kr[i]);
+            }
+            if (tile + 1 < tile_end) store_tile(cur ^ 1, vn, nxt_kind, nxt_lim, !v_sent);
+            v_sent = false;
             int new_kind = TILE_FULL;
             if (tile + 2 < tile_end) new_kind = issue_loads(tile + 2, pm_pend);
             nxt_kind = new_kind;
             nxt_lim = pm_pend.lim;
             pm_pend = load_page((tile + 3) * PAGES + gw);
             ++tile;
+            vcur = vn;
             __syncthreads();
         }
         return;
@@ -859,7 +973,10 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     // step ks in the instruction stream: the wave runs it while the matrix pipe works (the exponentials of the
     // other half, see the tile loop).
     auto qk_half = [&](const uint8_t *ktile, int sub, f32x16_t &s, auto between) {
-        const uint8_t *kp = ktile + (sub * 2 + (l32 >> 4)) * K_PAGE + gh * 256 + (l32 & 15) * 16;
+        // MFMA row l32 takes slot (l32 with bits 2 and 3 swapped) of page l32 / 16: a lane's accumulator registers
+        // then hold the scores of slots 8*gh .. 8*gh+7 of each page, the order of a V row's chunk gh
+        const int kslot = (l32 & 3) | ((l32 & 4) << 1) | ((l32 & 8) >> 1);
+        const uint8_t *kp = ktile + (sub * 2 + (l32 >> 4)) * K_PAGE + gh * 256 + kslot * 16;
         uint4 a[3], q[QREG ? 1 : 3];
         auto fetch = [&](int ks) {
             a[ks % 3] = *reinterpret_cast<const uint4 *>(kp + ks * 512);
@@ -876,17 +993,17 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    // ---- masks: register i of half `sub` holds key sub*32 + 8*(i/4) + 4*gh + i%4 ----
+    // ---- masks: register i of half `sub` holds key sub*32 + 16*(i/8) + 8*gh + i%8 ----
     // key0 = sequence position of the tile's first key (only used under a sliding window)
     auto mask_half = [&](f32x16_t &s, uint32_t vbits, int sub, int kind, int m0, int key0) {
-        const uint32_t w = vbits >> (4 * gh);
-        // causal: key m0 + kk <= row  <=>  8*(i/4) + i%4 <= row - m0 - sub*32 - 4*gh   (old_ops:371-372)
-        const int lim = kind == TILE_NEW ? row - m0 - sub * 32 - 4 * gh : 64;
-        // window: key0 + sub*32 + 4*gh + kb >= ctx_len + row - window + 1
-        const int lb = window ? ctx_len + row - window + 1 - key0 - sub * 32 - 4 * gh : -64;
+        const uint32_t w = vbits >> (8 * gh);
+        // causal: key m0 + kk <= row  <=>  16*(i/8) + i%8 <= row - m0 - sub*32 - 8*gh   (old_ops:371-372)
+        const int lim = kind == TILE_NEW ? row - m0 - sub * 32 - 8 * gh : 64;
+        // window: key0 + sub*32 + 8*gh + kb >= ctx_len + row - window + 1
+        const int lb = window ? ctx_len + row - window + 1 - key0 - sub * 32 - 8 * gh : -64;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            const int kb = 8 * (i >> 2) + (i & 3);
+            const int kb = 16 * (i >> 3) + (i & 7);
             const bool ok = ((w >> kb) & 1u) && kb <= lim && (!WIN || kb >= lb);
             s[i] = ok ? s[i] : -INFINITY;
         }
@@ -956,14 +1073,14 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         for (int i = 0; i < 8; ++i) exp_piece(s, h, i);
     };
     // ---- O^T += V^T . P^T for 32 keys (pages 2*sub, 2*sub+1 of the tile) ----
-    // k index j of a 16-key step <-> slot 4*gh + j (j < 4), 8 + 4*gh + j - 4 (j >= 4)
+    // k index j of a 16-key step <-> slot 8*gh + j of the page: chunk gh of every row of d, as it lies in the cache
     auto pv_half = [&](const uint8_t *vtile, int sub, const HalfP &h, auto between) {
-        const uint8_t *vp = vtile + (sub * 2) * V_PAGE + gh * V_G + l32 * 16;
+        const uint8_t *vp = vtile + (sub * 2) * V_PAGE + l32 * 32 + ((gh ^ (l32 >> 3)) & 1) * 16;
         const uint4 p0 = make_uint4(h.w[0], h.w[1], h.w[2], h.w[3]), p1 = make_uint4(h.w[4], h.w[5], h.w[6], h.w[7]);
         // 2 DT MFMAs: the 32-row blocks of d for the first page of the half, then for the second;
         // their V^T operands are requested two MFMAs ahead
         uint4 a[3];
-        auto fetch = [&](int j) { a[j % 3] = *reinterpret_cast<const uint4 *>(vp + (j / DT) * V_PAGE + (j % DT) * 512); };
+        auto fetch = [&](int j) { a[j % 3] = *reinterpret_cast<const uint4 *>(vp + (j / DT) * V_PAGE + (j % DT) * 1024); };
         fetch(0);
         fetch(1);
 #pragma unroll
@@ -1015,11 +1132,10 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     // new-token bookkeeping (between the two score phases a full tile now has a compare and a branch where the
     // common loop had some thirty scalar instructions, an eighth of the tile's time with one computing wave per SIMD).
     bool all_seen = false;       // wave-uniform: every row of this wave has met a key (full tiles then need no maximum)
-    auto tile_body = [&](int tile, auto new_tile) {
+    auto tile_body = [&](int tile, const uint8_t *vtile, auto new_tile) {
         constexpr bool NEWT = decltype(new_tile)::value;
         const int cur = (tile - tile_begin) & 1;
-        const uint8_t *ktile = lds + cur * K_TILE;
-        const uint8_t *vtile = lds + 2 * K_TILE + cur * V_TILE;
+        const uint8_t *ktile = lds + V_BUFS * V_TILE + cur * K_TILE;
         // valid-slot counts of the tile's pages: requested now, looked at after phase A
         uint32_t limw = FULL_LIMS;
         if constexpr (!NEWT) limw = *reinterpret_cast<const uint32_t *>(page_lims + cur * PAGES);
@@ -1087,14 +1203,18 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     __syncthreads();
     int tile = tile_begin;
     const int ctx_stop = tile_end < n_ctx_tiles ? tile_end : n_ctx_tiles;
+    const uint8_t *vtile = lds, *const v_wrap = lds + V_BUFS * V_TILE;   // V buffers go round in threes
+    auto v_advance = [&] { vtile += V_TILE; if (vtile == v_wrap) vtile = lds; };
     for (; tile < ctx_stop; ++tile) {
-        tile_body(tile, std::false_type{});
+        tile_body(tile, vtile, std::false_type{});
+        v_advance();
         __syncthreads();
     }
     for (; tile < tile_end; ++tile) {
         // Rows of an idle wave are all-zero queries (harmless, never stored); a new-token tile
         // entirely in this wave's future contributes nothing (causal) and is skipped.
-        if ((tile - n_ctx_tiles) * NT <= t0 + UNIT - 1) tile_body(tile, std::true_type{});
+        if ((tile - n_ctx_tiles) * NT <= t0 + UNIT - 1) tile_body(tile, vtile, std::true_type{});
+        v_advance();
         __syncthreads();
     }
 
