@@ -101,6 +101,35 @@ def time_calls(plan, n):
     return start.elapsed_time(end) / n
 
 
+COLD_BYTES = 320 << 20       # distinct K/V the cold-cache loop goes round: more than the 256 MB last-level cache
+
+
+def cold_plans(g, num_splits, phases):
+    """The same call on enough distinct copies of the paged K/V cache that no launch finds its keys and
+    values in L2 or the last-level cache (a served model's layers each own a cache)."""
+    import dataclasses
+    set_bytes = g.k_cache.numel() * g.k_cache.element_size() + g.v_cache.numel() * g.v_cache.element_size()
+    n = max(2, -(-COLD_BYTES // set_bytes) + 1)
+    plans = []
+    for _ in range(n):
+        gi = dataclasses.replace(g, k_cache=g.k_cache.clone(), v_cache=g.v_cache.clone())
+        plans.append(make_plan(gi, num_splits, phases)[0])
+    return plans, set_bytes
+
+
+def time_round_robin(plans, n):
+    """ms per call over n back-to-back launches that go round the plans."""
+    import torch
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(n):
+        plans[i % len(plans)].run()
+    end.record()
+    end.synchronize()
+    return start.elapsed_time(end) / n
+
+
 def cpu_baseline(w, reps):
     """The float32 PyTorch-eager statement of the same op on the host cores."""
     import torch
@@ -304,6 +333,71 @@ def bench_reposition(a):
     print(json.dumps(out))
 
 
+def bench_layer_step(a):
+    """What one engine step asks of this library for a prefill chunk, layer by layer (the call contract of the
+    reference's backend, lazy_attn/lazy/attention/backends/triton_attn.py:96-187, without the model around it):
+    per layer, rotary embedding of the new tokens' queries + write of their un-rotated K and V into that layer's
+    own paged cache (one launch), then ``chunked_prefill_paged_decode`` on that cache.  32 layers, persistent
+    buffers, the north-star shape (one request: 10 x 512 cached tokens in shuffled order, 128 new ones)."""
+    import torch
+    from lazy_amd import workloads as wl
+    from lazy_amd.attention.old_ops.chunked_prefill_paged_decode import chunked_prefill_paged_decode
+    from lazy_amd.model_executor.layers import rotary_embedding as rope
+    layers = a.layers
+    w = wl.config(2)
+    g = w.to("cuda:0")
+    d, bs = g.q.shape[-1], g.v_cache.shape[3]
+    ql, ctx = int(w.max_query_len), int(w.b_seq_len[0] - w.max_query_len)
+    caches = [(g.k_cache.clone(), g.v_cache.clone()) for _ in range(layers)]
+    positions = ctx + torch.arange(ql, device="cuda:0")
+    m = torch.arange(ql, device="cuda:0")
+    slots = (g.block_table[0, ctx // bs + m // bs].long() * bs + m % bs)
+    q_src, out = g.q.clone(), torch.zeros_like(g.q)
+    q = g.q
+
+    def step():
+        for kc, vc in caches:
+            rope.rotate_and_write(positions, q, g.k, g.v, d, g.cos_sin_cache, rotate_query=True, rotate_key=False,
+                                  key_cache=kc, value_cache=vc, slot_mapping=slots)
+            chunked_prefill_paged_decode(q, g.k, g.v, out, "auto", kc, vc, g.block_table, g.b_start_loc,
+                                         g.b_seq_len, g.max_seq_len, g.max_query_len, g.k_scale, g.v_scale,
+                                         cos_sin_cache=g.cos_sin_cache, rotary_dim=d, q_mask=g.q_mask, is_mepic=True)
+    for _ in range(max(a.warmup, 10)):
+        step()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    host = []
+    start.record()
+    for _ in range(a.steps):
+        step()
+    end.record()
+    end.synchronize()
+    gpu_us = start.elapsed_time(end) * 1e3 / (a.steps * layers)
+    for _ in range(20):                      # host side alone: the queue is empty when a step starts
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        step()
+        host.append((time.perf_counter() - t0) * 1e6 / layers)
+    torch.cuda.synchronize()
+    host_us = statistics.median(host)
+    tflops = w.flops / (gpu_us * 1e-6) / 1e12
+    set_mb = (g.k_cache.numel() * g.k_cache.element_size() + g.v_cache.numel() * g.v_cache.element_size()) / 1e6
+    print(json.dumps({
+        "metric": "deferred-RoPE prefill layer step (rotary + cache write, then attention): TFLOP/s of the attention "
+                  "work per layer time, 8B geometry, 5K context, every layer on its own cache",
+        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(gpu_us * layers * 1e-3, 5), "us_per_layer": round(gpu_us, 2),
+        "host_us_per_layer": round(host_us, 2), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "l1_8b_bf16_layer_step_10x512_q128", "layers": layers, "hq": 32, "hkv": 8,
+                   "head_dim": d, "page": bs, "ctx_keys": ctx, "query_tokens": ql,
+                   "cache_mb_per_layer": round(set_mb, 1), "launches_per_layer": 3},
+        "roofline": {"bound": "mfma", "achieved": round(tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(tflops / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "kernel": "rope_cache_write_kernel + prefill_mfma_kernel + prefill_combine_kernel"},
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -316,10 +410,14 @@ def main():
                     help="floor on the untimed warm-up calls, whatever --warmup says (profiler runs lower it)")
     ap.add_argument("--no-host-timing", action="store_true",
                     help="skip the 1 100 entry-point calls that measure host_us_per_call (profiler runs)")
-    ap.add_argument("--path", choices=["prefill", "decode", "rope_write", "reposition"], default="prefill",
+    ap.add_argument("--path", choices=["prefill", "decode", "rope_write", "reposition", "layer_step"], default="prefill",
                     help="prefill: the headline prefix-prefill call (default); decode: the q_len==1 kernel; "
                          "rope_write: Q rotary + paged-cache write of the new tokens; reposition: copy-on-write block "
-                         "re-positioning (all three HBM-bound)")
+                         "re-positioning (all three HBM-bound); layer_step: per layer the cache write and the attention "
+                         "call on that layer's own cache, as an engine step issues them")
+    ap.add_argument("--layers", type=int, default=32, help="layer_step: number of layers (each owns a K/V cache)")
+    ap.add_argument("--no-cold", action="store_true",
+                    help="skip the cold-cache figures (the call going round distinct copies of the K/V cache)")
     ap.add_argument("--variant", choices=["natural", "offset", "block_uniform"], default="natural",
                     help="how a cached key's rotation position is derived: its index (default), the page's q_offset "
                          "(per-block offsets of the un-rotated cache), or one rotation per page of a cache rotated at "
@@ -347,6 +445,8 @@ def main():
         return bench_rope_write(a)
     if a.path == "reposition":
         return bench_reposition(a)
+    if a.path == "layer_step":
+        return bench_layer_step(a)
     w = wl.config(a.config, variant=a.variant)
     g = w.to("cuda:0")
     plan, o = make_plan(g, a.num_splits, _ffi.PHASE_ALL)
@@ -372,6 +472,19 @@ def main():
     main_ms = statistics.median(reps)
     plan.run()
     torch.cuda.synchronize()
+    cold = None
+    if not a.no_cold:
+        # the same call when K/V come from HBM: round-robin over copies of the cache that together exceed the
+        # last-level cache; the headline figures above re-use one cache, which stays in L2 / last-level cache
+        cp, set_bytes = cold_plans(g, a.num_splits, _ffi.PHASE_ALL)
+        cm, _ = cold_plans(g, a.num_splits, _ffi.PHASE_MAIN)
+        n_cold = max(a.steps, 4 * len(cp))
+        for pl in (cp, cm):
+            time_round_robin(pl, 2 * len(pl))
+        cold = {"ms_per_call_cold": round(statistics.median(time_round_robin(cp, n_cold) for _ in range(5)), 5),
+                "kernel_ms_cold": round(statistics.median(time_round_robin(cm, n_cold) for _ in range(5)), 5),
+                "cold_cache_sets": len(cp), "cold_set_mb": round(set_bytes / 1e6, 1)}
+        del cp, cm
     if a.copy_calibration:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0")
         dst = torch.empty_like(src)
@@ -399,6 +512,9 @@ def main():
                      # an operand rate, not a measurement of HBM traffic (that is `traffic`)
                      "operand_gbs_algorithmic_cache_warm": round(w.bytes / (main_ms * 1e-3) / 1e9, 1)},
     }
+    if cold is not None:
+        out.update(cold)
+        out["tflops_cold"] = round(w.flops / (cold["ms_per_call_cold"] * 1e-3) / 1e12, 2)
     if not a.no_host_timing:
         entry_us, launches_us = host_us_per_call(g)
         out["host_us_per_call"] = round(entry_us, 1)            # entry point, repeat call on fixed buffers

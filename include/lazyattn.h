@@ -142,9 +142,23 @@ int lazyattn_prefix_prefill(const lazyattn_prefill_params *p, void *stream);
  * each GPU's memory until the process ends.  A call that would need more returns
  * LAZYATTN_E_SCRATCH_LIMIT (lazyattn_prefill_workspace_bytes() tells beforehand).  Allocates nothing.  All
  * calls on one GPU share that buffer: calls that overlap in time on one GPU (two streams) race; calls on one
- * stream, or otherwise ordered, are safe -- every partial a call merges was written by that call. */
+ * stream, or otherwise ordered, are safe -- every partial a call merges was written by that call.
+ * The first use on a GPU looks the buffer's address up (which may load the library's code onto that GPU):
+ * call lazyattn_static_scratch_prepare() -- or make one call -- with that GPU current before entering a region
+ * that must not allocate, such as a stream capture. */
 int lazyattn_prefix_prefill_static_scratch(const lazyattn_prefill_params *p, void *stream);
 size_t lazyattn_static_scratch_bytes(void);
+int lazyattn_static_scratch_prepare(void);
+
+/* Which kernel lazyattn_prefix_prefill() launches for these arguments: LAZYATTN_KERNEL_GENERIC, LAZYATTN_KERNEL_MFMA4
+ * or LAZYATTN_KERNEL_MFMA8 (a negative LAZYATTN_E_* code when the call would be refused).  *num_splits (optional)
+ * receives the number of key-axis splits; *reason (optional) a static string saying why the fp32 kernel -- some
+ * hundred times slower than the matrix-core kernels -- is the one, NULL otherwise.  Pure host arithmetic.  No
+ * reference counterpart (Triton has one kernel); for callers who want to see the fallback before they pay for it. */
+int lazyattn_prefill_kernel_for(const lazyattn_prefill_params *p, int32_t *num_splits, const char **reason);
+/* The same for lazyattn_paged_decode_rotary(): LAZYATTN_KERNEL_MFMA (the streaming kernel, the only one that reads
+ * packed_block_table / rope_freqs), LAZYATTN_KERNEL_GENERIC, or the LAZYATTN_E_* code the call would return. */
+int lazyattn_paged_decode_kernel_for(const lazyattn_prefill_params *p);
 
 /* q_len == 1 rows: every key (the new token included) comes from the paged cache.
  * pos_mode NATURAL: each key is rotated at its natural position; replaces

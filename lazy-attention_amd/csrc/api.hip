@@ -1,11 +1,14 @@
 // C ABI: argument checks and kernel selection.  Nothing here allocates or synchronises.
 #include "common.hpp"
+#include <atomic>
 #include <mutex>
 
 namespace lazyattn {
 int launch_prefill_generic(const lazyattn_prefill_params &p, int decode, hipStream_t stream);
 int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream);
 bool mfma_supports(const lazyattn_prefill_params &p);
+const char *mfma_unsupported_reason(const lazyattn_prefill_params &p);
+void mfma_choices(const lazyattn_prefill_params &p, int *waves, int *splits);
 size_t mfma_workspace_bytes(const lazyattn_prefill_params &p);
 int launch_decode_mfma(const lazyattn_prefill_params &p, hipStream_t stream);
 bool decode_mfma_supports(const lazyattn_prefill_params &p);
@@ -26,6 +29,21 @@ int launch_pack_cos_sin(const void *table, void *packed, int dtype, int64_t row_
 }  // namespace lazyattn
 
 using namespace lazyattn;
+
+int lazyattn::device_cus() {
+    constexpr int MAX_DEV = 64, FALLBACK = 256;
+    static std::atomic<int> cus[MAX_DEV];
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEV) { (void)hipGetLastError(); return FALLBACK; }
+    int n = cus[dev].load(std::memory_order_relaxed);
+    if (n > 0) return n;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+        (void)hipGetLastError();
+        return FALLBACK;
+    }
+    cus[dev].store(n, std::memory_order_relaxed);
+    return n;
+}
 
 static int elem_bytes(int dt) {
     switch (dt) {
@@ -89,6 +107,39 @@ extern "C" int lazyattn_prefix_prefill(const lazyattn_prefill_params *p, void *s
     return LAZYATTN_E_UNSUPPORTED;
 }
 
+extern "C" int lazyattn_prefill_kernel_for(const lazyattn_prefill_params *p, int32_t *num_splits, const char **reason) {
+    if (num_splits) *num_splits = 1;
+    if (reason) *reason = nullptr;
+    int rc = check_common(p, false);
+    if (rc != LAZYATTN_OK) return rc;
+    const char *why = mfma_unsupported_reason(*p);
+    int kernel = p->kernel;
+    if (kernel == LAZYATTN_KERNEL_AUTO) kernel = why ? LAZYATTN_KERNEL_GENERIC : LAZYATTN_KERNEL_MFMA;
+    if (kernel == LAZYATTN_KERNEL_GENERIC) {
+        if (reason) *reason = p->kernel == LAZYATTN_KERNEL_GENERIC ? "the call asks for it" : why;
+        return LAZYATTN_KERNEL_GENERIC;
+    }
+    if (kernel != LAZYATTN_KERNEL_MFMA && kernel != LAZYATTN_KERNEL_MFMA4 && kernel != LAZYATTN_KERNEL_MFMA8) return LAZYATTN_E_UNSUPPORTED;
+    if (why) {
+        if (reason) *reason = why;
+        return LAZYATTN_E_UNSUPPORTED;
+    }
+    int waves = 4, splits = 1;
+    mfma_choices(*p, &waves, &splits);
+    if (num_splits) *num_splits = splits;
+    return waves == 8 ? LAZYATTN_KERNEL_MFMA8 : LAZYATTN_KERNEL_MFMA4;
+}
+
+extern "C" int lazyattn_paged_decode_kernel_for(const lazyattn_prefill_params *p) {
+    int rc = check_common(p, true);
+    if (rc != LAZYATTN_OK) return rc;
+    if (p->pos_mode == LAZYATTN_POS_OFFSET) return LAZYATTN_E_UNSUPPORTED;
+    if (p->kernel != LAZYATTN_KERNEL_GENERIC && decode_mfma_supports(*p)) return LAZYATTN_KERNEL_MFMA;
+    if (p->packed_block_table || p->rope_freqs) return LAZYATTN_E_UNSUPPORTED;
+    if (p->kernel != LAZYATTN_KERNEL_AUTO && p->kernel != LAZYATTN_KERNEL_GENERIC) return LAZYATTN_E_UNSUPPORTED;
+    return LAZYATTN_KERNEL_GENERIC;
+}
+
 // ---- the prefill call for callers that may not allocate ----
 // Split-KV partials of lazyattn_prefix_prefill_static_scratch() live in this array instead of a caller-provided
 // workspace.  One copy per GPU the library runs on, held until the process ends.  In host code the array's name
@@ -101,6 +152,7 @@ std::mutex scratch_mutex;
 void *scratch_ptr[MAX_DEVICES] = {};
 
 int static_scratch_address(void **out) {
+    // (the current device: the kernels are launched on it, so this is the copy of the array they will see)
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return LAZYATTN_E_LAUNCH;
     std::lock_guard<std::mutex> lock(scratch_mutex);
@@ -115,6 +167,11 @@ int static_scratch_address(void **out) {
 }  // namespace
 
 extern "C" size_t lazyattn_static_scratch_bytes(void) { return STATIC_SCRATCH_BYTES; }
+
+extern "C" int lazyattn_static_scratch_prepare(void) {
+    void *ptr = nullptr;
+    return static_scratch_address(&ptr);
+}
 
 extern "C" int lazyattn_prefix_prefill_static_scratch(const lazyattn_prefill_params *p, void *stream) {
     int rc = check_common(p, false);
@@ -270,4 +327,4 @@ extern "C" const char *lazyattn_error_string(int code) {
     }
 }
 
-extern "C" int lazyattn_abi_version(void) { return 2; }
+extern "C" int lazyattn_abi_version(void) { return 3; }

@@ -9,6 +9,10 @@
 
 namespace lazyattn {
 
+// Compute units of the caller's current device, asked once per device (the launch heuristics fill whole rounds of
+// them).  256 -- an MI355X in its single-partition mode -- when no device can be asked.
+int device_cus();
+
 using bf16_t = __hip_bfloat16;
 using f16_t = __half;
 struct fp8e4m3_t { uint8_t v; };

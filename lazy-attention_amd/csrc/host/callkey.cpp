@@ -27,6 +27,10 @@ static PyObject *tensor_key(PyObject *, PyObject *const *args, Py_ssize_t nargs)
     try {
     for (Py_ssize_t i = 0; i < n; ++i) {
         PyObject *o = PyTuple_GET_ITEM(tup, i);
+        if (m >= 500) {                              // (every write below stays inside buf: a tensor adds at most 3 + 2 x 64)
+            PyErr_SetString(PyExc_ValueError, "tensor_key: too many entries");
+            return nullptr;
+        }
         if (o == Py_None) { buf[m++] = -1; continue; }
         if (!THPVariable_Check(o)) {
             PyErr_SetString(PyExc_TypeError, "tensor_key: not a tensor");
@@ -35,7 +39,7 @@ static PyObject *tensor_key(PyObject *, PyObject *const *args, Py_ssize_t nargs)
         const at::Tensor &t = THPVariable_Unpack(o);
         const auto sizes = t.sizes();
         const auto strides = t.strides();
-        if (m + 3 + 2 * (int)sizes.size() > 500) {
+        if (m + 2 + 2 * (int)sizes.size() > 512) {
             PyErr_SetString(PyExc_ValueError, "tensor_key: too many dimensions");
             return nullptr;
         }

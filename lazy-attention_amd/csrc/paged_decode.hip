@@ -612,7 +612,7 @@ bool decode_mfma_supports(const lazyattn_prefill_params &p) {
 }
 
 // Slices of the page axis per (request, kv head).  A workgroup is four independent waves, one work item each; the
-// launch is fastest when its workgroups fit the chip's 256 CUs in one round with none left over -- a few CUs with a
+// launch is fastest when its workgroups fit the chip's CUs (256 where these were measured) in one round with none left over -- a few CUs with a
 // second workgroup make the tail of the launch (32 requests of 5 K keys: 4 / 6 / 8 slices = 256 / 384 / 512
 // workgroups take 118 / 141 / 123 us; 12 requests: 8 / 12 / 16 slices = 192 / 288 / 384 workgroups 49 / 60 / 50 us) --
 // so: as many slices as keep the work items at or below 1 024, of at least five pages each (5 K keys, call = both
@@ -623,7 +623,7 @@ static int decode_splits(const lazyattn_prefill_params &p) {
     if (natural <= 0) return 1;
     // (or at or below two, three, four times as many -- whole rounds -- when that fills the rounds at least a tenth
     // better: 48 requests = 384 items, 2 / 5 slices fill 75 % of one / 94 % of two rounds: 189 / 181 us)
-    const int64_t round = 256 * WAVES;
+    const int64_t round = (int64_t)device_cus() * WAVES;
     int64_t s = round / natural;
     double fill = (double)(natural * s) / (double)round;
     for (int64_t k = 2; k <= 4; ++k) {

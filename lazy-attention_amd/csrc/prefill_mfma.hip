@@ -205,7 +205,7 @@ static int mfma_splits(const lazyattn_prefill_params &p, int nw);
 // units (computing waves) per workgroup: the shape with the lower estimated time.  Per workgroup a 64-key tile takes
 // about 1.34 us in the four-unit shape (128 rows) and 1.98 us in the eight-unit shape (256 rows: a third less per
 // row), a workgroup has some 8 us of launch, prologue, first-tile latency and epilogue, the workgroups run in rounds
-// of 256, and split partials cost about 2 us plus half a microsecond per split to write and merge.  (Measured on
+// of one per compute unit (256 on the part these figures were taken on), and split partials cost about 2 us plus half a microsecond per split to write and merge.  (Measured on
 // this part with bf16 operands at head size 128; the other element types and head sizes shift both shapes alike.)
 static int mfma_waves(const lazyattn_prefill_params &p) {
     if (p.kernel == LAZYATTN_KERNEL_MFMA4) return 4;
@@ -214,7 +214,8 @@ static int mfma_waves(const lazyattn_prefill_params &p) {
     const int64_t tiles = p.max_seq_len > 0 ? (p.max_seq_len + NT - 1) / NT : 64;
     auto cost = [&](int nw, double tile_us) {
         const int64_t s = mfma_splits(p, nw);
-        const int64_t wgs = p.num_kv_heads * mfma_mtiles_estimate(p, nw) * s, rounds = (wgs + 255) / 256;
+        const int64_t cus = device_cus();
+        const int64_t wgs = p.num_kv_heads * mfma_mtiles_estimate(p, nw) * s, rounds = (wgs + cus - 1) / cus;
         return (double)rounds * ((double)((tiles + s - 1) / s) * tile_us + 8.0) + (s > 1 ? 2.0 + 0.5 * (double)s : 0.0);
     };
     return cost(8, 1.98) <= cost(4, 1.34) ? 8 : 4;
@@ -225,12 +226,12 @@ static int mfma_splits(const lazyattn_prefill_params &p, int nw) {
     const int64_t natural = p.num_kv_heads * mfma_mtiles_estimate(p, nw);
     const int64_t ctx_tiles = p.max_seq_len > 0 ? (p.max_seq_len + NT - 1) / NT : 1;
     // One workgroup per CU and none left over: a CU holds one workgroup at a time, so a few workgroups beyond the
-    // chip's 256 CUs are a second round that most CUs sit out (3 requests of 128 new tokens over 5 K keys, 96
+    // chip's CUs (256 where these figures were taken) are a second round that most CUs sit out (3 requests of 128 new tokens over 5 K keys, 96
     // workgroups per split: 2 / 3 splits = 192 / 288 workgroups take 55 / 77 us; 6 x 64 over 8 K, 48 per split:
     // 5 / 6 splits 65 / 90 us).  Long workgroups (64 tiles and more) may take two to four whole rounds when that
     // fills the rounds at least a fifth better (3 x 512 new tokens over 16 K keys, 192 per split: 1 / 4 splits =
     // 75 % of one round / three full rounds: 448 / 427 us).
-    constexpr int64_t CUS = 256;
+    const int64_t CUS = device_cus();
     int64_t s = natural <= CUS ? CUS / natural : 1;
     auto fill = [&](int64_t sp) {
         const int64_t w = natural * sp, rounds = (w + CUS - 1) / CUS;
@@ -248,27 +249,38 @@ static int mfma_splits(const lazyattn_prefill_params &p, int nw) {
     return s < 1 ? 1 : (int)s;
 }
 
-bool mfma_supports(const lazyattn_prefill_params &p) {
+// Why the matrix-core kernel does not take a call (nullptr: it does).
+const char *mfma_unsupported_reason(const lazyattn_prefill_params &p) {
     const bool fp8 = p.cache_dtype == LAZYATTN_FP8_E4M3 || p.cache_dtype == LAZYATTN_FP8_E5M2;
-    if (p.dtype != LAZYATTN_BF16 && p.dtype != LAZYATTN_F16) return false;
-    if (!(p.cache_dtype == p.dtype || fp8)) return false;
-    if (p.table_dtype != p.dtype && p.table_dtype != LAZYATTN_F32) return false;
+    if (p.dtype != LAZYATTN_BF16 && p.dtype != LAZYATTN_F16) return "operands are not bfloat16 or float16";
+    if (!(p.cache_dtype == p.dtype || fp8)) return "the cache type is neither the operand type nor fp8";
+    if (p.table_dtype != p.dtype && p.table_dtype != LAZYATTN_F32) return "the cos/sin table is neither of the operand type nor float32";
     // 128, 64, or a multiple of 16 below 128 (padded to 128)
-    if (p.head_dim < 16 || p.head_dim > 128 || p.head_dim % 16 || p.rotary_dim != p.head_dim) return false;
-    if ((p.block_size != BS && p.block_size != 2 * BS) || p.x != (fp8 ? 16 : 8)) return false;
-    if (p.q_stride[2] != 1 || p.k_stride[2] != 1 || p.v_stride[2] != 1 || p.o_stride[2] != 1) return false;
-    if (p.kc_stride[4] != 1 || p.kc_stride[3] != p.x || p.kc_stride[2] != (int64_t)p.block_size * p.x) return false;
-    if (p.vc_stride[3] != 1 || p.vc_stride[2] != p.block_size) return false;
+    if (p.head_dim < 16 || p.head_dim > 128 || p.head_dim % 16) return "head size above 128 or not a multiple of 16";
+    if (p.rotary_dim != p.head_dim) return "rotary_dim differs from the head size";
+    if (p.block_size != BS && p.block_size != 2 * BS) return "cache pages of neither 16 nor 32 slots";
+    if (p.x != (fp8 ? 16 : 8)) return "the key cache's innermost axis is not 16 bytes";
+    if (p.q_stride[2] != 1 || p.k_stride[2] != 1 || p.v_stride[2] != 1 || p.o_stride[2] != 1) return "q/k/v/o rows are not contiguous";
+    if (p.kc_stride[4] != 1 || p.kc_stride[3] != p.x || p.kc_stride[2] != (int64_t)p.block_size * p.x)
+        return "a key cache page of one head is not contiguous";
+    if (p.vc_stride[3] != 1 || p.vc_stride[2] != p.block_size) return "a value cache page of one head is not contiguous";
     const int64_t al[] = {p.q_stride[0], p.q_stride[1], p.k_stride[0], p.k_stride[1], p.v_stride[0], p.v_stride[1],
                           p.o_stride[0], p.o_stride[1], p.kc_stride[0], p.kc_stride[1], p.vc_stride[0], p.vc_stride[1],
                           p.table_stride};
     for (int64_t s : al)
-        if (s % 16) return false;
+        if (s % 16) return "a stride is not a multiple of 16 elements";
     const void *ptrs[] = {p.q, p.k, p.v, p.o, p.k_cache, p.v_cache, p.cos_sin_cache};
     for (const void *q : ptrs)
-        if (((uintptr_t)q) & 15) return false;
-    if (p.num_tokens <= 0) return false;
-    return true;
+        if (((uintptr_t)q) & 15) return "a tensor is not 16-byte aligned";
+    if (p.num_tokens <= 0) return "num_tokens is not set";
+    return nullptr;
+}
+bool mfma_supports(const lazyattn_prefill_params &p) { return mfma_unsupported_reason(p) == nullptr; }
+
+// the choices launch_prefill_mfma() makes for a call: computing waves per workgroup (4 or 8) and key-axis splits
+void mfma_choices(const lazyattn_prefill_params &p, int *waves, int *splits) {
+    *waves = mfma_waves(p);
+    *splits = mfma_splits(p, *waves);
 }
 
 size_t mfma_workspace_bytes(const lazyattn_prefill_params &p) {

@@ -20,11 +20,13 @@ POS_NATURAL, POS_OFFSET, POS_BLOCK_UNIFORM = 0, 1, 2
 KERNEL_AUTO, KERNEL_GENERIC, KERNEL_MFMA, KERNEL_MFMA4, KERNEL_MFMA8 = 0, 1, 2, 3, 4
 PHASE_MAIN, PHASE_COMBINE, PHASE_ALL = 1, 2, 3
 
+E_UNSUPPORTED = -4
 ERRORS = {-1: "NULL", -2: "SHAPE", -3: "DTYPE", -4: "UNSUPPORTED", -5: "WORKSPACE", -6: "LAUNCH", -7: "SCRATCH_LIMIT"}
 EXPORTS = ("lazyattn_prefill_workspace_bytes", "lazyattn_prefix_prefill", "lazyattn_prefix_prefill_static_scratch",
            "lazyattn_static_scratch_bytes", "lazyattn_paged_decode_workspace_bytes",
            "lazyattn_paged_decode_rotary", "lazyattn_build_cos_sin_cache",
            "lazyattn_pack_cos_sin_cache", "lazyattn_rope_and_cache_write", "lazyattn_build_rotation_metadata", "lazyattn_reposition_blocks", "lazyattn_pack_block_table",
+           "lazyattn_static_scratch_prepare", "lazyattn_prefill_kernel_for", "lazyattn_paged_decode_kernel_for",
            "lazyattn_error_string", "lazyattn_abi_version")
 
 _DTYPE = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
@@ -84,6 +86,12 @@ def lib() -> C.CDLL:
         L.lazyattn_paged_decode_workspace_bytes.argtypes = [C.POINTER(PrefillParams)]
         L.lazyattn_static_scratch_bytes.restype = C.c_size_t
         L.lazyattn_static_scratch_bytes.argtypes = []
+        L.lazyattn_static_scratch_prepare.restype = C.c_int
+        L.lazyattn_static_scratch_prepare.argtypes = []
+        L.lazyattn_prefill_kernel_for.restype = C.c_int
+        L.lazyattn_prefill_kernel_for.argtypes = [C.POINTER(PrefillParams), C.POINTER(C.c_int32), C.POINTER(C.c_char_p)]
+        L.lazyattn_paged_decode_kernel_for.restype = C.c_int
+        L.lazyattn_paged_decode_kernel_for.argtypes = [C.POINTER(PrefillParams)]
         for name in ("lazyattn_prefix_prefill", "lazyattn_prefix_prefill_static_scratch", "lazyattn_paged_decode_rotary"):
             fn = getattr(L, name)
             fn.restype = C.c_int

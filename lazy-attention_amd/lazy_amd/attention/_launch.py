@@ -3,6 +3,8 @@
 ``old_ops/prefix_prefill.py:437-486``) and the hand-off to the C ABI."""
 from __future__ import annotations
 
+import ctypes
+import warnings
 from collections import OrderedDict
 from typing import Optional
 
@@ -97,6 +99,19 @@ def forget_calls() -> None:
 
 
 _ffi.on_workspace_growth(forget_calls)      # remembered plans point into the old buffer
+
+
+_warned_generic = set()
+
+
+def _warn_generic(reason: str) -> None:
+    """Once per reason: a 16-bit call that the matrix-core kernels do not take runs the fp32 kernel, some hundred
+    times slower, and nothing else would tell."""
+    if reason in _warned_generic:
+        return
+    _warned_generic.add(reason)
+    warnings.warn("lazy_amd: this prefix-prefill call runs the fp32 fallback kernel (about 100x slower than the "
+                  f"matrix-core kernels): {reason}", RuntimeWarning, stacklevel=4)
 
 
 def _cache_code(kv_cache_dtype: str, k_cache: torch.Tensor, v_cache: torch.Tensor, q_dtype) -> int:
@@ -199,6 +214,10 @@ def launch_prefill(*, q, k, v, o, kv_cache_dtype, k_cache, v_cache, b_loc, b_sta
         rotate_new_k=rotate_new_k, skip_decode=skip_decode, fp32_rotary=fp32_rotary,
         kernel=kernel, num_splits=num_splits, phases=phases, max_seq_len=max_seq_len, packed_table=packed,
         packed_block_table=packed_block_table, rope_freqs=rope_freqs)
+    if not decode and kernel == _ffi.KERNEL_AUTO and q.dtype in (torch.bfloat16, torch.float16):
+        why = ctypes.c_char_p()
+        if lib.lazyattn_prefill_kernel_for(p, None, ctypes.byref(why)) == _ffi.KERNEL_GENERIC and why.value:
+            _warn_generic(why.value.decode())
     plan = PrefillPlan(p, dev, decode, keep=(q, k, v, o, k_cache, v_cache, b_loc, b_start_loc, b_seq_len,
                                             cos_sin_cache, q_offset, q_mask, is_lazy, k_scale, v_scale,
                                             packed_block_table, rope_freqs), own=(packed,), repeatable=repeatable)
@@ -232,6 +251,15 @@ class PrefillPlan:
         rc = self._entry(self.params, stream)
         if rc:
             _ffi.check(rc, "lazyattn_paged_decode_rotary" if self.decode else "lazyattn_prefix_prefill")
+
+    def kernel(self):
+        """(LAZYATTN_KERNEL_* the call resolves to or a negative error code, key-axis splits, why the fp32 kernel if
+        it is the one) -- what ``run()`` will launch."""
+        if self.decode:
+            return self._lib.lazyattn_paged_decode_kernel_for(self.params), 0, None
+        splits, why = ctypes.c_int32(0), ctypes.c_char_p()
+        k = self._lib.lazyattn_prefill_kernel_for(self.params, ctypes.byref(splits), ctypes.byref(why))
+        return k, splits.value, why.value.decode() if why.value else None
 
     def resize(self, batch: int, num_tokens: int, max_seq_len: int, max_q_len: int) -> bool:
         """Set the counts of the call (the struct's only fields that depend on the first dimension of the per-token

@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol():
     assert set(names) == set(_ffi.EXPORTS)
     for n in names:
         assert getattr(lib, n) is not None
-    assert lib.lazyattn_abi_version() == 2
+    assert lib.lazyattn_abi_version() == 3
     assert lib.lazyattn_error_string(-4).decode().startswith("request not supported")
 
 
@@ -230,3 +230,57 @@ int main() {
     exe = tmp_path / "fd"
     subprocess.check_call(["g++", "-O2", "-std=c++17", "-I", os.path.join(ROOT, "lazy-attention_amd", "csrc"), str(src), "-o", str(exe)])
     assert subprocess.check_output([str(exe)]).split()[0] == b"0"
+
+
+def test_env_switches_take_the_reference_truthy_values(monkeypatch):
+    """lazy_attn/lazy/utils/variants.py:63-68: only 1 / true / yes / on (any case, stripped) switch something on."""
+    from lazy_amd.attention.ops.chunked_prefill_paged_decode import _env_flag
+    for value, want in (("1", True), (" True ", True), ("YES", True), ("on", True), ("0", False), ("false", False),
+                        ("off", False), ("", False), ("2", False)):
+        monkeypatch.setenv("NO_LAZY", value)
+        assert _env_flag("NO_LAZY") is want, value
+    monkeypatch.delenv("NO_LAZY")
+    assert _env_flag("NO_LAZY") is False
+
+
+def _fake_params(dtype=_ffi.BF16, head_dim=128, block_size=16, tokens=128, seq=5248, kernel=_ffi.KERNEL_AUTO):
+    """A parameter block with made-up (aligned, never dereferenced) addresses, for the host-side queries."""
+    p = _ffi.PrefillParams()
+    for i, n in enumerate(("q", "k", "v", "o", "k_cache", "v_cache", "block_table", "b_start_loc", "b_seq_len",
+                           "cos_sin_cache")):
+        setattr(p, n, 0x10000 * (i + 1))
+    p.batch, p.num_q_heads, p.num_kv_heads, p.head_dim, p.rotary_dim = 1, 32, 8, head_dim, head_dim
+    p.block_size, p.x = block_size, 8 if dtype != _ffi.F32 else 4
+    p.dtype = p.cache_dtype = p.table_dtype = dtype
+    p.index_bits, p.max_q_len, p.num_tokens, p.max_seq_len, p.kernel = 32, tokens, tokens, seq, kernel
+    for n, st in (("q_stride", (32 * head_dim, head_dim, 1)), ("o_stride", (32 * head_dim, head_dim, 1)),
+                  ("k_stride", (8 * head_dim, head_dim, 1)), ("v_stride", (8 * head_dim, head_dim, 1)),
+                  ("kc_stride", (8 * head_dim * block_size, head_dim * block_size, block_size * p.x, p.x, 1)),
+                  ("vc_stride", (8 * head_dim * block_size, head_dim * block_size, block_size, 1))):
+        getattr(p, n)[:] = st
+    p.bt_stride[:] = (512, 1)
+    p.table_stride = head_dim
+    return p
+
+
+def test_kernel_query_names_the_kernel_and_the_reason_for_the_fallback():
+    lib = _ffi.lib()
+    splits, why = ctypes.c_int32(0), ctypes.c_char_p()
+    p = _fake_params()
+    k = lib.lazyattn_prefill_kernel_for(ctypes.byref(p), ctypes.byref(splits), ctypes.byref(why))
+    assert k in (_ffi.KERNEL_MFMA4, _ffi.KERNEL_MFMA8) and splits.value >= 1 and why.value is None
+    p = _fake_params(dtype=_ffi.F32)
+    assert lib.lazyattn_prefill_kernel_for(ctypes.byref(p), None, ctypes.byref(why)) == _ffi.KERNEL_GENERIC
+    assert b"bfloat16" in why.value
+    p = _fake_params(head_dim=136)
+    assert lib.lazyattn_prefill_kernel_for(ctypes.byref(p), None, ctypes.byref(why)) == _ffi.KERNEL_GENERIC
+    assert b"head size" in why.value
+    p = _fake_params(block_size=8)
+    assert lib.lazyattn_prefill_kernel_for(ctypes.byref(p), None, ctypes.byref(why)) == _ffi.KERNEL_GENERIC
+    assert b"pages" in why.value
+    p = _fake_params(block_size=8, kernel=_ffi.KERNEL_MFMA)         # asked for, not available: what the call returns
+    assert lib.lazyattn_prefill_kernel_for(ctypes.byref(p), None, ctypes.byref(why)) == _ffi.E_UNSUPPORTED
+    p = _fake_params(); p.q = 0x10008
+    assert lib.lazyattn_prefill_kernel_for(ctypes.byref(p), None, ctypes.byref(why)) == _ffi.KERNEL_GENERIC
+    assert b"aligned" in why.value
+    assert lib.lazyattn_prefill_kernel_for(None, None, None) == -1

@@ -295,3 +295,83 @@ def test_views_of_persistent_buffers_reuse_the_call_made_for_other_counts(varian
     # one remembered call for the steps with several requests (made again at every change of the batch size when it
     # owns batch-sized tensors), one for the single request (no q_len == 1 launch there)
     assert len(_launch._calls) == 2
+
+
+def _block_uniform_call(g, out, lazy, packed=None, **kw):
+    entry_block_uniform(g.q, g.k, g.v, out, "auto", g.k_cache, g.v_cache, g.block_table, g.b_start_loc,
+                        g.b_seq_len, g.max_seq_len, g.max_query_len, g.k_scale, g.v_scale,
+                        sm_scale=g.q.shape[-1] ** -0.5, rotary_dim=g.q.shape[-1], cos_sin_cache=g.cos_sin_cache,
+                        is_lazy=lazy, q_offset=None if packed is not None else g.q_offset,
+                        q_mask=None if packed is not None else g.q_mask, packed_block_table=packed, **kw)
+
+
+@pytest.mark.parametrize("use_packed", [True, False])
+def test_ignore_q_mask_switch_drops_the_pad_counts_of_the_single_token_rows(monkeypatch, use_packed):
+    """LAZY_DECODE_IGNORE_Q_MASK (ops/chunked_prefill_paged_decode.py:146,218; ops/models/llama_v1.py:161-162):
+    the q_len == 1 rows see every slot of every page, the prefill rows keep their masks."""
+    print(f"case: LAZY_DECODE_IGNORE_Q_MASK packed={use_packed}", flush=True)
+    w = _mixed("block_uniform", torch.bfloat16, 128)
+    lazy = torch.tensor([True, True, True, True])
+    ref = torch.full_like(w.q, 5.0)
+    orc.prefix_prefill(w.q, w.k, w.v, w.k_cache, w.v_cache, w.block_table, w.b_start_loc, w.b_seq_len,
+                       w.cos_sin_cache, w.q_offset, w.q_mask, pos_mode=w.pos_mode, rotate_new_k=w.rotate_new_k,
+                       is_lazy=lazy, skip_decode=True, out=ref)
+    masked = ref.clone()
+    orc.paged_decode(w.q, w.k_cache, w.v_cache, w.block_table, w.b_start_loc, w.b_seq_len, w.cos_sin_cache,
+                     None, q_offset=w.q_offset, is_lazy=lazy, pos_mode=w.pos_mode, out=ref)
+    orc.paged_decode(w.q, w.k_cache, w.v_cache, w.block_table, w.b_start_loc, w.b_seq_len, w.cos_sin_cache,
+                     w.q_mask, q_offset=w.q_offset, is_lazy=lazy, pos_mode=w.pos_mode, out=masked)
+    assert (ref.float() - masked.float()).abs().max().item() > 5e-2      # the switch changes these rows
+    g = w.to(DEV)
+    packed = ((g.block_table.long() << 32) | (g.q_offset.long() << 16) | g.q_mask.long()) if use_packed else None
+    for value, want in (("1", ref), ("off", masked)):
+        monkeypatch.setenv("LAZY_DECODE_IGNORE_Q_MASK", value)
+        out = torch.full_like(g.q, 5.0)
+        _block_uniform_call(g, out, lazy.to(DEV), packed)
+        err = (out.cpu().float() - want.float()).abs().max().item()
+        assert err < 2e-2, (value, err)
+
+
+def test_computed_cos_sin_takes_its_frequencies_from_rope_meta_not_from_the_layers_bf16_buffer(monkeypatch):
+    """LAZY_DECODE_COMPUTE_COS_SIN: the reference passes the layer's bfloat16 ``inv_freq`` as ``freqs`` and its kernel
+    never reads it (ops/models/llama_v1.py:127-133 derives the frequencies from ``rope_meta``)."""
+    print("case: LAZY_DECODE_COMPUTE_COS_SIN with a bf16 freqs buffer", flush=True)
+    w = _mixed("block_uniform", torch.bfloat16, 128)
+    lazy = torch.tensor([True, True, False, True])
+    ref = _expected(w, lazy)
+    g = w.to(DEV)
+    inv = (500000.0 ** (-torch.arange(0, 128, 2, dtype=torch.float32) / 128)).to(torch.bfloat16).to(DEV)
+    meta = dict(ROPE_TYPE=0, BASE=500000.0, SCALING_FACTOR=1.0, LOW_FACTOR=1.0, HIGH_FACTOR=1.0,
+                ORIG_MAX_POSITION=8192, PI_VALUE=3.141592653589793)
+    monkeypatch.setenv("LAZY_DECODE_COMPUTE_COS_SIN", "1")
+    packed = (g.block_table.long() << 32) | (g.q_offset.long() << 16) | g.q_mask.long()
+    for _ in range(2):                                   # the second call is the remembered one
+        out = torch.full_like(g.q, 5.0)
+        _block_uniform_call(g, out, lazy.to(DEV), packed, freqs=inv, rope_meta=meta)
+        err = (out.cpu().float() - ref.float()).abs().max().item()
+        assert err < 2e-2, err
+    # another rope_meta is another call
+    out2 = torch.full_like(g.q, 5.0)
+    _block_uniform_call(g, out2, lazy.to(DEV), packed, freqs=inv, rope_meta=dict(meta, BASE=10000.0))
+    assert (out2.float() - out.float()).abs().max().item() > 1e-2
+
+
+def test_packed_table_with_operands_the_streaming_kernel_does_not_take():
+    """A query view that is not 16-byte aligned: only the library's own predicate sees that, and the call must then
+    run the generic kernel on un-packed tables instead of failing."""
+    print("case: packed table + misaligned query view", flush=True)
+    w = _mixed("block_uniform", torch.bfloat16, 128)
+    lazy = torch.tensor([True, False, True, True])
+    ref = _expected(w, lazy)
+    g = w.to(DEV)
+    buf = torch.zeros(g.q.shape[0], g.q.shape[1], 128 + 4, dtype=g.q.dtype, device=DEV)
+    buf[:, :, 4:] = g.q
+    import dataclasses
+    gv = dataclasses.replace(g, q=buf[:, :, 4:])
+    assert gv.q.data_ptr() % 16 == 8
+    packed = (g.block_table.long() << 32) | (g.q_offset.long() << 16) | g.q_mask.long()
+    out = torch.full_like(g.q, 5.0)
+    with pytest.warns(RuntimeWarning, match="fp32 fallback kernel"):
+        _block_uniform_call(gv, out, lazy.to(DEV), packed)
+    err = (out.cpu().float() - ref.float()).abs().max().item()
+    assert err < 2e-2, err

@@ -59,3 +59,40 @@ def test_static_scratch_entry_rejects_calls_beyond_its_buffer():
     assert rc == -7 and b"static buffer" in lib.lazyattn_error_string(rc)
     torch.cuda.synchronize()
     assert torch.all(o == 5.0)
+
+
+def test_static_scratch_entry_allocates_nothing_and_replays_from_a_captured_graph():
+    """Capture is what the entry point is for: after ``lazyattn_static_scratch_prepare()`` (outside the capture) a
+    call inside a stream capture must record, replay with the right result every time, and leave the amount of
+    free device memory where it was."""
+    print("case: no-alloc prefill entry under stream capture", flush=True)
+    lib = _ffi.lib()
+    g = wl.config(2, shrink=2).to(DEV)
+    ref = torch.full_like(g.q, 5.0)
+    _plan(g, ref, 0).run()
+    got = torch.full_like(g.q, 5.0)
+    plan = _plan(g, got, 0)
+    assert lib.lazyattn_prefill_workspace_bytes(ctypes.byref(plan.params)) > 0
+    plan.params.workspace = None
+    plan.params.workspace_bytes = 0
+    assert lib.lazyattn_static_scratch_prepare() == 0
+    # one eager call first: kernel attributes of this shape are set, nothing is left to do but launches
+    assert lib.lazyattn_prefix_prefill_static_scratch(ctypes.byref(plan.params), torch.cuda.current_stream().cuda_stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(got, ref)
+    free0 = torch.cuda.mem_get_info()[0]
+    assert lib.lazyattn_prefix_prefill_static_scratch(ctypes.byref(plan.params), torch.cuda.current_stream().cuda_stream) == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            rc = lib.lazyattn_prefix_prefill_static_scratch(ctypes.byref(plan.params), side.cuda_stream)
+    assert rc == 0, rc
+    for step in range(3):
+        got.fill_(7.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got, ref), step
+        torch.zeros(1 << 20, device=DEV).sum().item()          # unrelated eager work between the replays
