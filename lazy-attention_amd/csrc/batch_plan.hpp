@@ -1,0 +1,269 @@
+// How a batch of requests with different lengths is cut into work items of about equal length, decided on the device.
+//
+// The host knows the number of requests, of new tokens and the two maxima the caller passes; the lengths themselves
+// live in device memory (b_start_loc, b_seq_len).  A split count chosen on the host is therefore the same for every
+// request and sized for the longest one: a batch of ragged requests then leaves most compute units idle behind the
+// few workgroups of its long requests.  For calls with more than one request the host only fixes the number of work
+// items per kv head the grid has room for; the first wave of every workgroup of the main kernel reads all the
+// lengths -- one memory round trip, which its own lengths cost anyway -- and derives, identically everywhere:
+//   m_j     m-tiles (workgroups per kv head and split) of request j
+//   c_j     cost of its key axis in 64-key tiles (a new-token tile counts as three)
+//   T       tiles per work item: ceil(c_max / k) for the largest k = 1 .. 64 (splits of the longest request) with
+//           which the items still fit one round of the chip's compute units -- found by bisection, the item count
+//           being monotonic in k; no request is split when the m-tiles alone exceed a round
+//   s_j     = ceil(c_j / T) key-axis splits of request j (at least two tiles each, at most 64)
+// and from the prefix sums of m_j s_j which (request, m-tile, split) its work item is.  The first work item of every
+// request leaves (first item, splits, m-tiles) of the request in a small table at the head of the workspace, where
+// the merge kernel finds them with one scalar load.
+// The arithmetic per request is plain C++ (also compiled for the host, where a unit test checks its invariants).
+#pragma once
+#include <stdint.h>
+
+#include "fastdiv.hpp"
+
+namespace lazyattn {
+
+constexpr int PLAN_UNIT = 32;          // query rows per computing wave
+constexpr int PLAN_TILE = 64;          // keys per tile
+constexpr int PLAN_PAGE = 16;          // slots per run of context the kernel calls a page
+constexpr int PLAN_NEW_COST = 3;       // a new-token tile costs about three context tiles
+constexpr int PLAN_MAX_SPLITS = 64;
+
+struct BatchShape {
+    int32_t group;          // q-heads per kv-head
+    int32_t nc;             // 32-row units per workgroup (4 or 8)
+    int32_t n_mt_cap;       // m-tiles the caller's max_q_len allows per request (rows beyond are not computed)
+    int32_t skip_decode;    // requests with one new token are left out
+    int32_t items_cap;      // work items per kv head the grid has room for (at least the m-tiles)
+    int32_t items_target;   // work items per kv head that fill one round of the chip's compute units
+    int32_t items_split_cap;    // most work items per kv head of a batch that is split: what the partial rows have room for
+    int32_t forced_splits;  // > 0: every request gets this many splits (the caller's num_splits)
+    int32_t table_bytes;    // the requests' records at the head of the workspace (a multiple of 256); the partial rows follow
+};
+
+// (lengths are below 2^31: 32-bit arithmetic, shifts for the powers of two -- this runs at the head of every workgroup)
+LAZYATTN_HD int plan_mtiles(int32_t q_len, int32_t ctx_len, const BatchShape &s) {
+    if (q_len <= 0 || ctx_len < 0 || (s.skip_decode && q_len == 1)) return 0;
+    const uint32_t chunks = ((uint32_t)q_len + PLAN_UNIT - 1) / PLAN_UNIT;           // < 2^26
+    const uint32_t cap = (uint32_t)s.n_mt_cap;
+    if (chunks > (cap << (s.nc == 8 ? 3 : 2))) return (int)cap;                        // (also keeps the product below in range)
+    const uint32_t units = chunks * (uint32_t)s.group;
+    const uint32_t m = s.nc == 8 ? (units + 7) >> 3 : (units + 3) >> 2;
+    return (int)(m < cap ? m : cap);
+}
+// tiles of the key axis, weighted (below 2^24 for every context a 32-bit length can describe)
+LAZYATTN_HD uint32_t plan_cost(int32_t q_len, int32_t ctx_len) {
+    const uint32_t pages = ((uint32_t)ctx_len + PLAN_PAGE - 1) / PLAN_PAGE;
+    const uint32_t ctx_tiles = (pages + PLAN_TILE / PLAN_PAGE - 1) / (PLAN_TILE / PLAN_PAGE);
+    const uint32_t new_tiles = ((uint32_t)q_len + PLAN_TILE - 1) / PLAN_TILE;
+    const uint32_t c = ctx_tiles + PLAN_NEW_COST * new_tiles;
+    return c < (1u << 24) - 1 ? c : (1u << 24) - 1;
+}
+// n / d for n, d below 2^24, d > 0, through one float reciprocal and an integer correction (exact)
+LAZYATTN_HD uint32_t plan_udiv(uint32_t n, uint32_t d) {
+    uint32_t q = (uint32_t)((float)n * (1.0f / (float)d));
+    while (q * d > n) --q;
+    while ((q + 1) * d <= n) ++q;
+    return q;
+}
+// splits of a request of `cost` tiles when a work item is to have at most T tiles (T = 0: no request is split)
+LAZYATTN_HD int plan_splits(uint32_t cost, uint32_t T, const BatchShape &s) {
+    uint32_t n;
+    if (s.forced_splits > 0) n = (uint32_t)s.forced_splits;
+    else if (T == 0) n = 1;
+    else { n = plan_udiv(cost, T); n += n * T < cost; }
+    const uint32_t most = cost / 2 > 1 ? cost / 2 : 1;             // at least two tiles per split
+    n = n < most ? n : most;
+    n = n < (uint32_t)PLAN_MAX_SPLITS ? n : (uint32_t)PLAN_MAX_SPLITS;
+    return (int)(n < 1 ? 1 : n);
+}
+
+// What the first work item of a request leaves for the merge kernel (one entry per request at the head of the workspace).
+struct PlanRecord { int32_t item_base, nsplit, m, pad; };
+
+#if defined(__HIPCC__)
+// ---------------------------------------------------------------------------------------- one wave scans the batch
+struct PlanTables { const void *b_start_loc, *b_seq_len; int32_t batch, index_bits; };
+
+// The low 32 bits of an offset or length (all below 2^31), whatever the width of the entries: one load and no
+// branch, so that the nine of a lane are in flight together.
+__device__ __forceinline__ int32_t plan_index(const void *p, int64_t i, int bits) {
+    return *reinterpret_cast<const int32_t *>((const char *)p + i * (int64_t)(bits >> 3));
+}
+// Inclusive prefix sum / running maximum over the 64 lanes of a wave in six data-parallel steps (shifts by 1, 2, 4, 8
+// inside the rows of 16 lanes, then the last lane of a row combined into the rows after it): vector instructions, no
+// trip through the LDS crossbar as a shuffle takes.  Values are non-negative (the identity is 0).
+#define LAZYATTN_PLAN_SCAN(OP)                                                                       \
+    v = OP(v, __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false)); /* row_shr:1 */            \
+    v = OP(v, __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false)); /* row_shr:2 */            \
+    v = OP(v, __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false)); /* row_shr:4 */            \
+    v = OP(v, __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false)); /* row_shr:8 */            \
+    v = OP(v, __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false)); /* row_bcast:15 -> rows 1, 3 */ \
+    v = OP(v, __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false)); /* row_bcast:31 -> rows 2, 3 */
+__device__ __forceinline__ int plan_add(int a, int b) { return a + b; }
+__device__ __forceinline__ int plan_max(int a, int b) { return a > b ? a : b; }
+__device__ __forceinline__ int plan_wave_scan(int v) { LAZYATTN_PLAN_SCAN(plan_add) return v; }
+__device__ __forceinline__ int plan_wave_sum(int v) { return __builtin_amdgcn_readlane(plan_wave_scan(v), 63); }
+__device__ __forceinline__ int plan_wave_max(int v) { LAZYATTN_PLAN_SCAN(plan_max) return __builtin_amdgcn_readlane(v, 63); }
+#undef LAZYATTN_PLAN_SCAN
+
+// The balanced list is for batches of up to 256 requests (four per lane of the scanning wave; larger batches have
+// requests enough to fill the chip and take the plain grid).
+constexpr int PLAN_MAX_BATCH = 256;
+// The requests R lane .. R lane + R - 1 (R = 1 for batches of up to 64 requests, else 4): their m-tile counts and
+// costs (0 beyond the batch).  2 R + 1 loads per lane, requested together.
+template <int R> struct PlanLane { int m[R]; uint32_t c[R]; };
+template <int R> __device__ __forceinline__ PlanLane<R> plan_load(const PlanTables &t, const BatchShape &s, int lane) {
+    const int r0 = lane * R;
+    int32_t off[R + 1], seq[R];
+#pragma unroll
+    for (int j = 0; j < R + 1; ++j) {
+        const int rb = r0 + j;
+        off[j] = plan_index(t.b_start_loc, rb < t.batch ? rb : t.batch, t.index_bits);
+    }
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        const int rb = r0 + j;
+        seq[j] = plan_index(t.b_seq_len, rb < t.batch ? rb : t.batch - 1, t.index_bits);
+    }
+    PlanLane<R> r;
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        const int32_t ql = r0 + j < t.batch ? off[j + 1] - off[j] : 0;
+        const int32_t ctx = seq[j] - ql;
+        r.m[j] = plan_mtiles(ql, ctx, s);
+        r.c[j] = r.m[j] ? plan_cost(ql, ctx) : 0;
+    }
+    return r;
+}
+
+// plan_splits() for a T the whole wave shares: the reciprocal is formed once, the quotient needs one correction each
+// way (cost and T are below 2^24, so the float product is off by less than one)
+struct PlanDivisor { uint32_t T; float inv; };
+__device__ __forceinline__ PlanDivisor plan_divisor(uint32_t T) { return PlanDivisor{T, T ? 1.0f / (float)T : 0.f}; }
+__device__ __forceinline__ int plan_splits_fast(uint32_t cost, const PlanDivisor &d, const BatchShape &s) {
+    uint32_t n;
+    if (s.forced_splits > 0) n = (uint32_t)s.forced_splits;
+    else if (d.T == 0) n = 1;
+    else {
+        uint32_t q = (uint32_t)((float)cost * d.inv);
+        q -= q * d.T > cost;
+        q += (q + 1) * d.T <= cost;
+        n = q + (q * d.T < cost);
+    }
+    const uint32_t most = cost / 2 > 1 ? cost / 2 : 1;
+    n = n < most ? n : most;
+    n = n < (uint32_t)PLAN_MAX_SPLITS ? n : (uint32_t)PLAN_MAX_SPLITS;
+    return (int)(n < 1 ? 1 : n);
+}
+// work items per kv head when a work item is to have at most T tiles (wave-uniform)
+template <int R> __device__ __forceinline__ int plan_count(const PlanLane<R> &r, const BatchShape &s, uint32_t T) {
+    const PlanDivisor d = plan_divisor(T);
+    int n = 0;
+#pragma unroll
+    for (int j = 0; j < R; ++j) n += r.m[j] ? r.m[j] * plan_splits_fast(r.c[j], d, s) : 0;
+    return plan_wave_sum(n);
+}
+// Estimated time of the launch in microseconds when the batch is cut into N work items per kv head of at most L
+// tiles, W tiles in all per kv head: one round if the items fit the chip's compute units, else the work spread over
+// them plus half an item for the ragged end; a workgroup's fixed cost per item.
+// (Measured on an MI355X with 16-bit operands at head size 128: 1.34 / 1.98 us per tile for workgroups of 4 / 8
+// units, some 6 us of launch, prologue, first-tile latency and epilogue per workgroup.)
+constexpr float PLAN_ITEM_US = 6.f;
+__device__ __forceinline__ float plan_tile_us(const BatchShape &s) { return s.nc == 8 ? 1.98f : 1.34f; }
+__device__ __forceinline__ float plan_estimate_us(float W, int N, uint32_t L, const BatchShape &s) {
+    const float tile_us = plan_tile_us(s);
+    if (N <= s.items_target) return (float)L * tile_us + PLAN_ITEM_US;
+    return (W * tile_us + (float)N * PLAN_ITEM_US) / (float)s.items_target + 0.5f * (float)L * tile_us;
+}
+// T for the whole batch (wave-uniform; 0: no request is split): ceil(c_max / k) for the number k of splits of the
+// longest request with the lower estimate of
+//   the largest k whose items fit one round of the chip's compute units, and
+//   the largest k whose items fit the room the grid has beyond a round, if it has any (it has when the m-tiles alone
+//   come near a round, so that one round would leave the long requests whole)
+// -- both by bisection: the count grows with k.
+template <int R>
+__device__ __forceinline__ int plan_largest_k(const PlanLane<R> &r, const BatchShape &s, uint32_t c_max, int M, int limit, int guess, int *count) {
+    int lo = 1, hi = PLAN_MAX_SPLITS + 1, n_lo = M;                // fits(lo), !fits(hi)
+    int k = guess, fits_in_a_row = 0;
+#pragma nounroll
+    while (hi - lo > 1) {
+        if (k <= lo || k >= hi) k = (lo + hi) >> 1;
+        const int n = plan_count(r, s, (c_max + (uint32_t)k - 1) / (uint32_t)k);
+        // (after the first guess its neighbour above: equal requests are done in two probes)
+        if (n <= limit) { lo = k; n_lo = n; k = ++fits_in_a_row < 2 ? k + 1 : (lo + hi) >> 1; }
+        else { hi = k; k = (lo + hi) >> 1; fits_in_a_row = 2; }
+    }
+    *count = n_lo;
+    return lo;
+}
+template <int R> __device__ __forceinline__ uint32_t plan_target(const PlanLane<R> &r, const BatchShape &s) {
+    if (s.forced_splits > 0) return 0;
+    int cm = 0, ws = 0, ms = 0;
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        cm = plan_max(cm, (int)r.c[j]);
+        ws += (int)(((uint32_t)r.m[j] * r.c[j]) >> 4);             // (m c < 2^24 * m-tiles: sixteenths keep 256 requests' sum in range)
+        ms += r.m[j];
+    }
+    const uint32_t c_max = (uint32_t)plan_wave_max(cm);
+    if (c_max < 4) return 0;
+    const float W = 16.f * (float)(uint32_t)plan_wave_sum(ws);
+    const int M = plan_wave_sum(ms);
+    if (M > s.items_target) return 0;                              // more m-tiles than a round: nothing is split
+    auto T_of = [&](int k) { return (c_max + (uint32_t)k - 1) / (uint32_t)k; };
+    int n1 = M;
+    const int k1 = plan_largest_k(r, s, c_max, M, s.items_target, s.items_target / (M > 0 ? M : 1), &n1);
+    int k_best = k1;
+    if (s.items_split_cap > s.items_target && k1 < PLAN_MAX_SPLITS) {
+        // beyond a round the estimate is a + b k + c / k in k: least at k = sqrt(c / b), if the grid has room for that
+        float best = plan_estimate_us(W, n1, k1 == 1 ? c_max : T_of(k1), s);
+        const float b = PLAN_ITEM_US * (W / (float)c_max) / (float)s.items_target, c = 0.5f * (float)c_max * plan_tile_us(s);
+        int km = (int)(__builtin_sqrtf(c / (b > 1e-6f ? b : 1e-6f)) + 0.5f);
+        km = km > PLAN_MAX_SPLITS ? PLAN_MAX_SPLITS : km;
+        if (km > k1) {
+            int nm = plan_count(r, s, T_of(km));
+            if (nm > s.items_split_cap) km = plan_largest_k(r, s, c_max, M, s.items_split_cap, (k1 + km) >> 1, &nm);
+            if (km > k1) {
+                const float em = plan_estimate_us(W, nm, T_of(km), s);
+                if (em < best) { best = em; k_best = km; }
+            }
+        }
+    }
+    return k_best == 1 ? 0u : T_of(k_best);
+}
+
+struct PlanItem { int b, mt, split, nsplit, item_base; };      // b < 0: the item is beyond the batch's work
+// which (request, m-tile, split) work item `item` of a kv head is (wave-uniform result)
+template <int R> __device__ __forceinline__ PlanItem plan_locate(const PlanLane<R> &r, const BatchShape &s, uint32_t T, int item, int lane) {
+    PlanItem out{-1, 0, 0, 1, 0};
+    const PlanDivisor d = plan_divisor(T);
+    int ns[R], cn[R], tot = 0;
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        ns[j] = r.m[j] ? plan_splits_fast(r.c[j], d, s) : 0;
+        cn[j] = r.m[j] * ns[j];
+        tot += cn[j];
+    }
+    const int incl = plan_wave_scan(tot);
+    const uint64_t hit = __builtin_amdgcn_ballot_w64(incl > item);
+    if (!hit) return out;
+    const int idx = __builtin_ctzll(hit);
+    int first_item = __builtin_amdgcn_readlane(incl - tot, idx);
+    int rem = item - first_item;
+    int j = 0, nsel = __builtin_amdgcn_readlane(ns[0], idx);
+#pragma unroll
+    for (int k = 0; k + 1 < R; ++k) {
+        const int ck = __builtin_amdgcn_readlane(cn[k], idx), nk = __builtin_amdgcn_readlane(ns[k + 1], idx);
+        if (j == k && rem >= ck) { rem -= ck; first_item += ck; j = k + 1; nsel = nk; }
+    }
+    out.b = idx * R + j;
+    out.nsplit = nsel;
+    out.item_base = first_item;
+    out.mt = (int)plan_udiv((uint32_t)rem, (uint32_t)nsel);
+    out.split = rem - out.mt * nsel;
+    return out;
+}
+#endif  // __HIPCC__
+
+}  // namespace lazyattn

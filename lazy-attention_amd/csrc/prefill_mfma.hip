@@ -5,12 +5,12 @@
 namespace lazyattn {
 
 // instantiated in prefill_mfma_<type>[_<fp8 kind>].hip
-extern template int launch_mfma_family<bf16_t, 0>(const lazyattn_prefill_params &, int, int, int, int, hipStream_t);
-extern template int launch_mfma_family<bf16_t, 1>(const lazyattn_prefill_params &, int, int, int, int, hipStream_t);
-extern template int launch_mfma_family<bf16_t, 2>(const lazyattn_prefill_params &, int, int, int, int, hipStream_t);
-extern template int launch_mfma_family<f16_t, 0>(const lazyattn_prefill_params &, int, int, int, int, hipStream_t);
-extern template int launch_mfma_family<f16_t, 1>(const lazyattn_prefill_params &, int, int, int, int, hipStream_t);
-extern template int launch_mfma_family<f16_t, 2>(const lazyattn_prefill_params &, int, int, int, int, hipStream_t);
+extern template int launch_mfma_family<bf16_t, 0>(const lazyattn_prefill_params &, int, int, int, const BatchShape &, hipStream_t);
+extern template int launch_mfma_family<bf16_t, 1>(const lazyattn_prefill_params &, int, int, int, const BatchShape &, hipStream_t);
+extern template int launch_mfma_family<bf16_t, 2>(const lazyattn_prefill_params &, int, int, int, const BatchShape &, hipStream_t);
+extern template int launch_mfma_family<f16_t, 0>(const lazyattn_prefill_params &, int, int, int, const BatchShape &, hipStream_t);
+extern template int launch_mfma_family<f16_t, 1>(const lazyattn_prefill_params &, int, int, int, const BatchShape &, hipStream_t);
+extern template int launch_mfma_family<f16_t, 2>(const lazyattn_prefill_params &, int, int, int, const BatchShape &, hipStream_t);
 
 // ---- merge split-KV partials ----
 // The few fields the merge needs, not the whole parameter block.
@@ -18,37 +18,84 @@ struct MergeArgs {
     const void *workspace, *b_start_loc, *b_seq_len;
     void *o;
     int64_t o_stride[2];
-    int32_t num_tokens, num_q_heads, index_bits, skip_decode;
-    int32_t batch, token_grid;      // token_grid: the 32-token windows are cut over all tokens instead of per request
-    int32_t head_dim;               // elements of an output row (below HD when the partial rows are padded)
-    int32_t group, unit_cap;        // q-heads per kv-head; 32-row units per (request, kv-head) the main grid covers
+    int64_t items_per_kv;           // work items per kv head the partial rows are numbered by
+    int32_t num_q_heads, num_kv_heads, index_bits, skip_decode;
+    int32_t batch, head_dim;        // head_dim: elements of an output row (below HD when the partial rows are padded)
+    int32_t group, nc, n_mt;        // q-heads per kv-head; 32-row units per workgroup of the main kernel; its m-tiles per request
+    int32_t nsplit;                 // splits of every request (the plain grid)
     // xcd_map: one-dimensional grid in which the workgroups of a (request, kv-head) go to the XCD whose L2 the main
     // kernel's workgroups of that (request, kv-head) wrote the partial rows through (consecutive workgroup ids go
     // round the eight XCDs; a hint only: any placement gives the same result)
     int32_t xcd_map;
+    BatchShape bal;                 // items_cap > 0: the main kernel ran the balanced list, splits differ per request
     FastDiv by_group, by_windows, by_kv_heads;
 };
-// One workgroup = 32 consecutive tokens x one q-head; wave dt merges the columns dt*32 .. +31, lane (gh, l32) the
-// 4-column groups 8*i4 + 4*gh of token l32 -- the mapping of the main kernel's accumulators, so that a load
-// instruction reads one contiguous run of the partial rows as the main kernel wrote them (see its epilogue: the R
-// rows of a request's 32-token chunk are stored [head][piece][gh][row][4 halves]).  Log-sum-exps and row pieces of NB
-// splits (2, 4 or 8, the smallest that covers nsplit; more only when nsplit > 8) are requested together and before
-// the first use: one memory round trip per batch; batches are chained like the tiles of the main kernel, by a
-// running maximum.  The merged tile is turned through LDS (rows padded by 8 bytes: conflict-free both ways) so
-// that the output leaves as whole rows, 32 bytes per thread.  The windows are cut per request (grid y = request),
-// or over all tokens of the call when that grid is at most half as large (one long request among one-token
-// requests): then the 32 tokens of a workgroup need not belong to one request, and every lane finds its own by a
-// binary search of the offsets.
-template <typename T, int HD, int NB>
+
+// One workgroup = 32 consecutive tokens of one request x one q-head; wave dt merges the columns dt*32 .. +31, lane
+// (gh, l32) the 4-column groups 8*i4 + 4*gh of token l32 -- the mapping of the main kernel's accumulators, so that a
+// load instruction reads one contiguous run of the partial rows as the main kernel wrote them (see its epilogue: the
+// R rows of a unit are stored [piece][gh][row][4 halves] in the slot of (kv head, work item, wave)).
+// Log-sum-exps and row pieces of NB splits (2, 4 or 8, the smallest that covers the request's splits; more only
+// beyond eight) are requested together and before the first use: one memory round trip per batch; batches are
+// chained like the tiles of the main kernel, by a running maximum.  The merged tile is turned through LDS (rows
+// padded by 8 bytes: conflict-free both ways) so that the output leaves as whole rows, 32 bytes per thread.
+template <int D, int NB>
+__device__ __forceinline__ void merge_splits(const _Float16 *wb, const float2 *we, int64_t split_stride_rows, int R,
+                                             int nsplit, float (&o)[16], float &wsum) {
+    float mx = -INFINITY;
+    for (int s0 = 0; s0 < nsplit; s0 += NB) {
+        float2 e[NB];                                        // (log2-sum-exp, scale of the row's halves)
+        uint2 v[NB][4];
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+            const int64_t so = (int64_t)(s0 + j < nsplit ? s0 + j : nsplit - 1) * split_stride_rows;
+            e[j] = we[so];
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
+                typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+                const u32x2_t t = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t *>(wb + so * D + i4 * (2 * R * 4)));
+                v[j][i4] = make_uint2(t[0], t[1]);
+            }
+        }
+        float bm = e[0].x;
+#pragma unroll
+        for (int j = 1; j < NB; ++j) bm = fmaxf(bm, e[j].x);
+        const float m_new = fmaxf(mx, bm);
+        if (m_new == -INFINITY) continue;                    // nothing visible so far
+        const float keep = __builtin_amdgcn_exp2f(mx - m_new);   // mx = -inf -> 0
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[i] *= keep;
+        wsum *= keep;
+        mx = m_new;
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+            const float w = s0 + j < nsplit ? __builtin_amdgcn_exp2f(e[j].x - mx) : 0.f;
+            const float ws = w * e[j].y;
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
+                const f16x2_t a = *reinterpret_cast<const f16x2_t *>(&v[j][i4].x), c = *reinterpret_cast<const f16x2_t *>(&v[j][i4].y);
+                o[4 * i4] = fmaf(ws, (float)a[0], o[4 * i4]);
+                o[4 * i4 + 1] = fmaf(ws, (float)a[1], o[4 * i4 + 1]);
+                o[4 * i4 + 2] = fmaf(ws, (float)c[0], o[4 * i4 + 2]);
+                o[4 * i4 + 3] = fmaf(ws, (float)c[1], o[4 * i4 + 3]);
+            }
+            wsum += w;
+        }
+    }
+}
+
+template <typename T, int HD>
 __global__ void __launch_bounds__(HD * 2)
-prefill_combine_kernel(const MergeArgs p, const int nsplit) {
+prefill_combine_kernel(const MergeArgs p) {
     using E = Elem<T>;
     constexpr int D = HD, ROW = HD * 2 + 8;                   // bytes of a tile row in LDS
     __shared__ __attribute__((aligned(16))) uint8_t tile[UNIT * ROW];
     __shared__ int row_ok[UNIT];
     const int lane = threadIdx.x & 63, dt = threadIdx.x >> 6, l32 = lane & 31, gh = lane >> 5;
-    int h, b;
-    int64_t win;                                              // first token of the window
+    int h, b, nsplit = p.nsplit;
+    int64_t win;                                              // first token of the window, in its request
+    int64_t item0;                                            // first work item of the request (balanced) or of (request, m-tile 0)
+    int m_req = p.n_mt;                                       // m-tiles of the request the main grid covered
     if (p.xcd_map) {
         const uint32_t L = blockIdx.x, xcd = L & 7u, q = L >> 3;
         const uint32_t t = p.by_group.quot(q), hh = p.by_group.rem(q, t);
@@ -57,94 +104,54 @@ prefill_combine_kernel(const MergeArgs p, const int nsplit) {
         b = (int)p.by_kv_heads.quot(bg);
         h = (int)(p.by_kv_heads.rem(bg, (uint32_t)b) * (uint32_t)p.group + hh);
         win = (int64_t)w * UNIT;
+        item0 = (int64_t)b * p.n_mt * p.nsplit;
     } else {
         h = (int)(blockIdx.x % (unsigned)p.num_q_heads);
         win = (int64_t)(blockIdx.x / (unsigned)p.num_q_heads) * UNIT;
         b = blockIdx.y;
-    }
-    bool valid = true;
-    if (p.token_grid) {
-        valid = win + l32 < load_index(p.b_start_loc, p.batch, p.index_bits);
-        int lo = 0, hi = p.batch;                             // offsets[lo] <= token < offsets[hi]
-        while (hi - lo > 1) {
-            const int mid = (lo + hi) >> 1;
-            if (load_index(p.b_start_loc, mid, p.index_bits) <= win + l32) lo = mid; else hi = mid;
-        }
-        b = lo;
+        item0 = (int64_t)b * p.n_mt * p.nsplit;
     }
     // Exactly the rows the main kernel wrote partials for: anything else would merge whatever an earlier call
     // left in the workspace.
-    // (per-request windows: the request is the same for the whole workgroup and its three entries come as scalar
-    // loads in flight together -- this kernel is a chain of memory round trips and little else)
-    int64_t qs, qe, seq;
-    if (p.token_grid) {
-        qs = load_index(p.b_start_loc, b, p.index_bits);
-        qe = load_index(p.b_start_loc, b + 1, p.index_bits);
-        seq = load_index(p.b_seq_len, b, p.index_bits);
-    } else {
-        qs = load_index_uniform(p.b_start_loc, b, p.index_bits);
-        qe = load_index_uniform(p.b_start_loc, b + 1, p.index_bits);
-        seq = load_index_uniform(p.b_seq_len, b, p.index_bits);
-    }
+    // (the request is the same for the whole workgroup and its three entries come as scalar loads in flight
+    // together -- this kernel is a chain of memory round trips and little else)
+    const int64_t qs = load_index_uniform(p.b_start_loc, b, p.index_bits);
+    const int64_t qe = load_index_uniform(p.b_start_loc, b + 1, p.index_bits);
+    const int64_t seq = load_index_uniform(p.b_seq_len, b, p.index_bits);
     const int64_t q_len = qe - qs;
-    const int64_t tok0 = p.token_grid ? win : qs + win;       // token of the window's row 0
-    const int64_t row = tok0 + l32 - qs;
-    valid = valid && q_len > 0 && !(p.skip_decode && q_len == 1) && row < q_len &&
-            (row / UNIT) * p.group + h % p.group < p.unit_cap &&                 // (past the grid sized by max_q_len)
-            seq - q_len >= 0;
+    if (p.bal.items_cap > 0) {
+        // balanced list: where the request's work items start and how many splits it has was left at the head of the
+        // workspace by its first work item (a request without work has no record: its rows are not valid below,
+        // whatever an older call left in its place)
+        typedef const int32_t __attribute__((address_space(4))) *sptr_record;
+        const sptr_record rec = (sptr_record)((const int32_t *)p.workspace + (int64_t)b * 4);
+        item0 = rec[0];
+        nsplit = rec[1];
+        m_req = plan_mtiles((int32_t)q_len, (int32_t)(seq - q_len), p.bal);
+        if (m_req > 0 && nsplit <= 1) return;                 // its rows were written directly
+        if (nsplit < 1 || nsplit > PLAN_MAX_SPLITS || item0 < 0 || item0 + (int64_t)m_req * nsplit > p.items_per_kv) m_req = 0;
+    }
+    const int64_t row = win + l32;
+    const int unit = (int)(win / UNIT) * p.group + h % p.group;
+    const int mt = unit / p.nc, wave = unit % p.nc;
+    const bool valid = q_len > 0 && !(p.skip_decode && q_len == 1) && row < q_len && mt < m_req &&   // (past the grid sized by max_q_len)
+                       seq - q_len >= 0;
     float o[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) o[i] = 0.f;
     float wsum = 0.f;
     if (valid) {
-        const int64_t t0 = (row / UNIT) * UNIT;
-        const int R = (int)(q_len - t0 < UNIT ? q_len - t0 : UNIT), lr = (int)(row - t0);
-        const int64_t NTOK = p.num_tokens, split_rows = NTOK * p.num_q_heads;
-        const _Float16 *wo = (const _Float16 *)p.workspace;
-        const float2 *wl = reinterpret_cast<const float2 *>(wo + (int64_t)nsplit * split_rows * D);
-        const int64_t blk = (qs + t0) * p.num_q_heads + (int64_t)h * R;                  // in rows, split 0
-        const _Float16 *wb = wo + blk * D + (dt * 4 * 2 * R + gh * R + lr) * 4;
-        const float2 *we = wl + blk + lr;
-        float mx = -INFINITY;
-        for (int s0 = 0; s0 < nsplit; s0 += NB) {
-            float2 e[NB];                                        // (log2-sum-exp, scale of the row's halves)
-            uint2 v[NB][4];
-#pragma unroll
-            for (int j = 0; j < NB; ++j) {
-                const int64_t so = (int64_t)(s0 + j < nsplit ? s0 + j : nsplit - 1) * split_rows;
-                e[j] = we[so];
-#pragma unroll
-                for (int i4 = 0; i4 < 4; ++i4) {
-                    typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
-                    const u32x2_t t = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t *>(wb + so * D + i4 * (2 * R * 4)));
-                    v[j][i4] = make_uint2(t[0], t[1]);
-                }
-            }
-            float bm = e[0].x;
-#pragma unroll
-            for (int j = 1; j < NB; ++j) bm = fmaxf(bm, e[j].x);
-            const float m_new = fmaxf(mx, bm);
-            if (m_new == -INFINITY) continue;                    // nothing visible so far
-            const float keep = __builtin_amdgcn_exp2f(mx - m_new);   // mx = -inf -> 0
-#pragma unroll
-            for (int i = 0; i < 16; ++i) o[i] *= keep;
-            wsum *= keep;
-            mx = m_new;
-#pragma unroll
-            for (int j = 0; j < NB; ++j) {
-                const float w = s0 + j < nsplit ? __builtin_amdgcn_exp2f(e[j].x - mx) : 0.f;
-                const float ws = w * e[j].y;
-#pragma unroll
-                for (int i4 = 0; i4 < 4; ++i4) {
-                    const f16x2_t a = *reinterpret_cast<const f16x2_t *>(&v[j][i4].x), c = *reinterpret_cast<const f16x2_t *>(&v[j][i4].y);
-                    o[4 * i4] = fmaf(ws, (float)a[0], o[4 * i4]);
-                    o[4 * i4 + 1] = fmaf(ws, (float)a[1], o[4 * i4 + 1]);
-                    o[4 * i4 + 2] = fmaf(ws, (float)c[0], o[4 * i4 + 2]);
-                    o[4 * i4 + 3] = fmaf(ws, (float)c[1], o[4 * i4 + 3]);
-                }
-                wsum += w;
-            }
-        }
+        const int R = (int)(q_len - win < UNIT ? q_len - win : UNIT);
+        const int64_t slots = (int64_t)p.num_kv_heads * p.items_per_kv * p.nc;
+        const int64_t slot = ((int64_t)(h / p.group) * p.items_per_kv + item0 + (int64_t)mt * nsplit) * p.nc + wave;   // split 0
+        const _Float16 *wo = (const _Float16 *)((const uint8_t *)p.workspace + p.bal.table_bytes);
+        const float2 *wl = reinterpret_cast<const float2 *>(wo + slots * UNIT * D);
+        const _Float16 *wb = wo + slot * UNIT * D + (dt * 4 * 2 * R + gh * R + l32) * 4;
+        const float2 *we = wl + slot * UNIT + l32;
+        const int64_t stride = (int64_t)p.nc * UNIT;             // rows from one split's slot to the next
+        if (nsplit <= 2) merge_splits<D, 2>(wb, we, stride, R, nsplit, o, wsum);
+        else if (nsplit <= 4) merge_splits<D, 4>(wb, we, stride, R, nsplit, o, wsum);
+        else merge_splits<D, 8>(wb, we, stride, R, nsplit, o, wsum);
     }
     const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
 #pragma unroll
@@ -158,7 +165,7 @@ prefill_combine_kernel(const MergeArgs p, const int nsplit) {
     if (row_ok[r] && seg * 16 < p.head_dim) {                 // (beyond head_dim: padding columns of the partial rows)
         const uint4 a = *reinterpret_cast<const uint4 *>(tile + r * ROW + seg * 32);
         const uint4 c = *reinterpret_cast<const uint4 *>(tile + r * ROW + seg * 32 + 16);
-        T *op = (T *)p.o + (tok0 + r) * p.o_stride[0] + (int64_t)h * p.o_stride[1] + seg * 16;
+        T *op = (T *)p.o + (qs + win + r) * p.o_stride[0] + (int64_t)h * p.o_stride[1] + seg * 16;
         *reinterpret_cast<uint4 *>(op) = a;
         *reinterpret_cast<uint4 *>(op + 8) = c;
     }
@@ -211,6 +218,16 @@ static int mfma_waves(const lazyattn_prefill_params &p) {
     if (p.kernel == LAZYATTN_KERNEL_MFMA4) return 4;
     if (p.kernel == LAZYATTN_KERNEL_MFMA8) return 8;
     if (mfma_units(p) <= 4) return 4;
+    if (p.batch > 1 && p.batch <= PLAN_MAX_BATCH && p.num_splits <= 0) {
+        // Several requests, cut into work items on the device: the wider workgroup (a third less time per row) when
+        // the average request fills most of it and the batch has rows for a few dozen of them; else its rows would
+        // stand empty, or the few workgroups would need many splits.  (Measured over thirty ragged batches at
+        // Llama-3-8B geometry: the better shape in all but two, those within 7 %.)
+        const int group = p.num_q_heads / p.num_kv_heads;
+        const int64_t avg_units = (((int64_t)p.num_tokens / p.batch + UNIT - 1) / UNIT) * group;
+        const int64_t all_units = (((int64_t)p.num_tokens + UNIT - 1) / UNIT) * group;
+        return avg_units >= 6 && all_units >= 32 ? 8 : 4;
+    }
     const int64_t tiles = p.max_seq_len > 0 ? (p.max_seq_len + NT - 1) / NT : 64;
     auto cost = [&](int nw, double tile_us) {
         const int64_t s = mfma_splits(p, nw);
@@ -277,28 +294,75 @@ const char *mfma_unsupported_reason(const lazyattn_prefill_params &p) {
 }
 bool mfma_supports(const lazyattn_prefill_params &p) { return mfma_unsupported_reason(p) == nullptr; }
 
-// the choices launch_prefill_mfma() makes for a call: computing waves per workgroup (4 or 8) and key-axis splits
-void mfma_choices(const lazyattn_prefill_params &p, int *waves, int *splits) {
-    *waves = mfma_waves(p);
-    *splits = mfma_splits(p, *waves);
+
+
+// What one call launches: the workgroup shape, and either the plain grid (request, kv head, split, m-tile) with one
+// split count for every request -- a single request, or a caller who fixes the split count for a batch without
+// one-token requests -- or the balanced list of work items (batch_plan.hpp), whose splits are decided on the device.
+struct MfmaLaunch {
+    int nw, n_mt, nsplit;           // nsplit: of the plain grid (1 under the balanced list)
+    BatchShape bal;                 // items_cap > 0: balanced list
+    int64_t items_per_kv;           // work items per kv head the partial rows are numbered by (0: no partial rows)
+};
+static MfmaLaunch mfma_launch_shape(const lazyattn_prefill_params &p) {
+    MfmaLaunch L{};
+    L.nw = mfma_waves(p);
+    L.n_mt = mfma_mtiles(p, L.nw);
+    const int group = p.num_q_heads / p.num_kv_heads;
+    const int forced = p.num_splits > 0 ? (p.num_splits > PLAN_MAX_SPLITS ? PLAN_MAX_SPLITS : p.num_splits) : 0;
+    const bool balanced = p.batch > 1 && p.batch <= PLAN_MAX_BATCH && (forced == 0 || mfma_compact(p, L.nw));
+    auto plain = [&] {
+        L.nsplit = mfma_splits(p, L.nw);
+        L.items_per_kv = L.nsplit > 1 ? (int64_t)p.batch * L.n_mt * L.nsplit : 0;
+        return L;
+    };
+    if (!balanced) return plain();
+    L.nsplit = 1;
+    const int64_t m_bound = [&] {                                    // at least the m-tiles the batch really has
+        const int64_t by_chunks = mfma_mtiles_bound(p, L.nw), by_requests = (int64_t)p.batch * L.n_mt;
+        return by_chunks < by_requests ? by_chunks : by_requests;
+    }();
+    // One round of the chip's compute units is what the device cuts a batch for (batch_plan.hpp); a batch with more
+    // m-tiles than that is not split, and the grid has room for it.
+    // Room beyond one round -- up to every m-tile cut in four, and three rounds at most -- is made when one round
+    // could not even cut every m-tile in two: it would then leave the long requests whole.  (Work items the
+    // device does not use return after their scan of the batch: they cost a little at the launch's end, so the grid
+    // is not made larger than the device can be expected to fill.)
+    const int64_t target = (device_cus() + p.num_kv_heads - 1) / p.num_kv_heads;
+    int64_t split_cap = target;
+    if (forced) split_cap = m_bound * forced;
+    else if (2 * m_bound > target) split_cap = 4 * m_bound < 3 * target ? 4 * m_bound : 3 * target;
+    const int64_t cap = split_cap < m_bound ? m_bound : split_cap;
+    // (no records when nothing is split: there is no merge to read them, and no workspace to hold them)
+    const int64_t table_bytes = forced == 1 ? 0 : ((int64_t)p.batch * (int64_t)sizeof(PlanRecord) + 255) / 256 * 256;
+    if (cap > 0x3fffffff || table_bytes > 0x3fffffff) return plain();     // (beyond any real batch)
+    L.bal = BatchShape{group, L.nw, L.n_mt, p.skip_decode, (int32_t)cap, (int32_t)target, (int32_t)split_cap, forced,
+                       (int32_t)table_bytes};
+    // the slots of the partial rows: a batch that is split has at most split_cap items per kv head
+    L.items_per_kv = forced == 1 ? 0 : split_cap;
+    return L;
+}
+// the requests' records (balanced list) and the partial rows
+static size_t mfma_partial_bytes(const lazyattn_prefill_params &p, const MfmaLaunch &L) {
+    if (L.items_per_kv <= 0) return 0;
+    return (size_t)L.bal.table_bytes + (size_t)p.num_kv_heads * (size_t)L.items_per_kv * L.nw * UNIT * partial_row_bytes(p);
 }
 
-size_t mfma_workspace_bytes(const lazyattn_prefill_params &p) {
-    const int nw = mfma_waves(p);
-    const int ns = mfma_splits(p, nw);
-    if (ns <= 1) return 0;
-    return (size_t)ns * (size_t)p.num_tokens * p.num_q_heads * partial_row_bytes(p);
+size_t mfma_workspace_bytes(const lazyattn_prefill_params &p) { return mfma_partial_bytes(p, mfma_launch_shape(p)); }
+
+// the choices a call gets: computing waves per workgroup (4 or 8) and key-axis splits (0: decided per request on the device)
+void mfma_choices(const lazyattn_prefill_params &p, int *waves, int *splits) {
+    const MfmaLaunch L = mfma_launch_shape(p);
+    *waves = L.nw;
+    *splits = L.bal.items_cap > 0 ? L.bal.forced_splits : L.nsplit;
 }
 
 int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
-    const int nw = mfma_waves(p);
-    const int nsplit = mfma_splits(p, nw);
-    const int n_mt = mfma_mtiles(p, nw);
-    const int64_t bound = mfma_mtiles_bound(p, nw);
-    const int mt_total = mfma_compact(p, nw) && bound <= 0x7fffffff ? (int)bound : 0;
+    const MfmaLaunch L = mfma_launch_shape(p);
+    const int nw = L.nw, nsplit = L.nsplit, n_mt = L.n_mt;
     const int phases = p.phases ? p.phases : LAZYATTN_PHASE_ALL;
-    if (nsplit > 1) {
-        const size_t need = (size_t)nsplit * (size_t)p.num_tokens * p.num_q_heads * partial_row_bytes(p);
+    if (mfma_partial_bytes(p, L) > 0) {
+        const size_t need = mfma_partial_bytes(p, L);
         if (!p.workspace || (size_t)p.workspace_bytes < need) return LAZYATTN_E_WORKSPACE;
         if (((uintptr_t)p.workspace) & 15) return LAZYATTN_E_WORKSPACE;
     }
@@ -306,40 +370,35 @@ int launch_prefill_mfma(const lazyattn_prefill_params &p, hipStream_t stream) {
         const bool f16 = p.dtype == LAZYATTN_F16;
         int rc;
         if (p.cache_dtype == LAZYATTN_FP8_E4M3)
-            rc = f16 ? launch_mfma_family<f16_t, 1>(p, nw, nsplit, n_mt, mt_total, stream) : launch_mfma_family<bf16_t, 1>(p, nw, nsplit, n_mt, mt_total, stream);
+            rc = f16 ? launch_mfma_family<f16_t, 1>(p, nw, nsplit, n_mt, L.bal, stream) : launch_mfma_family<bf16_t, 1>(p, nw, nsplit, n_mt, L.bal, stream);
         else if (p.cache_dtype == LAZYATTN_FP8_E5M2)
-            rc = f16 ? launch_mfma_family<f16_t, 2>(p, nw, nsplit, n_mt, mt_total, stream) : launch_mfma_family<bf16_t, 2>(p, nw, nsplit, n_mt, mt_total, stream);
+            rc = f16 ? launch_mfma_family<f16_t, 2>(p, nw, nsplit, n_mt, L.bal, stream) : launch_mfma_family<bf16_t, 2>(p, nw, nsplit, n_mt, L.bal, stream);
         else
-            rc = f16 ? launch_mfma_family<f16_t, 0>(p, nw, nsplit, n_mt, mt_total, stream) : launch_mfma_family<bf16_t, 0>(p, nw, nsplit, n_mt, mt_total, stream);
+            rc = f16 ? launch_mfma_family<f16_t, 0>(p, nw, nsplit, n_mt, L.bal, stream) : launch_mfma_family<bf16_t, 0>(p, nw, nsplit, n_mt, L.bal, stream);
         if (rc != LAZYATTN_OK) return rc;
     }
-    if (nsplit > 1 && (phases & LAZYATTN_PHASE_COMBINE)) {
-        // windows per request x requests, or windows over all tokens when that is at most half as many
-        const int token_grid = p.batch > 1 && 2 * (int64_t)p.num_tokens <= (int64_t)p.batch * p.max_q_len;
-        // 32 tokens x one q-head per workgroup
-        const int64_t windows = ((int64_t)(token_grid ? p.num_tokens : p.max_q_len) + UNIT - 1) / UNIT;
+    if (L.items_per_kv > 0 && (phases & LAZYATTN_PHASE_COMBINE)) {
         const int group = p.num_q_heads / p.num_kv_heads;
-        // (the condition under which the main kernel gives a (request, kv-head) to one XCD)
-        const int xcd_map = !token_grid && mt_total == 0 && ((p.batch * p.num_kv_heads) & 7) == 0 &&
-                            windows * p.num_q_heads * p.batch <= 0x7fffffff;
-        const MergeArgs m{p.workspace, p.b_start_loc, p.b_seq_len, p.o, {p.o_stride[0], p.o_stride[1]}, p.num_tokens, p.num_q_heads,
-                          p.index_bits, p.skip_decode, p.batch, token_grid, p.head_dim, group,
-                          mt_total > 0 ? 0x7fffffff : n_mt * nw, xcd_map,
+        // 32 tokens x one q-head per workgroup: windows per request x requests
+        const int64_t windows = ((int64_t)p.max_q_len + UNIT - 1) / UNIT;
+        // (the condition under which the main kernel gives a (request, kv-head) to one XCD; under the balanced list
+        // a kv head stays on one XCD, which the same numbering gives when the kv heads are a multiple of eight)
+        const int xcd_map = ((p.batch * p.num_kv_heads) & 7) == 0 && windows * p.num_q_heads * p.batch <= 0x7fffffff;
+        if (windows * p.num_q_heads > 0x7fffffff) return LAZYATTN_E_SHAPE;
+        const MergeArgs m{p.workspace, p.b_start_loc, p.b_seq_len, p.o, {p.o_stride[0], p.o_stride[1]}, L.items_per_kv,
+                          p.num_q_heads, p.num_kv_heads, p.index_bits, p.skip_decode, p.batch, p.head_dim, group, nw, n_mt,
+                          nsplit, xcd_map, L.bal,
                           FastDiv((uint32_t)group), FastDiv((uint32_t)windows), FastDiv((uint32_t)p.num_kv_heads)};
         const dim3 grid = xcd_map ? dim3((unsigned)(windows * p.num_q_heads * p.batch))
-                                  : dim3((unsigned)(windows * p.num_q_heads), token_grid ? 1 : p.batch);
+                                  : dim3((unsigned)(windows * p.num_q_heads), p.batch);
         const bool f16 = p.dtype == LAZYATTN_F16;
-#define LAZYATTN_COMBINE(HD, NB)                                                                                  \
-    {                                                                                                             \
-        if (f16) hipLaunchKernelGGL((prefill_combine_kernel<f16_t, HD, NB>), grid, dim3(HD * 2), 0, stream, m, nsplit); \
-        else hipLaunchKernelGGL((prefill_combine_kernel<bf16_t, HD, NB>), grid, dim3(HD * 2), 0, stream, m, nsplit);    \
-    }
-        if (p.head_dim == 64) {
-            if (nsplit <= 2) LAZYATTN_COMBINE(64, 2) else if (nsplit <= 4) LAZYATTN_COMBINE(64, 4) else LAZYATTN_COMBINE(64, 8)
+        if (tile_dim(p) == 64) {
+            if (f16) hipLaunchKernelGGL((prefill_combine_kernel<f16_t, 64>), grid, dim3(128), 0, stream, m);
+            else hipLaunchKernelGGL((prefill_combine_kernel<bf16_t, 64>), grid, dim3(128), 0, stream, m);
         } else {
-            if (nsplit <= 2) LAZYATTN_COMBINE(128, 2) else if (nsplit <= 4) LAZYATTN_COMBINE(128, 4) else LAZYATTN_COMBINE(128, 8)
+            if (f16) hipLaunchKernelGGL((prefill_combine_kernel<f16_t, 128>), grid, dim3(256), 0, stream, m);
+            else hipLaunchKernelGGL((prefill_combine_kernel<bf16_t, 128>), grid, dim3(256), 0, stream, m);
         }
-#undef LAZYATTN_COMBINE
         if (hipGetLastError() != hipSuccess) return LAZYATTN_E_LAUNCH;
     }
     return LAZYATTN_OK;

@@ -2,5 +2,5 @@
 #include "prefill_mfma_kernel.hpp"
 
 namespace lazyattn {
-template int launch_mfma_family<bf16_t, 0>(const lazyattn_prefill_params &, int, int, int, int, hipStream_t);
+template int launch_mfma_family<bf16_t, 0>(const lazyattn_prefill_params &, int, int, int, const BatchShape &, hipStream_t);
 }  // namespace lazyattn

@@ -2,5 +2,5 @@
 #include "prefill_mfma_kernel.hpp"
 
 namespace lazyattn {
-template int launch_mfma_family<f16_t, 1>(const lazyattn_prefill_params &, int, int, int, int, hipStream_t);
+template int launch_mfma_family<f16_t, 1>(const lazyattn_prefill_params &, int, int, int, const BatchShape &, hipStream_t);
 }  // namespace lazyattn

@@ -34,6 +34,7 @@
 #include "common.hpp"
 #include "elem16.hpp"
 #include "fastdiv.hpp"
+#include "batch_plan.hpp"
 #include <atomic>
 #include <type_traits>
 
@@ -226,7 +227,7 @@ template <int HD> constexpr int lds_bytes(int nc) {      // K and V tiles + Q^T 
 // halves of the real head at (0 .., 64 ..) so that the rotation pairs stay (d, 64 + d)
 template <int NC, int HD, int FP8, bool WIN, bool PAD, typename T, typename TT>
 __global__ void __launch_bounds__((NC + gather_waves(NC, HD)) * 64)
-prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int n_mt, const int mt_total, const MfmaDivs dv) {
+prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int n_mt, const BatchShape bal, const MfmaDivs dv) {
     using G = Geo<HD>;
     constexpr int D = HD, HALF = HD / 2;
     const int Dr = PAD ? p.head_dim : D, HALFr = Dr / 2, CPr = Dr / 16;   // real head size, its half, its chunk pairs
@@ -257,59 +258,42 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
 
     // ---- work item: the m-tiles of one (request, kv-head, split) land on the same XCD ----
     const int group = p.num_q_heads / p.num_kv_heads;
-    int mt, split, g, b;
-    if (mt_total > 0) {
-        // Compact list: the grid holds (kv head, split, I) for I below a host-side bound on the number of m-tiles
-        // of all requests together; I is resolved to (request, m-tile) here from the token offsets.  Used when
-        // most (request, m-tile) pairs of the plain mapping would be empty: requests with one new token next to
-        // a long one.  Workgroups of one kv head stay on one XCD.
+    // mt, split, g, b: this workgroup's m-tile, key-axis split, kv head and request; nsplit_wg: the splits of its
+    // request; witem: its number among the work items of its kv head (where its partial rows go)
+    int mt, split, g, b, nsplit_wg = nsplit, witem;
+    uint32_t split_mul = 0;                          // ceil(2^32 / nsplit_wg) under the balanced list (0: one split)
+    if (bal.items_cap > 0) {
+        // Balanced list: the grid holds (kv head, I) for I below the number of work items the host made room for; which
+        // (request, m-tile, split) item I is, follows from all the requests' lengths (batch_plan.hpp): the first wave
+        // works it out and leaves it in LDS for the others, which meanwhile form the per-lane constants below.
+        // Workgroups of one kv head stay on one XCD.
         const int L = blockIdx.x, hkv = p.num_kv_heads;
-        int q;
-        if ((hkv & 7) == 0) { g = (L & 7) + 8 * ((L >> 3) % (hkv >> 3)); q = (L >> 3) / (hkv >> 3); }
-        else { g = L % hkv; q = L / hkv; }
-        split = q % nsplit;
-        const int item = q / nsplit;
-        int base = 0;
-        b = -1; mt = 0;
-        // 256 requests per round, four per lane: their offsets are requested together (one memory round trip),
-        // the m-tile counts are summed per lane, scanned over the wave, and the hit is located inside its lane
-        for (int c = 0; c < p.batch; c += 256) {
-            const int r0 = c + lane * 4;
-            int64_t off[5];
-#pragma unroll
-            for (int j = 0; j < 5; ++j) {
-                const int rb = r0 + j;
-                off[j] = load_index(p.b_start_loc, rb < p.batch ? rb : p.batch, p.index_bits);
+        if ((hkv & 7) == 0) { g = (L & 7) + 8 * ((L >> 3) % (hkv >> 3)); witem = (L >> 3) / (hkv >> 3); }
+        else { g = L % hkv; witem = L / hkv; }
+        int *found = reinterpret_cast<int *>(lds + lds_bytes<HD>(NC) - 24);      // (behind the page limits, unused otherwise)
+        if (wave == 0) {
+            const PlanTables tabs{p.b_start_loc, p.b_seq_len, p.batch, p.index_bits};
+            PlanItem it;
+            if (p.batch <= 64) {                                 // one request per lane: a quarter of the arithmetic
+                const PlanLane<1> reqs = plan_load<1>(tabs, bal, lane);
+                it = plan_locate(reqs, bal, plan_target(reqs, bal), witem, lane);
+            } else {
+                const PlanLane<4> reqs = plan_load<4>(tabs, bal, lane);
+                it = plan_locate(reqs, bal, plan_target(reqs, bal), witem, lane);
             }
-            int cn[4], tot = 0;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int ql = r0 + j < p.batch ? (int)(off[j + 1] - off[j]) : 0;
-                cn[j] = (ql > 0 && !(p.skip_decode && ql == 1)) ? (((ql + UNIT - 1) / UNIT) * group + NC - 1) / NC : 0;
-                tot += cn[j];
+            if (lane == 0) {
+                found[0] = it.b; found[1] = it.mt; found[2] = it.split; found[3] = it.nsplit;
+                found[4] = it.nsplit > 1 ? (int)(0xffffffffu / (uint32_t)it.nsplit + 1u) : 0;
+                // the first work item of a request tells the merge where the request's items start and how many
+                // splits it has
+                if (it.b >= 0 && it.mt == 0 && it.split == 0 && g == 0 && bal.table_bytes > 0)
+                    reinterpret_cast<PlanRecord *>(p.workspace)[it.b] = PlanRecord{it.item_base, it.nsplit, 0, 0};
             }
-            int incl = tot;                                       // inclusive prefix sum over the wave
-#pragma unroll
-            for (int d = 1; d < 64; d <<= 1) {
-                const int up = __shfl_up(incl, d);
-                if (lane >= d) incl += up;
-            }
-            const uint64_t hit = __builtin_amdgcn_ballot_w64(base + incl > item);
-            if (hit) {
-                const int idx = __builtin_ctzll(hit);
-                int rem = item - (base + __builtin_amdgcn_readlane(incl - tot, idx));
-                const int c0 = __builtin_amdgcn_readlane(cn[0], idx), c1 = __builtin_amdgcn_readlane(cn[1], idx),
-                          c2 = __builtin_amdgcn_readlane(cn[2], idx);
-                int j = 0;
-                if (rem >= c0) { rem -= c0; j = 1; if (rem >= c1) { rem -= c1; j = 2; if (rem >= c2) { rem -= c2; j = 3; } } }
-                b = c + idx * 4 + j;
-                mt = rem;
-                break;
-            }
-            base += __builtin_amdgcn_readlane(incl, 63);
         }
+        __syncthreads();
+        b = uniform(found[0]); mt = uniform(found[1]); split = uniform(found[2]); nsplit_wg = uniform(found[3]);
+        split_mul = (uint32_t)uniform(found[4]);
         if (b < 0) return;
-        b = uniform(b); mt = uniform(mt);
     } else {
         const int n_groups = p.batch * p.num_kv_heads * nsplit;
         int kvgrp;
@@ -334,6 +318,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         split = (int)dv.nsplit.rem(kvgrp, bg);
         b = (int)dv.kv_heads.quot(bg);
         g = (int)dv.kv_heads.rem(bg, b);
+        witem = (b * n_mt + mt) * nsplit + split;
     }
 
     // The request's lengths are requested here, ahead of the gathering waves' per-lane constants: nothing in
@@ -464,8 +449,16 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     auto tile_at = [&](uint32_t c) -> int {        // first tile whose cost interval ends after c
         return skip_ctx + skip_new + (c <= (uint32_t)live_ctx ? (int)c : live_ctx + (int)((c - (uint32_t)live_ctx) / NEW_COST));
     };
-    const int tile_begin = tile_at(dv.nsplit.quot(cost * (uint32_t)split));
-    const int tile_end = split + 1 == nsplit ? n_ctx_tiles + n_new_tiles : tile_at(dv.nsplit.quot(cost * (uint32_t)(split + 1)));
+    // Equal shares of the cost, the first (cost mod splits) of them one longer.  The split count is the request's own
+    // under the balanced list, where no multiplier can come from the host: the wave that located the work item left
+    // ceil(2^32 / splits), exact for costs below 2^26 and at most 64 splits.  (A division here -- forty instructions
+    // from a cold instruction cache on every wave's way to its first memory request -- cost 0.5 us of an 18 us launch.)
+    const uint32_t share = bal.items_cap > 0 ? (split_mul ? FastDiv::mulhi(cost, split_mul) : cost) : dv.nsplit.quot(cost);
+    const uint32_t longer = cost - share * (uint32_t)nsplit_wg;
+    const uint32_t c_lo = (uint32_t)split * share + ((uint32_t)split < longer ? (uint32_t)split : longer);
+    const uint32_t c_hi = c_lo + share + ((uint32_t)split < longer ? 1u : 0u);
+    const int tile_begin = tile_at(c_lo);
+    const int tile_end = split + 1 == nsplit_wg ? n_ctx_tiles + n_new_tiles : tile_at(c_hi);
 
     // ---- page metadata, fetched ahead of its use ----
     // Gathering wave w owns page w of every tile, so it needs one block-table entry, one
@@ -1228,7 +1221,7 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
     if (!row_ok) return;
     const float out_scale = FOLD ? v_scale : 1.f;
     const float inv = l_run > 0.f ? out_scale / l_run : 0.f;
-    if (nsplit == 1) {
+    if (nsplit_wg == 1) {
         T *op = (T *)p.o + (qs + row) * p.o_stride[0] + (int64_t)h * p.o_stride[1];
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
@@ -1255,18 +1248,20 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
         eb = eb > 252u ? 252u : eb;
         const float down = __uint_as_float((253u - eb) << 23) * inv;   // 2^-(eb-126) / l
         const float up = __uint_as_float((eb + 1u) << 23);            // 2^(eb-126)
-        // Where the rows go: the R rows of a 32-token chunk (R < 32 only at a request's end), all q-heads, fill
-        // the same stretch of the workspace as in [token][head][D] order, but laid out [head][piece][gh][row][4]:
-        // one store instruction of this wave then writes one contiguous run (512 bytes for a full chunk) instead of
-        // 32 runs of 16 bytes a row apart -- the partial rows leave in a quarter of the time (measured with the
-        // bytes kept and only the addresses changed: 1.8 of the 3.2 us the stores cost at 5 K keys).  The merge
-        // kernel reads with the same lane mapping.  (piece = the 8 columns dt*32 + 8*i4 .. +7, gh its half)
-        const int64_t NTOK = p.num_tokens;
-        _Float16 *wo = (_Float16 *)p.workspace;
-        float2 *wl = reinterpret_cast<float2 *>(wo + (int64_t)nsplit * NTOK * p.num_q_heads * D);
+        // Where the rows go: every computing wave of every work item has a slot of 32 rows, numbered
+        // (kv head, work item of that kv head, wave); inside it the R rows of the unit (R < 32 only at a request's
+        // end) are laid out [piece][gh][row][4]: one store instruction of this wave then writes one contiguous run
+        // (512 bytes for a full unit) instead of 32 runs of 16 bytes a row apart -- the partial rows leave in a
+        // quarter of the time (measured with the bytes kept and only the addresses changed: 1.8 of the 3.2 us the
+        // stores cost at 5 K keys).  The merge kernel reads with the same lane mapping.  (piece = the 8 columns
+        // dt*32 + 8*i4 .. +7, gh its half)
+        const int64_t items_per_kv = bal.items_cap > 0 ? (int64_t)bal.items_split_cap : (int64_t)p.batch * n_mt * nsplit;
+        const int64_t slots = (int64_t)p.num_kv_heads * items_per_kv * NC;
+        const int64_t slot = ((int64_t)g * items_per_kv + witem) * NC + wave;
+        _Float16 *wo = (_Float16 *)((uint8_t *)p.workspace + bal.table_bytes);
+        float2 *wl = reinterpret_cast<float2 *>(wo + slots * UNIT * D);
         const int R = q_len - t0 < UNIT ? q_len - t0 : UNIT;
-        const int64_t blk = ((int64_t)split * NTOK + (qs + t0)) * p.num_q_heads + (int64_t)h * R;   // in rows
-        _Float16 *wb = wo + blk * D + (gh * R + l32) * 4;
+        _Float16 *wb = wo + slot * UNIT * D + (gh * R + l32) * 4;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -1278,12 +1273,12 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
                     make_uint2(*reinterpret_cast<const uint32_t *>(&hl), *reinterpret_cast<const uint32_t *>(&hh));
             }
         if (gh == 0)
-            wl[blk + l32] = make_float2(l_run > 0.f ? m_ref + __builtin_amdgcn_logf(l_run) : -INFINITY, up);
+            wl[slot * UNIT + l32] = make_float2(l_run > 0.f ? m_ref + __builtin_amdgcn_logf(l_run) : -INFINITY, up);
     }
 }
 
 template <int NC, int HD, int FP8, bool WIN, bool PAD, typename T, typename TT>
-int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt, int mt_total, hipStream_t stream) {
+int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt, const BatchShape &bal, hipStream_t stream) {
     auto kern = prefill_mfma_kernel<NC, HD, FP8, WIN, PAD, T, TT>;
     constexpr int LDS_BYTES = lds_bytes<HD>(NC);
     // the attribute belongs to the device's copy of the kernel: once per device, on the caller's current device
@@ -1296,37 +1291,37 @@ int launch_mfma_t(const lazyattn_prefill_params &p, int nsplit, int n_mt, int mt
             return LAZYATTN_E_LAUNCH;
         attr_set[dev].store(true, std::memory_order_release);
     }
-    const int64_t nb = (int64_t)p.num_kv_heads * nsplit * (mt_total > 0 ? (int64_t)mt_total : (int64_t)p.batch * n_mt);
+    const int64_t nb = (int64_t)p.num_kv_heads * (bal.items_cap > 0 ? (int64_t)bal.items_cap : (int64_t)nsplit * p.batch * n_mt);
     if (nb <= 0 || nb > 0x7fffffff) return LAZYATTN_E_SHAPE;
     const MfmaDivs dv{FastDiv((uint32_t)n_mt), FastDiv((uint32_t)nsplit), FastDiv((uint32_t)p.num_kv_heads),
                       FastDiv((uint32_t)(p.num_q_heads / p.num_kv_heads))};
-    hipLaunchKernelGGL(kern, dim3((unsigned)nb), dim3((NC + gather_waves(NC, HD)) * 64), LDS_BYTES, stream, p, nsplit, n_mt, mt_total, dv);
+    hipLaunchKernelGGL(kern, dim3((unsigned)nb), dim3((NC + gather_waves(NC, HD)) * 64), LDS_BYTES, stream, p, nsplit, n_mt, bal, dv);
     return hipGetLastError() == hipSuccess ? LAZYATTN_OK : LAZYATTN_E_LAUNCH;
 }
 
 // table type: the element type or float
 template <int NC, int HD, int FP8, bool WIN, bool PAD, typename T>
-int launch_mfma_table(const lazyattn_prefill_params &p, int nsplit, int n_mt, int mt_total, hipStream_t stream) {
-    if (p.table_dtype == LAZYATTN_F32) return launch_mfma_t<NC, HD, FP8, WIN, PAD, T, float>(p, nsplit, n_mt, mt_total, stream);
-    return launch_mfma_t<NC, HD, FP8, WIN, PAD, T, T>(p, nsplit, n_mt, mt_total, stream);
+int launch_mfma_table(const lazyattn_prefill_params &p, int nsplit, int n_mt, const BatchShape &bal, hipStream_t stream) {
+    if (p.table_dtype == LAZYATTN_F32) return launch_mfma_t<NC, HD, FP8, WIN, PAD, T, float>(p, nsplit, n_mt, bal, stream);
+    return launch_mfma_t<NC, HD, FP8, WIN, PAD, T, T>(p, nsplit, n_mt, bal, stream);
 }
 // head size and sliding window
 template <int NC, int FP8, typename T>
-int launch_mfma_shape(const lazyattn_prefill_params &p, int nsplit, int n_mt, int mt_total, hipStream_t stream) {
+int launch_mfma_shape(const lazyattn_prefill_params &p, int nsplit, int n_mt, const BatchShape &bal, hipStream_t stream) {
     if (p.head_dim == 64)
-        return p.sliding_window > 0 ? launch_mfma_table<NC, 64, FP8, true, false, T>(p, nsplit, n_mt, mt_total, stream)
-                                    : launch_mfma_table<NC, 64, FP8, false, false, T>(p, nsplit, n_mt, mt_total, stream);
+        return p.sliding_window > 0 ? launch_mfma_table<NC, 64, FP8, true, false, T>(p, nsplit, n_mt, bal, stream)
+                                    : launch_mfma_table<NC, 64, FP8, false, false, T>(p, nsplit, n_mt, bal, stream);
     // other head sizes: the 128-wide kernel with padding (built with the window code, which a window of 0 switches off)
-    if (p.head_dim != 128) return launch_mfma_table<NC, 128, FP8, true, true, T>(p, nsplit, n_mt, mt_total, stream);
-    if (p.sliding_window > 0) return launch_mfma_table<NC, 128, FP8, true, false, T>(p, nsplit, n_mt, mt_total, stream);
-    return launch_mfma_table<NC, 128, FP8, false, false, T>(p, nsplit, n_mt, mt_total, stream);
+    if (p.head_dim != 128) return launch_mfma_table<NC, 128, FP8, true, true, T>(p, nsplit, n_mt, bal, stream);
+    if (p.sliding_window > 0) return launch_mfma_table<NC, 128, FP8, true, false, T>(p, nsplit, n_mt, bal, stream);
+    return launch_mfma_table<NC, 128, FP8, false, false, T>(p, nsplit, n_mt, bal, stream);
 }
 // Every kernel of one (element type, cache page kind: 0 the element type, 1 fp8 e4m3, 2 fp8 e5m2); nw = computing
 // waves per workgroup (4 or 8).  Explicitly instantiated, one translation unit each.
 template <typename T, int FP8>
-int launch_mfma_family(const lazyattn_prefill_params &p, int nw, int nsplit, int n_mt, int mt_total, hipStream_t stream) {
-    return nw == 8 ? launch_mfma_shape<8, FP8, T>(p, nsplit, n_mt, mt_total, stream)
-                   : launch_mfma_shape<4, FP8, T>(p, nsplit, n_mt, mt_total, stream);
+int launch_mfma_family(const lazyattn_prefill_params &p, int nw, int nsplit, int n_mt, const BatchShape &bal, hipStream_t stream) {
+    return nw == 8 ? launch_mfma_shape<8, FP8, T>(p, nsplit, n_mt, bal, stream)
+                   : launch_mfma_shape<4, FP8, T>(p, nsplit, n_mt, bal, stream);
 }
 
 }  // namespace lazyattn
