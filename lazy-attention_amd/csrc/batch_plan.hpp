@@ -8,9 +8,12 @@
 // lengths -- one memory round trip, which its own lengths cost anyway -- and derives, identically everywhere:
 //   m_j     m-tiles (workgroups per kv head and split) of request j
 //   c_j     cost of its key axis in 64-key tiles (a new-token tile counts as three)
-//   T       tiles per work item: ceil(c_max / k) for the largest k = 1 .. 64 (splits of the longest request) with
-//           which the items still fit one round of the chip's compute units -- found by bisection, the item count
-//           being monotonic in k; no request is split when the m-tiles alone exceed a round
+//   T       tiles per work item: the work items of a launch run in rounds of one per compute unit, and being of
+//           about T tiles each they finish round by round; for every number of rounds r the grid has room for, the
+//           batch's W = sum m_j c_j tiles give the T that fills r rounds, W / (r rounds' items - half the m-tiles),
+//           and r (T tile time + a work item's fixed time) estimates the launch; for the r with the lowest estimate,
+//           T starts at the value whose item count fits for certain, W / (items - m-tiles), and is lowered in up to
+//           three probes of the real item count toward the value that fills the rounds exactly
 //   s_j     = ceil(c_j / T) key-axis splits of request j (at least two tiles each, at most 64)
 // and from the prefix sums of m_j s_j which (request, m-tile, split) its work item is.  The first work item of every
 // request leaves (first item, splits, m-tiles) of the request in a small table at the head of the workspace, where
@@ -76,6 +79,65 @@ LAZYATTN_HD int plan_splits(uint32_t cost, uint32_t T, const BatchShape &s) {
     n = n < most ? n : most;
     n = n < (uint32_t)PLAN_MAX_SPLITS ? n : (uint32_t)PLAN_MAX_SPLITS;
     return (int)(n < 1 ? 1 : n);
+}
+
+// Per workgroup a 64-key tile takes about 1.34 us in the four-unit shape and 1.98 us in the eight-unit shape, and a
+// work item some 6 us of prologue, first-tile latency, epilogue and this planning (measured on an MI355X with 16-bit
+// operands at head size 128).
+constexpr float PLAN_ITEM_US = 6.f;
+constexpr int PLAN_PROBES = 3;
+LAZYATTN_HD float plan_tile_us(const BatchShape &s) { return s.nc == 8 ? 1.98f : 1.34f; }
+LAZYATTN_HD float plan_ratio(float a, float b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return a * __builtin_amdgcn_rcpf(b);                 // (every workgroup forms the same value; what must hold is checked by counting)
+#else
+    return a / b;
+#endif
+}
+LAZYATTN_HD uint32_t plan_clamp_tiles(float t, uint32_t c_max) {
+    const uint32_t T = t < 2.f ? 2u : (t < 16777216.f ? (uint32_t)t : (1u << 24));
+    return T < c_max ? T : c_max;
+}
+// T for the whole batch (0: no request is split).  W: sum of m_j c_j, M: sum of m_j, c_max: largest c_j,
+// count(T): the work items per kv head a given T makes -- on the device a reduction over the scanning wave.
+// Whatever the approximations in W and the quotients: a T is only returned after count(T) was seen to fit.
+template <class Count>
+LAZYATTN_HD uint32_t plan_choose_tiles(float W, int M, uint32_t c_max, const BatchShape &s, Count count) {
+    if (s.forced_splits > 0 || c_max < 4 || M <= 0 || s.items_target <= 0 || M >= s.items_split_cap) return 0;
+    const int target = s.items_target;
+    int r = 1, lim = target;                              // the fewest rounds the m-tiles leave room to split in
+    while (lim <= M) { ++r; lim += target; }
+    if (lim > s.items_split_cap) return 0;
+    const float tile_us = plan_tile_us(s);
+    float best = 0.f;
+    int lim_best = 0;
+    for (; lim <= s.items_split_cap; ++r, lim += target) {
+        const uint32_t T0 = plan_clamp_tiles(plan_ratio(W, (float)(lim - (M >> 1))) + 1.f, c_max);
+        const float e = (float)r * ((float)T0 * tile_us + PLAN_ITEM_US);
+        if (lim_best == 0 || e < best) { best = e; lim_best = lim; }
+    }
+    lim = lim_best;
+    uint32_t T = plan_clamp_tiles(plan_ratio(W, (float)(lim - M)) + 1.f, c_max);
+    int n = count(T);
+    for (int i = 0; i < 4 && n > lim; ++i) {              // (only if W was off)
+        if (T >= c_max) return 0;
+        T = plan_clamp_tiles(plan_ratio((float)T * (float)n, (float)lim) + 1.f, c_max);
+        n = count(T);
+    }
+    if (n > lim) return 0;
+    for (int i = 0; i < PLAN_PROBES; ++i) {
+        uint32_t T1 = plan_clamp_tiles(plan_ratio((float)T * (float)n, (float)lim), c_max);
+        if (T1 >= T) break;
+        int n1 = count(T1);
+        if (n1 > lim) {
+            T1 = (T + T1 + 1) >> 1;
+            if (T1 >= T) break;
+            n1 = count(T1);
+            if (n1 > lim) break;
+        }
+        T = T1; n = n1;
+    }
+    return T >= c_max ? 0u : T;
 }
 
 // What the first work item of a request leaves for the merge kernel (one entry per request at the head of the workspace).
@@ -164,39 +226,6 @@ template <int R> __device__ __forceinline__ int plan_count(const PlanLane<R> &r,
     for (int j = 0; j < R; ++j) n += r.m[j] ? r.m[j] * plan_splits_fast(r.c[j], d, s) : 0;
     return plan_wave_sum(n);
 }
-// Estimated time of the launch in microseconds when the batch is cut into N work items per kv head of at most L
-// tiles, W tiles in all per kv head: one round if the items fit the chip's compute units, else the work spread over
-// them plus half an item for the ragged end; a workgroup's fixed cost per item.
-// (Measured on an MI355X with 16-bit operands at head size 128: 1.34 / 1.98 us per tile for workgroups of 4 / 8
-// units, some 6 us of launch, prologue, first-tile latency and epilogue per workgroup.)
-constexpr float PLAN_ITEM_US = 6.f;
-__device__ __forceinline__ float plan_tile_us(const BatchShape &s) { return s.nc == 8 ? 1.98f : 1.34f; }
-__device__ __forceinline__ float plan_estimate_us(float W, int N, uint32_t L, const BatchShape &s) {
-    const float tile_us = plan_tile_us(s);
-    if (N <= s.items_target) return (float)L * tile_us + PLAN_ITEM_US;
-    return (W * tile_us + (float)N * PLAN_ITEM_US) / (float)s.items_target + 0.5f * (float)L * tile_us;
-}
-// T for the whole batch (wave-uniform; 0: no request is split): ceil(c_max / k) for the number k of splits of the
-// longest request with the lower estimate of
-//   the largest k whose items fit one round of the chip's compute units, and
-//   the largest k whose items fit the room the grid has beyond a round, if it has any (it has when the m-tiles alone
-//   come near a round, so that one round would leave the long requests whole)
-// -- both by bisection: the count grows with k.
-template <int R>
-__device__ __forceinline__ int plan_largest_k(const PlanLane<R> &r, const BatchShape &s, uint32_t c_max, int M, int limit, int guess, int *count) {
-    int lo = 1, hi = PLAN_MAX_SPLITS + 1, n_lo = M;                // fits(lo), !fits(hi)
-    int k = guess, fits_in_a_row = 0;
-#pragma nounroll
-    while (hi - lo > 1) {
-        if (k <= lo || k >= hi) k = (lo + hi) >> 1;
-        const int n = plan_count(r, s, (c_max + (uint32_t)k - 1) / (uint32_t)k);
-        // (after the first guess its neighbour above: equal requests are done in two probes)
-        if (n <= limit) { lo = k; n_lo = n; k = ++fits_in_a_row < 2 ? k + 1 : (lo + hi) >> 1; }
-        else { hi = k; k = (lo + hi) >> 1; fits_in_a_row = 2; }
-    }
-    *count = n_lo;
-    return lo;
-}
 template <int R> __device__ __forceinline__ uint32_t plan_target(const PlanLane<R> &r, const BatchShape &s) {
     if (s.forced_splits > 0) return 0;
     int cm = 0, ws = 0, ms = 0;
@@ -207,30 +236,9 @@ template <int R> __device__ __forceinline__ uint32_t plan_target(const PlanLane<
         ms += r.m[j];
     }
     const uint32_t c_max = (uint32_t)plan_wave_max(cm);
-    if (c_max < 4) return 0;
     const float W = 16.f * (float)(uint32_t)plan_wave_sum(ws);
     const int M = plan_wave_sum(ms);
-    if (M > s.items_target) return 0;                              // more m-tiles than a round: nothing is split
-    auto T_of = [&](int k) { return (c_max + (uint32_t)k - 1) / (uint32_t)k; };
-    int n1 = M;
-    const int k1 = plan_largest_k(r, s, c_max, M, s.items_target, s.items_target / (M > 0 ? M : 1), &n1);
-    int k_best = k1;
-    if (s.items_split_cap > s.items_target && k1 < PLAN_MAX_SPLITS) {
-        // beyond a round the estimate is a + b k + c / k in k: least at k = sqrt(c / b), if the grid has room for that
-        float best = plan_estimate_us(W, n1, k1 == 1 ? c_max : T_of(k1), s);
-        const float b = PLAN_ITEM_US * (W / (float)c_max) / (float)s.items_target, c = 0.5f * (float)c_max * plan_tile_us(s);
-        int km = (int)(__builtin_sqrtf(c / (b > 1e-6f ? b : 1e-6f)) + 0.5f);
-        km = km > PLAN_MAX_SPLITS ? PLAN_MAX_SPLITS : km;
-        if (km > k1) {
-            int nm = plan_count(r, s, T_of(km));
-            if (nm > s.items_split_cap) km = plan_largest_k(r, s, c_max, M, s.items_split_cap, (k1 + km) >> 1, &nm);
-            if (km > k1) {
-                const float em = plan_estimate_us(W, nm, T_of(km), s);
-                if (em < best) { best = em; k_best = km; }
-            }
-        }
-    }
-    return k_best == 1 ? 0u : T_of(k_best);
+    return plan_choose_tiles(W, M, c_max, s, [&](uint32_t T) { return plan_count(r, s, T); });
 }
 
 struct PlanItem { int b, mt, split, nsplit, item_base; };      // b < 0: the item is beyond the batch's work

@@ -1,6 +1,7 @@
 // Host side of the matrix-core prefill path: which workgroup shape and how many key-axis splits a call gets, the
 // merge of the split partials, and the launch.  The kernel itself is in prefill_mfma_kernel.hpp.
 #include "prefill_mfma_kernel.hpp"
+#include <cmath>
 
 namespace lazyattn {
 
@@ -261,6 +262,11 @@ static int mfma_splits(const lazyattn_prefill_params &p, int nw) {
             if (sk > s && fill(sk) > best * 1.2) { s = sk; best = fill(sk); }
         }
     }
+    // A split more costs about half a microsecond (its partial rows written, read and merged) and saves
+    // tiles / s^2 tile times: past s = sqrt(2 tiles tile_us) the launch gets longer even with compute units to spare
+    // (32 new tokens over 5.4 K keys, 8 workgroups per split: 16 / 32 splits take 21.0 / 24.0 us).
+    const double s_most = std::sqrt(2.0 * (double)ctx_tiles * (nw == 8 ? 1.98 : 1.34));
+    if ((double)s > s_most) s = (int64_t)(s_most + 0.5);
     if (s > ctx_tiles / 2) s = ctx_tiles / 2;        // at least two tiles per split
     if (s > 64) s = 64;
     return s < 1 ? 1 : (int)s;

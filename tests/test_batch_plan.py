@@ -1,6 +1,7 @@
 """The arithmetic that cuts a ragged batch into work items on the device (csrc/batch_plan.hpp), compiled for the
 host: no split is shorter than two tiles, no request is cut into more than 64, more splits of the longest request
-never mean fewer work items, and the small-number division is exact.  No GPU needed."""
+never mean fewer work items, the small-number division is exact, and the tiles per work item chosen for a batch
+never make more work items than the grid has room for -- also when the totals it starts from are off.  No GPU needed."""
 import os
 import subprocess
 
@@ -26,8 +27,7 @@ int main() {
             if (n < (1u << 24) && plan_udiv(n, d) != n / d) { printf("udiv edge %u %u\n", n, d); return 1; }
     // random batches, every candidate the planning kernel looks at (the longest request cut into k = 1 .. 64):
     // every request with work gets between 1 and 64 splits of at least two tiles, none longer than the candidate's
-    // item length unless one of those bounds holds it back; k = 1 splits nothing; more splits never mean fewer items;
-    // the estimate is finite and positive
+    // item length unless one of those bounds holds it back; k = 1 splits nothing; more splits never mean fewer items
     for (int trial = 0; trial < 3000; ++trial) {
         BatchShape s{};
         s.group = 1 << (rng() % 4);
@@ -66,6 +66,32 @@ int main() {
             if (k == 1 && items != M) { printf("k = 1 splits something\n"); return 1; }
             if (items < prev) { printf("fewer items for more splits\n"); return 1; }
             prev = items;
+        }
+        // the choice of T: whatever it is, the items it makes fit the rounds the grid has room for; every candidate
+        // it was offered is counted with the real counts; totals off by a quarter either way change nothing in that
+        s.items_target = 1 + rng() % 40;
+        s.items_split_cap = s.items_target * (1 + rng() % 3) + rng() % 3;
+        s.items_cap = s.items_split_cap > (int)M ? s.items_split_cap : (int)M;
+        for (float off : {1.0f, 0.75f, 1.25f}) {
+            int probes = 0;
+            auto count = [&](uint32_t T) {
+                ++probes;
+                int n = 0;
+                for (int j = 0; j < batch; ++j) n += m[j] ? m[j] * plan_splits(c[j], T, s) : 0;
+                return n;
+            };
+            const uint32_t T = plan_choose_tiles((float)W * off, (int)M, c_max, s, count);
+            if (probes > 5 + 2 * PLAN_PROBES) { printf("%d probes\n", probes); return 1; }
+            const int n = count(T);
+            if (T == 0 ? n != (int)M : (n > s.items_split_cap || T < 2 || T >= c_max)) {
+                printf("T %u makes %d items (m-tiles %u, room %d, c_max %u)\n", T, n, M, s.items_split_cap, c_max);
+                return 1;
+            }
+            // a batch that fits half a round and has a request worth cutting is cut
+            if (off == 1.0f && T == 0 && (int)M * 2 <= s.items_target && c_max >= 64 && s.items_target >= 8) {
+                printf("nothing split: m-tiles %u of %d, c_max %u\n", M, s.items_target, c_max);
+                return 1;
+            }
         }
         s.forced_splits = 1 + rng() % 70;
         for (int j = 0; j < batch; ++j)
