@@ -65,8 +65,12 @@ LAZYATTN_HD uint32_t plan_cost(int32_t q_len, int32_t ctx_len) {
 // n / d for n, d below 2^24, d > 0, through one float reciprocal and an integer correction (exact)
 LAZYATTN_HD uint32_t plan_udiv(uint32_t n, uint32_t d) {
     uint32_t q = (uint32_t)((float)n * (1.0f / (float)d));
-    while (q * d > n) --q;
-    while ((q + 1) * d <= n) ++q;
+    // (the float product is off by less than two for such operands: two corrections each way, and no loop that
+    // operands out of range could keep going)
+    q -= q * d > n;
+    q -= q * d > n;
+    q += (q + 1) * d <= n;
+    q += (q + 1) * d <= n;
     return q;
 }
 // splits of a request of `cost` tiles when a work item is to have at most T tiles (T = 0: no request is split)
@@ -169,14 +173,14 @@ __device__ __forceinline__ int plan_wave_sum(int v) { return __builtin_amdgcn_re
 __device__ __forceinline__ int plan_wave_max(int v) { LAZYATTN_PLAN_SCAN(plan_max) return __builtin_amdgcn_readlane(v, 63); }
 #undef LAZYATTN_PLAN_SCAN
 
-// The balanced list is for batches of up to 256 requests (four per lane of the scanning wave; larger batches have
-// requests enough to fill the chip and take the plain grid).
+// T is chosen on the device for batches of up to 256 requests (four per lane of the scanning wave); larger batches
+// are scanned 256 requests at a time for the split count the host fixed.
 constexpr int PLAN_MAX_BATCH = 256;
 // The requests R lane .. R lane + R - 1 (R = 1 for batches of up to 64 requests, else 4): their m-tile counts and
 // costs (0 beyond the batch).  2 R + 1 loads per lane, requested together.
 template <int R> struct PlanLane { int m[R]; uint32_t c[R]; };
-template <int R> __device__ __forceinline__ PlanLane<R> plan_load(const PlanTables &t, const BatchShape &s, int lane) {
-    const int r0 = lane * R;
+template <int R> __device__ __forceinline__ PlanLane<R> plan_load(const PlanTables &t, const BatchShape &s, int lane, int first = 0) {
+    const int r0 = first + lane * R;
     int32_t off[R + 1], seq[R];
 #pragma unroll
     for (int j = 0; j < R + 1; ++j) {
@@ -242,8 +246,11 @@ template <int R> __device__ __forceinline__ uint32_t plan_target(const PlanLane<
 }
 
 struct PlanItem { int b, mt, split, nsplit, item_base; };      // b < 0: the item is beyond the batch's work
-// which (request, m-tile, split) work item `item` of a kv head is (wave-uniform result)
-template <int R> __device__ __forceinline__ PlanItem plan_locate(const PlanLane<R> &r, const BatchShape &s, uint32_t T, int item, int lane) {
+// which (request, m-tile, split) work item `item` of a kv head is (wave-uniform result); the lanes hold the requests
+// first .. first + 64 R - 1, whose work items start at item_base; *total: the work items of these requests
+template <int R>
+__device__ __forceinline__ PlanItem plan_locate(const PlanLane<R> &r, const BatchShape &s, uint32_t T, int item, int lane,
+                                                int first = 0, int item_base = 0, int *total = nullptr) {
     PlanItem out{-1, 0, 0, 1, 0};
     const PlanDivisor d = plan_divisor(T);
     int ns[R], cn[R], tot = 0;
@@ -254,10 +261,13 @@ template <int R> __device__ __forceinline__ PlanItem plan_locate(const PlanLane<
         tot += cn[j];
     }
     const int incl = plan_wave_scan(tot);
-    const uint64_t hit = __builtin_amdgcn_ballot_w64(incl > item);
+    if (total) *total = __builtin_amdgcn_readlane(incl, 63);
+    // (an item before these requests' first is not theirs: without this test the first lane would claim it with a
+    // negative remainder -- and the division below does not end for such operands)
+    const uint64_t hit = item >= item_base ? __builtin_amdgcn_ballot_w64(item_base + incl > item) : 0ull;
     if (!hit) return out;
     const int idx = __builtin_ctzll(hit);
-    int first_item = __builtin_amdgcn_readlane(incl - tot, idx);
+    int first_item = item_base + __builtin_amdgcn_readlane(incl - tot, idx);
     int rem = item - first_item;
     int j = 0, nsel = __builtin_amdgcn_readlane(ns[0], idx);
 #pragma unroll
@@ -265,11 +275,26 @@ template <int R> __device__ __forceinline__ PlanItem plan_locate(const PlanLane<
         const int ck = __builtin_amdgcn_readlane(cn[k], idx), nk = __builtin_amdgcn_readlane(ns[k + 1], idx);
         if (j == k && rem >= ck) { rem -= ck; first_item += ck; j = k + 1; nsel = nk; }
     }
-    out.b = idx * R + j;
+    out.b = first + idx * R + j;
     out.nsplit = nsel;
     out.item_base = first_item;
     out.mt = (int)plan_udiv((uint32_t)rem, (uint32_t)nsel);
     out.split = rem - out.mt * nsel;
+    return out;
+}
+// The same for a batch of any size, 256 requests at a time, for the split count the host fixed (T is not chosen on
+// the device for such batches).
+__device__ __forceinline__ PlanItem plan_locate_chunks(const PlanTables &t, const BatchShape &s, int item, int lane) {
+    PlanItem out{-1, 0, 0, 1, 0};
+    int base = 0;
+#pragma nounroll
+    for (int first = 0; first < t.batch; first += PLAN_MAX_BATCH) {
+        const PlanLane<4> reqs = plan_load<4>(t, s, lane, first);
+        int total = 0;
+        out = plan_locate(reqs, s, 0, item, lane, first, base, &total);
+        if (out.b >= 0) break;
+        base += total;
+    }
     return out;
 }
 #endif  // __HIPCC__

@@ -315,14 +315,18 @@ static MfmaLaunch mfma_launch_shape(const lazyattn_prefill_params &p) {
     L.nw = mfma_waves(p);
     L.n_mt = mfma_mtiles(p, L.nw);
     const int group = p.num_q_heads / p.num_kv_heads;
-    const int forced = p.num_splits > 0 ? (p.num_splits > PLAN_MAX_SPLITS ? PLAN_MAX_SPLITS : p.num_splits) : 0;
-    const bool balanced = p.batch > 1 && p.batch <= PLAN_MAX_BATCH && (forced == 0 || mfma_compact(p, L.nw));
+    int forced = p.num_splits > 0 ? (p.num_splits > PLAN_MAX_SPLITS ? PLAN_MAX_SPLITS : p.num_splits) : 0;
+    // The list of work items replaces the plain grid when the device chooses the splits (up to 256 requests, no count
+    // from the caller), else when it at least halves the grid (requests with one new token beside long ones).
+    const bool device_splits = p.batch <= PLAN_MAX_BATCH && forced == 0;
+    const bool balanced = p.batch > 1 && (device_splits || mfma_compact(p, L.nw));
     auto plain = [&] {
         L.nsplit = mfma_splits(p, L.nw);
         L.items_per_kv = L.nsplit > 1 ? (int64_t)p.batch * L.n_mt * L.nsplit : 0;
         return L;
     };
     if (!balanced) return plain();
+    if (!device_splits && forced == 0) forced = mfma_splits(p, L.nw);   // one count for every request, from the host's estimate
     L.nsplit = 1;
     const int64_t m_bound = [&] {                                    // at least the m-tiles the batch really has
         const int64_t by_chunks = mfma_mtiles_bound(p, L.nw), by_requests = (int64_t)p.batch * L.n_mt;

@@ -277,9 +277,11 @@ prefill_mfma_kernel(const lazyattn_prefill_params p, const int nsplit, const int
             if (p.batch <= 64) {                                 // one request per lane: a quarter of the arithmetic
                 const PlanLane<1> reqs = plan_load<1>(tabs, bal, lane);
                 it = plan_locate(reqs, bal, plan_target(reqs, bal), witem, lane);
-            } else {
+            } else if (p.batch <= PLAN_MAX_BATCH) {
                 const PlanLane<4> reqs = plan_load<4>(tabs, bal, lane);
                 it = plan_locate(reqs, bal, plan_target(reqs, bal), witem, lane);
+            } else {
+                it = plan_locate_chunks(tabs, bal, witem, lane);
             }
             if (lane == 0) {
                 found[0] = it.b; found[1] = it.mt; found[2] = it.split; found[3] = it.nsplit;

@@ -182,14 +182,14 @@ def test_mfma_pages_of_32_slots(variant, dtype, kv, d):
 
 
 @pytest.mark.parametrize("n_short,q_short,skip", [(63, 1, True), (63, 1, False), (150, 1, True), (7, 1, True),
-                                                  (299, 3, True), (270, 2, False)])
+                                                  (299, 3, True), (270, 2, False), (600, 1, True)])
 @pytest.mark.parametrize("kernel", [_ffi.KERNEL_MFMA4, _ffi.KERNEL_MFMA8, _ffi.KERNEL_AUTO])
 def test_mfma_one_long_request_among_short_requests(n_short, q_short, skip, kernel):
     """A serving batch: a prefill chunk and many requests with one new token.  The plain (request, m-tile) grid
-    would be almost empty; the kernel takes its compact work list (m-tiles resolved from the token offsets, 256
-    requests scanned per round) and the split count follows the real amount of work.  With hundreds of
-    two- or three-token requests the host's estimate of the work is far too low; the list is sized by a bound, so
-    every m-tile still has its workgroup."""
+    would be almost empty; the kernel takes its list of work items (resolved from the token offsets on the device:
+    up to 256 requests at once with the splits chosen there, larger batches 256 requests at a time with the host's
+    split count).  With hundreds of two- or three-token requests the host's estimate of the work is far too low;
+    the list is sized by a bound, so every m-tile still has its workgroup."""
     print(f"case: mfma mixed batch, {n_short} requests of {q_short}, skip_decode={skip}, kernel {kernel}", flush=True)
     docs = [100, 16, 333, 70, 5, 250]
     requests = [[0, 2, 3, 5]] + [[b % 6] for b in range(n_short // 2)] + [[2, 1, 5, 0, 4]] + [[(b + 1) % 6, b % 6][: 1 + b % 2] for b in range(n_short - n_short // 2)]
