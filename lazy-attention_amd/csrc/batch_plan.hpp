@@ -54,6 +54,19 @@ LAZYATTN_HD int plan_mtiles(int32_t q_len, int32_t ctx_len, const BatchShape &s)
     const uint32_t m = s.nc == 8 ? (units + 7) >> 3 : (units + 3) >> 2;
     return (int)(m < cap ? m : cap);
 }
+// What the host can say of the m-tiles of a whole batch from its totals alone (the lengths are on the device): an
+// upper bound.  A request with work has at least one new token (two when one-token requests are skipped), so at most
+// R = min(batch, tokens / that) requests have any; each may end with a partly filled 32-row chunk -- the chunks
+// together are at most (tokens + 31 R) / 32 -- and, unless the workgroup's units divide the q-heads of a kv head, with
+// a partly filled m-tile; and none has more m-tiles than n_mt_cap.
+LAZYATTN_HD int64_t plan_mtiles_bound(int64_t tokens, int64_t batch, const BatchShape &s) {
+    const int64_t least = s.skip_decode ? 2 : 1;
+    const int64_t with_work = tokens / least < batch ? tokens / least : batch;
+    const int64_t chunks = (tokens + (PLAN_UNIT - 1) * with_work) / PLAN_UNIT;
+    const int64_t by_chunks = (chunks * s.group + s.nc - 1) / s.nc + (s.group % s.nc ? with_work : 0);
+    const int64_t by_requests = with_work * s.n_mt_cap;
+    return by_chunks < by_requests ? by_chunks : by_requests;
+}
 // tiles of the key axis, weighted (below 2^24 for every context a 32-bit length can describe)
 LAZYATTN_HD uint32_t plan_cost(int32_t q_len, int32_t ctx_len) {
     const uint32_t pages = ((uint32_t)ctx_len + PLAN_PAGE - 1) / PLAN_PAGE;

@@ -196,12 +196,14 @@ static int64_t mfma_mtiles_estimate(const lazyattn_prefill_params &p, int nw) {
     const int64_t per_short = (group + nw - 1) / nw;             // a one-token request, unless it is skipped
     return longs * per_req + (p.skip_decode ? 0 : (p.batch - longs) * per_short);
 }
-// Upper bound on the same number: every request may end with a partly filled 32-row chunk and a partly filled
-// m-tile.  The compact work list is sized by it.
+// Upper bound on the same number (batch_plan.hpp).
 static int64_t mfma_mtiles_bound(const lazyattn_prefill_params &p, int nw) {
-    const int group = p.num_q_heads / p.num_kv_heads;
-    const int64_t chunks = ((int64_t)p.num_tokens + UNIT - 1) / UNIT + p.batch;
-    return (chunks * group + nw - 1) / nw + p.batch;
+    BatchShape s{};
+    s.group = p.num_q_heads / p.num_kv_heads;
+    s.nc = nw;
+    s.n_mt_cap = mfma_mtiles(p, nw);
+    s.skip_decode = p.skip_decode;
+    return plan_mtiles_bound(p.num_tokens, p.batch, s);
 }
 // The compact list pays a scan of the token offsets per workgroup: taken when it at least halves the grid.
 static bool mfma_compact(const lazyattn_prefill_params &p, int nw) {
@@ -326,12 +328,15 @@ static MfmaLaunch mfma_launch_shape(const lazyattn_prefill_params &p) {
         return L;
     };
     if (!balanced) return plain();
-    if (!device_splits && forced == 0) forced = mfma_splits(p, L.nw);   // one count for every request, from the host's estimate
     L.nsplit = 1;
-    const int64_t m_bound = [&] {                                    // at least the m-tiles the batch really has
-        const int64_t by_chunks = mfma_mtiles_bound(p, L.nw), by_requests = (int64_t)p.batch * L.n_mt;
-        return by_chunks < by_requests ? by_chunks : by_requests;
-    }();
+    const int64_t m_bound = mfma_mtiles_bound(p, L.nw);             // at least the m-tiles the batch really has
+    if (!device_splits && forced == 0) {
+        // one count for every request, from the host's estimate of the work -- as far as the partial rows of that
+        // many splits of every m-tile the batch may have (the bound, not the estimate) stay within a quarter GB
+        forced = mfma_splits(p, L.nw);
+        const size_t per_item = (size_t)p.num_kv_heads * L.nw * UNIT * partial_row_bytes(p);
+        while (forced > 1 && (size_t)m_bound * (size_t)forced * per_item > ((size_t)256 << 20)) --forced;
+    }
     // One round of the chip's compute units is what the device cuts a batch for (batch_plan.hpp); a batch with more
     // m-tiles than that is not split, and the grid has room for it.
     // Room beyond one round -- up to every m-tile cut in four, and three rounds at most -- is made when one round

@@ -1,7 +1,8 @@
 """The arithmetic that cuts a ragged batch into work items on the device (csrc/batch_plan.hpp), compiled for the
 host: no split is shorter than two tiles, no request is cut into more than 64, more splits of the longest request
 never mean fewer work items, the small-number division is exact, and the tiles per work item chosen for a batch
-never make more work items than the grid has room for -- also when the totals it starts from are off.  No GPU needed."""
+never make more work items than the grid has room for -- also when the totals it starts from are off -- and the
+host's bound on a batch's m-tiles holds.  No GPU needed."""
 import os
 import subprocess
 
@@ -37,16 +38,27 @@ int main() {
         const int batch = 1 + rng() % 40;
         std::vector<int> m(batch);
         std::vector<uint32_t> c(batch);
+        std::vector<int64_t> ql_of(batch);
         uint64_t W = 0;
         uint32_t M = 0, c_max = 0;
         for (int j = 0; j < batch; ++j) {
-            const int64_t ql = (rng() % 5 == 0) ? 1 : 1 + rng() % 600;
+            const int64_t ql = (rng() % 5 == 0) ? 1 : (rng() % 4 == 0 ? 2 + rng() % 3 : 1 + rng() % 600);
             const int64_t ctx = (rng() % 7 == 0) ? 0 : rng() % (1 << (8 + rng() % 12));
+            ql_of[j] = ql;
             m[j] = plan_mtiles(ql, ctx, s);
             c[j] = m[j] ? plan_cost(ql, ctx) : 0;
             W += (uint64_t)m[j] * c[j];
             M += m[j];
             c_max = c[j] > c_max ? c[j] : c_max;
+        }
+        {   // the host's bound on the m-tiles, from the totals alone
+            int64_t tokens = 0;
+            for (int j = 0; j < batch; ++j) tokens += ql_of[j];
+            if ((int64_t)M > plan_mtiles_bound(tokens, batch, s)) {
+                printf("%u m-tiles, bound %lld (tokens %lld, batch %d, group %d, nc %d, cap %d, skip %d)\n", M,
+                       (long long)plan_mtiles_bound(tokens, batch, s), (long long)tokens, batch, s.group, s.nc, s.n_mt_cap, s.skip_decode);
+                return 1;
+            }
         }
         if (!c_max) continue;
         uint64_t prev = 0;
