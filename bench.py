@@ -27,8 +27,8 @@ PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
 # WRITE_SIZE, each scaled by what the same counter reads for a 256 MiB copy; summary under profiles/).
 # Counters cannot be read from inside this script, so the figure is the committed measurement of the
 # named workload; workloads without one report null.
-MEASURED_TRAFFIC_BYTES = {"c2_8b_bf16_10x512_q128": 43_300_000, "c3_8b_bf16_pool64x256_16req_x20_q64": 241_700_000,
-                          "c4_8b_bf16_64x1024_q256": 445_900_000, "c5_8b_fp8kv_8req_32x512_q128": 336_000_000,
+MEASURED_TRAFFIC_BYTES = {"c2_8b_bf16_10x512_q128": 43_300_000, "c3_8b_bf16_pool64x256_16req_x20_q64": 242_200_000,
+                          "c4_8b_bf16_64x1024_q256": 441_100_000, "c5_8b_fp8kv_8req_32x512_q128": 335_000_000,
                           "d1_8b_bf16_decode_32req_20x256": 679_600_000}
 PEAK_HBM_GBS = 8000.0
 
