@@ -284,3 +284,39 @@ def test_kernel_query_names_the_kernel_and_the_reason_for_the_fallback():
     assert lib.lazyattn_prefill_kernel_for(ctypes.byref(p), None, ctypes.byref(why)) == _ffi.KERNEL_GENERIC
     assert b"aligned" in why.value
     assert lib.lazyattn_prefill_kernel_for(None, None, None) == -1
+
+
+def test_launch_shape_queries_for_batches():
+    """What the host decides for a call with several requests, asked without a GPU (the CU count falls back to 256):
+    the splits of a batch are left to the device (0) unless the caller fixes them; every batch needs a workspace
+    (the device may split any request), sized for at most three rounds of the chip's compute units -- 96 work items per
+    kv head, 4 or 8 waves of 32 partial rows of 128 halves + 2 floats each -- plus one 16-byte record per request; a
+    caller's split count is sized by the bound on the batch's m-tiles; batches beyond 256 requests get one split count
+    from the host, within a quarter of a GB."""
+    lib = _ffi.lib()
+    splits, why = ctypes.c_int32(-1), ctypes.c_char_p()
+    row = 128 * 2 + 8
+
+    def ask(batch, tokens, max_q, seq, num_splits=0, skip=0):
+        p = _fake_params(tokens=tokens, seq=seq)
+        p.batch, p.max_q_len, p.num_splits, p.skip_decode = batch, max_q, num_splits, skip
+        k = lib.lazyattn_prefill_kernel_for(ctypes.byref(p), ctypes.byref(splits), ctypes.byref(why))
+        return k, splits.value, lib.lazyattn_prefill_workspace_bytes(ctypes.byref(p))
+
+    for batch, tokens, max_q in ((16, 1024, 64), (3, 384, 128), (8, 1024, 128), (6, 777, 400), (200, 328, 128)):
+        k, s, ws = ask(batch, tokens, max_q, 5248)
+        nw = 4 if k == _ffi.KERNEL_MFMA4 else 8
+        assert k in (_ffi.KERNEL_MFMA4, _ffi.KERNEL_MFMA8) and s == 0, (batch, k, s)
+        table = (batch * 16 + 255) // 256 * 256
+        assert table < ws <= table + 8 * 96 * nw * 32 * row, (batch, ws)
+        assert (ws - table) % (8 * nw * 32 * row) == 0
+        k3, s3, ws3 = ask(batch, tokens, max_q, 5248, num_splits=3)
+        assert s3 == 3 and ws3 > table
+    # one request: the host's split count, a workspace only when it is split
+    k, s, ws = ask(1, 128, 128, 5248)
+    assert s >= 2 and ws == 8 * (128 // 32 * 4 // (4 if k == _ffi.KERNEL_MFMA4 else 8)) * s * (4 if k == _ffi.KERNEL_MFMA4 else 8) * 32 * row
+    k, s, ws = ask(1, 128, 128, 5248, num_splits=1)
+    assert s == 1 and ws == 0
+    # a large serving batch: one split count for all, and a bounded workspace
+    k, s, ws = ask(600, 728, 128, 5248, skip=1)
+    assert s >= 1 and ws <= (256 << 20) + 600 * 16 + 256
