@@ -108,7 +108,8 @@ typedef struct lazyattn_prefill_params {
     int32_t fp32_rotary;        /* FORCE_FP32_ROTARY (old_ops:248-254); the MFMA kernel always
                                    rotates in fp32 and rounds once */
     int32_t kernel;             /* LAZYATTN_KERNEL_* */
-    int32_t num_splits;         /* context splits per work item; 0 = choose */
+    int32_t num_splits;         /* key-axis splits of every request; 0 = choose: for one request on the host, for a
+                                   batch of up to 256 requests per request on the device, from the lengths */
     int32_t phases;             /* LAZYATTN_PHASE_*; 0 = all */
     float sm_scale;
     int32_t num_tokens;         /* rows of `o` (>= b_start_loc[B]); sizes the split-KV workspace */
@@ -127,7 +128,10 @@ typedef struct lazyattn_prefill_params {
 } lazyattn_prefill_params;
 
 /* Bytes of workspace lazyattn_prefix_prefill() may need for these sizes (0 when the
- * chosen kernel writes `o` directly).  Pure host arithmetic.  No reference
+ * chosen kernel writes `o` directly: one request that is not split, or num_splits = 1).  A call with several
+ * requests and num_splits = 0 always needs it: which requests are split is decided on the device.  The workspace
+ * holds partial rows (and, for batches, a 16-byte record per request at its head); nothing in it has to be
+ * initialised, and a call reads only what the same call wrote.  Pure host arithmetic.  No reference
  * counterpart: Triton's launch has no split-KV. */
 size_t lazyattn_prefill_workspace_bytes(const lazyattn_prefill_params *p);
 
