@@ -1,6 +1,7 @@
 """The library's own choice of workgroup shape and key-axis splits (``_kernel`` / ``_num_splits`` left at AUTO)
-against every forced choice, timed on thirty seeded ragged batches at Llama-3-8B geometry: AUTO may be at most 15 %
-slower than the best forced choice on any shape and 4 % on average (measured: 9 % and -1 %), and its output
+against every forced choice, timed on thirty seeded ragged batches at Llama-3-8B geometry: AUTO may be at most 20 %
+slower than the best forced choice on any shape and 5 % on average (measured on three boxes: 8-9 % and -1 %; the
+bounds leave room for the few per cent two timings of one launch differ by), and its output
 must agree with the single-split plain grid's.  A timing test: collected late, generous bounds, medians."""
 import random
 import statistics
@@ -77,5 +78,5 @@ def test_auto_choice_is_close_to_the_best_forced_choice():
                     f"{forced[best]:7.1f} us, ratio {ratios[-1]:.3f}")
     table = "\n".join(rows)
     print(table)
-    assert max(ratios) <= 1.15, table
-    assert sum(ratios) / len(ratios) <= 1.04, table
+    assert max(ratios) <= 1.20, table
+    assert sum(ratios) / len(ratios) <= 1.05, table
