@@ -205,7 +205,8 @@ static int64_t mfma_mtiles_bound(const lazyattn_prefill_params &p, int nw) {
     s.skip_decode = p.skip_decode;
     return plan_mtiles_bound(p.num_tokens, p.batch, s);
 }
-// The compact list pays a scan of the token offsets per workgroup: taken when it at least halves the grid.
+// A list of work items with a fixed split count pays a scan of the lengths per workgroup where the plain grid pays
+// nothing: taken when it at least halves the grid (requests with one new token beside long ones).
 static bool mfma_compact(const lazyattn_prefill_params &p, int nw) {
     return p.batch > 1 && mfma_mtiles_bound(p, nw) * 2 <= (int64_t)p.batch * mfma_mtiles(p, nw);
 }
@@ -305,8 +306,9 @@ bool mfma_supports(const lazyattn_prefill_params &p) { return mfma_unsupported_r
 
 
 // What one call launches: the workgroup shape, and either the plain grid (request, kv head, split, m-tile) with one
-// split count for every request -- a single request, or a caller who fixes the split count for a batch without
-// one-token requests -- or the balanced list of work items (batch_plan.hpp), whose splits are decided on the device.
+// split count for every request -- a single request, or a fixed split count (the caller's, or the host's for more
+// than 256 requests) on a batch without many one-token requests -- or the list of work items (batch_plan.hpp): with
+// the splits decided per request on the device (up to 256 requests, no count from the caller) or with the fixed count.
 struct MfmaLaunch {
     int nw, n_mt, nsplit;           // nsplit: of the plain grid (1 under the balanced list)
     BatchShape bal;                 // items_cap > 0: balanced list
