@@ -16,8 +16,8 @@
 //           three probes of the real item count toward the value that fills the rounds exactly
 //   s_j     = ceil(c_j / T) key-axis splits of request j (at least two tiles each, at most 64)
 // and from the prefix sums of m_j s_j which (request, m-tile, split) its work item is.  The first work item of every
-// request leaves (first item, splits, m-tiles) of the request in a small table at the head of the workspace, where
-// the merge kernel finds them with one scalar load.
+// request leaves (first item, splits) of the request in a small table at the head of the workspace, where the merge
+// kernel finds them with one scalar load.
 // The arithmetic per request is plain C++ (also compiled for the host, where a unit test checks its invariants).
 #pragma once
 #include <stdint.h>
@@ -40,7 +40,7 @@ struct BatchShape {
     int32_t items_cap;      // work items per kv head the grid has room for (at least the m-tiles)
     int32_t items_target;   // work items per kv head that fill one round of the chip's compute units
     int32_t items_split_cap;    // most work items per kv head of a batch that is split: what the partial rows have room for
-    int32_t forced_splits;  // > 0: every request gets this many splits (the caller's num_splits)
+    int32_t forced_splits;  // > 0: every request gets this many splits (the caller's num_splits, or the host's for a large batch)
     int32_t table_bytes;    // the requests' records at the head of the workspace (a multiple of 256); the partial rows follow
 };
 
@@ -158,7 +158,7 @@ LAZYATTN_HD uint32_t plan_choose_tiles(float W, int M, uint32_t c_max, const Bat
 }
 
 // What the first work item of a request leaves for the merge kernel (one entry per request at the head of the workspace).
-struct PlanRecord { int32_t item_base, nsplit, m, pad; };
+struct PlanRecord { int32_t item_base, nsplit, m, pad; };      // (m, pad: zero; 16 bytes, one scalar load)
 
 #if defined(__HIPCC__)
 // ---------------------------------------------------------------------------------------- one wave scans the batch
